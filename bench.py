@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Throughput of the fused ConEF compress + error-feedback step on one MI355X.
+
+Workload (the configuration the headline metric is quoted on): RandomBlock compressor, 10 %
+contiguous block, with a count-sketch error compressor at 10 % memory, on one flat fp32 bucket of
+6.5 M elements viewed [5, 1_300_000] (sketch [5, 130_000]); gradients N(0, 1e-6) with 1 % heavy-tail
+entries Laplace(0, 1e-2); synthetic, seeded.
+
+A "step" is one call of the fused C-ABI entry point `conef_randblock_conef_step_f32` on one
+bucket whose gradient already sits in HBM: it adds the unsketched error, extracts the payload
+block, leaves the decompressed gradient in place and writes the new sketch.  Every timed step gets a gradient buffer
+no earlier step has touched and one of a rotating set of sketch states, so nothing it reads is left
+in the 256 MB Infinity Cache from before: the rate is an HBM rate, not a cache rate.  The
+same-buffer rate is reported next to it.
+
+Prints ONE JSON line.  `roofline` prices the step against MI355X's 8 TB/s HBM peak with the
+algorithmic byte count 8L + 8nW + 4k; `cpu_baseline` times the scalar C oracle on a bounded sample
+of the same workload on this box's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+
+N_ROWS, N_COLS = 5, 1_300_000
+SKETCH_SIZE = 0.1
+RATIO = 0.1
+BETA = 0.9
+N_BUCKETS = 12           # sketch states / payload buffers in rotation (a fresh 26 MB gradient every step)
+MAX_GRAD_BUFFERS = 2000  # 52 GB of gradients at most; beyond that the buffers are stepped on again
+
+
+def algorithmic_bytes(L, n, w, k):
+    """read g (4L) + read sketch (4nW) + write decompressed g (4L) + write sketch (4nW) + write payload (4k)"""
+    return 8 * L + 8 * n * w + 4 * k
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=600)
+    ap.add_argument("--warmup", type=int, default=60)
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget for the CPU baseline sample")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: the ConEF compress+EF step has no cross-GPU part in this build "
+              "(run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from conef_amd import _lib
+    from conef_amd.compressors.CountSketch import DenseCS
+
+    if not torch.cuda.is_available():
+        print("bench.py needs the GPU; there is no CPU path for the ConEF kernels", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    lib = _lib.load()
+    L = N_ROWS * N_COLS
+    block = max(1, int(RATIO * L))
+    alpha = 1 - BETA
+
+    # ---- resident inputs: one fresh gradient bucket per step (288 GB of HBM make that cheap), a
+    # rotating set of sketch states and payload buffers, pre-drawn block offsets
+    total_steps = args.warmup + args.steps
+    n_grads = min(total_steps, MAX_GRAD_BUFFERS)
+    gen = torch.Generator(device="cuda").manual_seed(20240607)
+
+    def device_gradient():
+        x = torch.randn(L, generator=gen, device="cuda") * 1e-3
+        mask = torch.rand(L, generator=gen, device="cuda") < 0.01
+        u = torch.rand(L, generator=gen, device="cuda") - 0.5
+        lap = -1e-2 * torch.sign(u) * torch.log1p(-2 * u.abs())
+        return torch.where(mask, lap, x).view(N_ROWS, N_COLS).contiguous()
+
+    grads = [device_gradient() for _ in range(n_grads)]
+    host_grad0 = grads[0].cpu()
+    sketches = [DenseCS(N_ROWS, N_COLS, SKETCH_SIZE) for _ in range(N_BUCKETS)]
+    payloads = [torch.empty(block, dtype=torch.float32, device="cuda") for _ in range(N_BUCKETS)]
+    W = sketches[0].range
+    rng = np.random.RandomState(42)
+    starts = [int(rng.choice(L)) for _ in range(total_steps + 64)]
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def one_step(i, g, b):
+        cs = sketches[b]
+        out = cs.next_buffer()
+        rc = lib.conef_randblock_conef_step_f32(g.data_ptr(), cs.cs.data_ptr(), out.data_ptr(),
+                                                payloads[b].data_ptr(), N_ROWS, N_COLS, W, starts[i], block,
+                                                alpha, BETA, cs.a, cs.b, stream)
+        if rc != 0:
+            raise RuntimeError("conef_randblock_conef_step_f32 returned %d" % rc)
+        cs.commit(out)
+
+    torch.cuda.synchronize()
+    for i in range(args.warmup):
+        one_step(i, grads[i % n_grads], i % N_BUCKETS)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for i in range(args.warmup, total_steps):
+        one_step(i, grads[i % n_grads], i % N_BUCKETS)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    gpu_ms = ev0.elapsed_time(ev1)
+    ms_per_step = max(wall_ms, gpu_ms) / args.steps
+    ev_ms_per_step = gpu_ms / args.steps
+
+    # same-buffer (cache-resident) rate, reported for contrast
+    same_steps = max(50, args.steps // 4)
+    for i in range(10):
+        one_step(i, grads[0], 0)
+    torch.cuda.synchronize()
+    ev0.record()
+    for i in range(same_steps):
+        one_step(i, grads[0], 0)
+    ev1.record()
+    torch.cuda.synchronize()
+    same_ms = ev0.elapsed_time(ev1) / same_steps
+
+    # practical ceiling: device-to-device copy of a > 256 MB buffer
+    big = torch.empty(128 * 1024 * 1024, dtype=torch.float32, device="cuda")
+    big2 = torch.empty_like(big)
+    for _ in range(3):
+        big2.copy_(big)
+    torch.cuda.synchronize()
+    ev0.record()
+    for _ in range(10):
+        big2.copy_(big)
+    ev1.record()
+    torch.cuda.synchronize()
+    copy_gbs = 2 * big.numel() * 4 * 10 / (ev0.elapsed_time(ev1) * 1e-3) / 1e9
+    del big, big2
+
+    grad_gb = 4 * L / 1e9
+    alg_bytes = algorithmic_bytes(L, N_ROWS, W, block)
+    achieved = alg_bytes / (ev_ms_per_step * 1e-3) / 1e9
+
+    result = {
+        "metric": "GB/s gradient per ConEF compress+EF step (% HBM roofline), 25MB bucket, 1 GPU",
+        "value": round(grad_gb / (ms_per_step * 1e-3), 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "RandomBlock 10% + count-sketch ConEF 10%, flat fp32 bucket [5,1300000] (26 MB), "
+                        "sketch [5,130000], block 650000, beta 0.9",
+            "entry_point": "conef_randblock_conef_step_f32",
+            "gradient_buffers": n_grads,
+            "sketch_states_rotated": N_BUCKETS,
+            "working_set_mb": round((n_grads * 4 * L + N_BUCKETS * (4 * block + 8 * N_ROWS * W)) / 1e6, 1),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "algorithmic_bytes_per_step": alg_bytes,
+            "ms_per_step_hip_events": round(ev_ms_per_step, 5),
+            "measured_copy_gbs": round(copy_gbs, 1),
+            "frac_of_measured_copy": round(achieved / copy_gbs, 4),
+        },
+        "same_buffer": {"ms_per_step": round(same_ms, 5), "value": round(grad_gb / (same_ms * 1e-3), 2)},
+        "host_wall_ms_per_step": round(wall_ms / args.steps, 5),
+    }
+
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(host_grad0, W, block, alpha, args.cpu_seconds)
+    print(json.dumps(result))
+
+
+def cpu_baseline(grad, W, block, alpha, budget_s):
+    """The scalar C oracle's fused step on full 6.5 M-element buckets, one host thread."""
+    import numpy as np
+    from oracle import conef_oracle as oracle
+
+    L = N_ROWS * N_COLS
+    x0 = grad.numpy().reshape(N_ROWS, N_COLS)
+    cs = np.zeros((N_ROWS, W), dtype=np.float32)
+    payload = np.empty(block, dtype=np.float32)
+    rng = np.random.RandomState(42)
+    x = x0.copy()
+    oracle.randblock_conef_step(x, cs, payload, int(rng.choice(L)), block, alpha, BETA)   # warm-up
+    times = []
+    t_begin = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_begin < budget_s and len(times) < 200):
+        x = x0.copy()
+        start = int(rng.choice(L))
+        t0 = time.perf_counter()
+        oracle.randblock_conef_step(x, cs, payload, start, block, alpha, BETA)
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {
+        "value": round(4 * L / 1e9 / med, 4),
+        "unit": "GB/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": "%d full steps of the same [5,1300000] workload, scalar C oracle, median of %d (%.1f ms/step); "
+                  "host has %d logical CPUs" % (len(times), len(times), med * 1e3, os.cpu_count()),
+    }
+
+
+if __name__ == "__main__":
+    main()

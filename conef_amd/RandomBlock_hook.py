@@ -1,0 +1,193 @@
+"""Random contiguous-block compressor with (contractive) error feedback as a DDP communication hook.
+
+Drop-in for the reference's communication/RandomBlock_hook.py: same ``RandomBlockState`` constructor
+arguments, defaults, fields and error messages (:60-115), same ``RandomBlock_hook(state, bucket)``
+contract (:138-295).  What differs is how a step executes: for each >=2-D gradient the reference
+issues a query kernel, a clone, slice copies, memsets, an update kernel, a zero_ and copies back;
+here one fused gfx950 kernel reads the gradient once and leaves payload, decompressed gradient and
+new error state behind (``conef_randblock_conef_step_f32`` / ``conef_randblock_ef_step_f32``).
+"""
+import logging
+
+import numpy as np
+import torch
+import torch.distributed as dist
+
+from . import _bucket, _lib
+from .compressors.CountSketch import DenseCS
+
+
+class RandomBlockState(object):
+    """Hyper-parameters and per-bucket state (reference: RandomBlock_hook.py:16-135).
+
+    ``compression_ratio`` is the fraction of entries of every >=2-D gradient that is kept;
+    ``start_compression_iter`` (must exceed 1 because DDP rebuilds its buckets after the first
+    iteration) is the number of leading iterations that use a plain all-reduce;
+    ``use_error_compression`` stores the residual in a count sketch of ``sketch_size * columns``
+    buckets per row with decay ``beta`` instead of a dense tensor.
+    """
+
+    __slots__ = [
+        "process_group",
+        "compression_ratio",
+        "start_compression_iter",
+        "n_blocks",
+        "use_error_compression",
+        "beta",
+        "sketch_size",
+        "use_error_feedback",
+        "rng",
+        "error_dict",
+        "iter",
+        "compression_stats_logging_frequency",
+        "next_stats_report",
+        "compressed_tensor_memory",
+    ]
+
+    def __init__(
+        self,
+        process_group,
+        compression_ratio=0.1,
+        start_compression_iter=1_000,
+        use_error_compression=False,
+        beta=0.9,
+        sketch_size=0.5,
+        use_error_feedback=True,
+        random_seed=42,
+        compression_stats_logging_frequency=10_000,
+    ):
+        if start_compression_iter <= 1:
+            raise ValueError(
+                "Expect `start_compression_iter` > 1 if `use_error_feedback`, "
+                "because gradient compression can only be applied after the first two iterations in DDP."
+            )
+        if (not use_error_feedback) and use_error_compression:
+            raise ValueError(
+                "Expect `use_error_feedback` = True if `use_error_compression`, "
+                "otherwise there is no need to use error compression."
+            )
+        self.process_group = process_group
+        self.compression_ratio = compression_ratio
+        self.start_compression_iter = start_compression_iter
+        self.use_error_feedback = use_error_feedback
+        self.use_error_compression = use_error_compression
+        self.beta = beta
+        self.sketch_size = sketch_size
+        self.rng = np.random.RandomState(random_seed)
+        self.error_dict = {}
+        self.iter = 0
+        self.compression_stats_logging_frequency = max(1, compression_stats_logging_frequency)
+        self.next_stats_report = 0
+        self.compressed_tensor_memory = {}
+
+    def maybe_increase_iter(self, bucket):
+        # the last bucket to be reduced closes an iteration
+        if _bucket.is_last(bucket):
+            self.iter += 1
+        if self.iter == self.start_compression_iter:
+            logging.info("Start to apply PowerSGD after {} iterations.".format(self.iter))
+
+    def clean_error(self):
+        """Zeroes the sketches (reference :129-135; only meaningful with error compression)."""
+        if self.use_error_feedback and self.use_error_compression:
+            for errors in self.error_dict.values():
+                for cs in errors or ():
+                    cs.clean(0)
+
+
+def _block_size(state, numel):
+    return max(1, int(state.compression_ratio * numel))      # RandomBlock_hook.py:207,216
+
+
+def RandomBlock_hook(state: RandomBlockState, bucket) -> torch.futures.Future:
+    group, world_size = _bucket.group_and_size(state.process_group)
+    input_tensor = _bucket.buffer(bucket)
+
+    if state.iter < state.start_compression_iter:
+        state.maybe_increase_iter(bucket)
+        return _bucket.allreduce_fut(group, input_tensor, world_size)
+
+    _lib.require_device_f32(input_tensor, "bucket buffer")
+    lib = _lib.load()
+    stream = _lib.stream_ptr(input_tensor)
+    device = input_tensor.device
+    bucket_index = _bucket.index(bucket)
+
+    if not state.use_error_feedback:
+        # the reference indexes error_dict[bucket_index] unconditionally (:215) although it only
+        # creates the entry under use_error_feedback (:158-160); same failure, same exception type
+        raise KeyError(bucket_index)
+    errors = state.error_dict.setdefault(bucket_index, [])
+
+    matrices, uncompressed = [], []
+    for tensor in _bucket.gradients(bucket):
+        if tensor.ndimension() > 1:
+            matrices.append(tensor.view(tensor.shape[0], -1))
+        else:
+            uncompressed.append(tensor)
+
+    for cnt, matrix in enumerate(matrices):
+        if len(errors) <= cnt:
+            if state.use_error_compression:
+                errors.append(DenseCS(matrix.shape[0], matrix.shape[1], state.sketch_size, device=device))
+            else:
+                errors.append(torch.zeros_like(matrix))
+
+    if bucket_index not in state.compressed_tensor_memory:
+        total = sum(_block_size(state, m.numel()) for m in matrices)
+        state.compressed_tensor_memory[bucket_index] = torch.empty(total, dtype=torch.float32, device=device)
+    payload_all = state.compressed_tensor_memory[bucket_index]
+
+    alpha = 1 - state.beta          # python double, rounded to fp32 at the boundary (reference :190)
+    spans, idx = [], 0
+    for matrix, error in zip(matrices, errors):
+        numel = matrix.numel()
+        block = _block_size(state, numel)
+        start = int(state.rng.choice(numel))                   # one draw per tensor, in bucket order (:218)
+        payload = payload_all[idx: idx + block]
+        n, m = matrix.shape
+        if state.use_error_compression:
+            out = error.next_buffer()
+            rc = lib.conef_randblock_conef_step_f32(
+                matrix.data_ptr(), error.cs.data_ptr(), out.data_ptr(), payload.data_ptr(), n, m, error.range,
+                start, block, float(alpha), float(state.beta), error.a, error.b, stream)
+            _lib.check(rc, "conef_randblock_conef_step_f32")
+            error.commit(out)
+        else:
+            rc = lib.conef_randblock_ef_step_f32(matrix.data_ptr(), error.data_ptr(), payload.data_ptr(), numel,
+                                                 start, block, stream)
+            _lib.check(rc, "conef_randblock_ef_step_f32")
+        spans.append((matrix, start, block, idx))
+        idx += block
+
+    if world_size == 1:
+        # every all-reduce is the identity: the fused kernels already left zeros + block in place
+        state.maybe_increase_iter(bucket)
+        return _bucket.completed_future(input_tensor)
+
+    # More than one rank (not exercised on the single-GPU boxes this was developed on): average the
+    # small tensors and the payload, then put the averaged block back.
+    flat_small = (torch.cat([t.view(-1) for t in uncompressed]) if uncompressed
+                  else torch.tensor([], device=device, dtype=input_tensor.dtype))
+    fut = dist.all_reduce(flat_small, group=group, async_op=True).get_future()
+
+    def unpack_small_and_reduce_payload(f):
+        small = f.value()[0].div_(world_size)
+        off = 0
+        for t in uncompressed:
+            t.copy_(small[off: off + t.numel()].view_as(t))
+            off += t.numel()
+        return dist.all_reduce(payload_all, group=group, async_op=True).get_future().wait()[0]
+
+    def decompress(f):
+        reduced = f.value().div_(world_size)
+        state.compressed_tensor_memory[bucket_index] = reduced
+        s = _lib.stream_ptr(input_tensor)
+        for matrix, start, block, off in spans:
+            rc = lib.conef_randblock_scatter_f32(matrix.data_ptr(), reduced[off: off + block].data_ptr(),
+                                                 matrix.numel(), start, block, s)
+            _lib.check(rc, "conef_randblock_scatter_f32")
+        state.maybe_increase_iter(bucket)
+        return input_tensor
+
+    return fut.then(unpack_small_and_reduce_payload).then(decompress)

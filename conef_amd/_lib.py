@@ -1,0 +1,101 @@
+"""ctypes binding of libconef_hip.so - the one native boundary of the package.
+
+This replaces what communication/compressors/cupy_kernel.py:10-45 does in the reference
+(NVRTC-compile a CUDA string and launch it with raw pointers on torch's current stream): here the
+kernels are precompiled for gfx950 and every entry point takes raw device pointers, sizes,
+scalars by value and the stream.  There is no CPU implementation behind these calls: if the
+library is missing the import of any op fails loudly.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIBPATH = os.path.join(_HERE, "lib", "libconef_hip.so")
+
+_P = ctypes.c_void_p
+_I64 = ctypes.c_int64
+_I32 = ctypes.c_int32
+_F32 = ctypes.c_float
+
+# name -> argtypes; every function returns int (0 = ok, >0 hipError_t, -1 invalid argument),
+# except conef_topk_workspace_bytes which returns a byte count as int64
+SIGNATURES = {
+    "conef_version": [],
+    "conef_hash_table_i32": [_P, _P, _I64, _I32, _I32, _I32, _I32, _I32, _P],
+    "conef_hash_table_host_i32": [_P, _P, _I64, _I32, _I32, _I32, _I32, _I32],
+    "conef_cs_query_f32": [_P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],
+    "conef_cs_query_f16": [_P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],
+    "conef_cs_update_inplace_ok": [_I64, _I64, _I32],
+    "conef_cs_update_f32": [_P, _P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],
+    "conef_cs_update_f16": [_P, _P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],
+    "conef_cs3_query_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _F32, _P],
+    "conef_cs3_update_f32": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I32, _F32, _P],
+    "conef_scale_f32": [_P, _I64, _F32, _P],
+    "conef_scale_f16": [_P, _I64, _F32, _P],
+    "conef_convert_f16_to_f32": [_P, _P, _I64, _P],
+    "conef_convert_f32_to_f16": [_P, _P, _I64, _P],
+    "conef_randblock_conef_step_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _I64, _I64, _F32, _F32, _I32, _I32, _P],
+    "conef_randblock_ef_step_f32": [_P, _P, _P, _I64, _I64, _I64, _P],
+    "conef_randblock_unbiased_step_f32": [_P, _P, _I64, _I64, _I64, _F32, _P],
+    "conef_randblock_gather_f32": [_P, _P, _I64, _I64, _I64, _F32, _P],
+    "conef_randblock_scatter_f32": [_P, _P, _I64, _I64, _I64, _P],
+    "conef_psgd_mq_f32": [_P, _P, _P, _I64, _I64, _I32, _P],
+    "conef_psgd_mq_ef_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _P],
+    "conef_psgd_mq_conef_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P],
+    "conef_psgd_mtp_f32": [_P, _P, _P, _I64, _I64, _I32, _P],
+    "conef_psgd_pqt_f32": [_P, _P, _P, _I64, _I64, _I32, _P],
+    "conef_psgd_pqt_ef_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _P],
+    "conef_psgd_pqt_conef_f32": [_P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P],
+    "conef_gram_schmidt_f32": [_P, _I64, _I32, _F32, _P],
+    "conef_ef_passthrough_f32": [_P, _P, _I64, _P],
+    "conef_topk_workspace_bytes": [_I64],
+    "conef_topk_sparsify_f32": [_P, _I64, _I64, _P, _I64, _P],
+}
+
+_handle = None
+
+
+class ConefLibraryError(RuntimeError):
+    pass
+
+
+def load():
+    """Loads the shared library (once) and types every entry point.  Raises if it is not built."""
+    global _handle
+    if _handle is not None:
+        return _handle
+    if not os.path.exists(LIBPATH):
+        raise ConefLibraryError(
+            "libconef_hip.so is not built (expected at %s); run `python -m conef_amd.build`. "
+            "There is no CPU fallback for the ConEF kernels." % LIBPATH)
+    lib = ctypes.CDLL(LIBPATH)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)      # AttributeError here means header and library disagree
+        fn.argtypes = argtypes
+        fn.restype = _I64 if name == "conef_topk_workspace_bytes" else ctypes.c_int
+    _handle = lib
+    return lib
+
+
+def check(code, what):
+    if code != 0:
+        if code == -1:
+            raise ValueError("%s: invalid argument" % what)
+        raise ConefLibraryError("%s: HIP error %d" % (what, code))
+
+
+def stream_ptr(tensor):
+    """hipStream_t of torch's current stream on the tensor's device, as an integer."""
+    return torch.cuda.current_stream(tensor.device).cuda_stream
+
+
+def require_device_f32(t, name, dtype=torch.float32):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise ValueError("%s must be a tensor on the GPU; the ConEF kernels have no CPU path" % name)
+    if t.dtype != dtype:
+        raise ValueError("%s must be %s, got %s" % (name, dtype, t.dtype))
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % name)
+    return t

@@ -1,0 +1,101 @@
+"""Single-hash count sketch held in fp32 (reference: communication/compressors/CountSketch.py:102-182).
+
+Same constructor, attributes (N, D, blk_size, range, cs, a, b) and methods as the reference class.
+Differences a maintainer should know about:
+  * the kernels are precompiled gfx950 code reached through libconef_hip.so, not CuPy/NVRTC;
+  * alpha, beta, a, b travel by value, so ``a``/``b`` are Python ints, not 1-element device tensors;
+  * when a sketch row does not fit LDS (W above a few thousand) ``update`` writes into a second
+    buffer and ``self.cs`` is rebound to it, so do not keep a stale reference to ``cs`` across updates;
+  * ``state_dict``/``load_state_dict`` round-trip (the reference's __setstate__ loses a, b).
+"""
+import torch
+
+from .. import _lib
+
+HASH_A = 994443   # CountSketch.py:112
+HASH_B = 609478   # CountSketch.py:113
+
+
+class DenseCS:
+    def __init__(self, N, D, sketch_size, device=None):
+        self.N = int(N)
+        self.D = int(D)
+        self.blk_size = 256
+        self.range = max(int(D * sketch_size), 1)          # CountSketch.py:107
+        if device is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        self.cs = torch.zeros(self.N, self.range, dtype=torch.float32, device=device)
+        self.a = HASH_A
+        self.b = HASH_B
+        self._lib = _lib.load()
+        self._inplace = bool(self._lib.conef_cs_update_inplace_ok(self.N, self.D, self.range))
+        self._spare = None
+
+    # -- persistence ---------------------------------------------------------------------------
+    def state_dict(self):
+        return {"N": self.N, "D": self.D, "blk_size": self.blk_size, "range": self.range,
+                "cs": self.cs.detach().cpu().numpy(), "a": self.a, "b": self.b}
+
+    def load_state_dict(self, d):
+        if (d["N"], d["D"], d["range"]) != (self.N, self.D, self.range):
+            raise ValueError("sketch shape mismatch: have (%d,%d,%d), state holds (%d,%d,%d)" % (
+                self.N, self.D, self.range, d["N"], d["D"], d["range"]))
+        self.cs.copy_(torch.from_numpy(d["cs"]).to(self.cs.device))
+        self.a = int(d.get("a", HASH_A))
+        self.b = int(d.get("b", HASH_B))
+
+    __getstate__ = state_dict
+
+    def __setstate__(self, d):
+        device = torch.device("cuda", torch.cuda.current_device())
+        self.N, self.D, self.blk_size, self.range = d["N"], d["D"], d["blk_size"], d["range"]
+        self.cs = torch.from_numpy(d["cs"]).to(device)
+        self.a, self.b = int(d.get("a", HASH_A)), int(d.get("b", HASH_B))
+        self._lib = _lib.load()
+        self._inplace = bool(self._lib.conef_cs_update_inplace_ok(self.N, self.D, self.range))
+        self._spare = None
+
+    # -- kernels -------------------------------------------------------------------------------
+    def _check(self, t, name):
+        _lib.require_device_f32(t, name)
+        if t.numel() != self.N * self.D:
+            raise ValueError("%s has %d elements, the sketch was built for %d x %d" % (
+                name, t.numel(), self.N, self.D))
+        if t.device != self.cs.device:
+            raise ValueError("%s is on %s, the sketch on %s" % (name, t.device, self.cs.device))
+
+    def next_buffer(self):
+        """Buffer the next update writes into: ``cs`` itself when a row fits LDS, else a spare."""
+        if self._inplace:
+            return self.cs
+        if self._spare is None:
+            self._spare = torch.empty_like(self.cs)
+        return self._spare
+
+    def commit(self, written):
+        """Makes the buffer an update wrote into the current sketch."""
+        if written is not self.cs:
+            self._spare, self.cs = self.cs, written
+
+    def update(self, vec, beta):
+        """cs <- cs + sketch-accumulate(vec) with the reference's per-element decay (CountSketch.py:27-67)."""
+        self._check(vec, "vec")
+        out = self.next_buffer()
+        rc = self._lib.conef_cs_update_f32(vec.data_ptr(), self.cs.data_ptr(), out.data_ptr(), self.N, self.D,
+                                           self.range, float(beta), self.a, self.b, _lib.stream_ptr(vec))
+        _lib.check(rc, "conef_cs_update_f32")
+        self.commit(out)
+
+    def query(self, grad_plus_error, alpha):
+        """grad_plus_error += alpha * unsketch(cs), in place (CountSketch.py:70-98)."""
+        self._check(grad_plus_error, "grad_plus_error")
+        rc = self._lib.conef_cs_query_f32(grad_plus_error.data_ptr(), self.cs.data_ptr(), self.N, self.D,
+                                          self.range, float(alpha), self.a, self.b,
+                                          _lib.stream_ptr(grad_plus_error))
+        _lib.check(rc, "conef_cs_query_f32")
+
+    def clean(self, alpha):
+        """cs *= alpha (CountSketch.py:181-182)."""
+        rc = self._lib.conef_scale_f32(self.cs.data_ptr(), self.cs.numel(), float(alpha),
+                                       _lib.stream_ptr(self.cs))
+        _lib.check(rc, "conef_scale_f32")

@@ -1,0 +1,113 @@
+"""PowerSGD with a magnitude-sparsified (top-k) error as a DDP communication hook.
+
+Drop-in for the reference's communication/hPowerSGD_hook.py: ``hPowerSGDState`` keeps the
+arguments and defaults of :157-233, ``hpowerSGD_hook`` the contract of :274-570.  With
+``use_error_compression`` the residual of every compressed matrix is kept dense and cut down to
+its ``int(0.5 * topk_ratio * numel)`` largest magnitudes after each step (:90-97,:549-554);
+without it the hook is plain PowerSGD with dense error feedback over the whole bucket.
+"""
+import logging
+
+import numpy as np
+import torch
+
+from . import _bucket
+from ._psgd_engine import orthogonalize as _orthogonalize  # noqa: F401
+from ._psgd_engine import run_round, topk_sparsify
+from ._psgd_engine import should_compress as _should_compress  # noqa: F401
+
+
+def _topk(error_tensor, topk_ratio):
+    """In-place magnitude top-k of a device tensor (reference name, :90-97)."""
+    topk_sparsify(error_tensor, topk_ratio)
+
+
+class hPowerSGDState(object):
+    __slots__ = [
+        "process_group",
+        "matrix_approximation_rank",
+        "start_powerSGD_iter",
+        "min_compression_rate",
+        "orthogonalization_epsilon",
+        "use_error_compression",
+        "topk_ratio",
+        "use_error_feedback",
+        "warm_start",
+        "rng",
+        "error_dict",
+        "p_memory_dict",
+        "q_memory_dict",
+        "iter",
+        "total_numel_before_compression",
+        "total_numel_after_compression",
+        "compression_stats_logging_frequency",
+        "next_stats_report",
+    ]
+
+    def __init__(
+        self,
+        process_group,
+        matrix_approximation_rank=1,
+        start_powerSGD_iter=1_000,
+        min_compression_rate=2,
+        use_error_compression=False,
+        use_error_feedback=True,
+        topk_ratio=0.4,
+        warm_start=True,
+        orthogonalization_epsilon=0,
+        random_seed=0,
+        compression_stats_logging_frequency=10_000,
+    ):
+        if (use_error_feedback or warm_start) and start_powerSGD_iter <= 1:
+            raise ValueError(
+                "Expect `start_powerSGD_iter` > 1 if `use_error_feedback` or `warm_start` is enabled, "
+                "because PowerSGD can only be applied after the first two iterations in DDP."
+            )
+        self.process_group = process_group
+        self.matrix_approximation_rank = matrix_approximation_rank
+        self.start_powerSGD_iter = start_powerSGD_iter
+        self.min_compression_rate = min_compression_rate
+        self.use_error_feedback = use_error_feedback
+        self.warm_start = warm_start
+        self.orthogonalization_epsilon = orthogonalization_epsilon
+        self.rng = np.random.RandomState(random_seed)
+        self.error_dict = {}
+        self.p_memory_dict = {}
+        self.q_memory_dict = {}
+        self.iter = 0
+        self.total_numel_before_compression = 0
+        self.total_numel_after_compression = 0
+        self.compression_stats_logging_frequency = max(1, compression_stats_logging_frequency)
+        self.next_stats_report = 0
+        self.use_error_compression = use_error_compression
+        self.topk_ratio = topk_ratio
+
+    def maybe_increase_iter(self, bucket):
+        if _bucket.is_last(bucket):
+            self.iter += 1
+        if self.iter == self.start_powerSGD_iter:
+            logging.info("Start to apply PowerSGD after {} iterations.".format(self.iter))
+
+    def compression_stats(self):
+        after = self.total_numel_after_compression
+        rate = self.total_numel_before_compression / after if after > 0 else 0
+        return (rate, self.total_numel_before_compression, after)
+
+    def clean_error(self):
+        """Zeroes the kept errors.  (The reference calls ``.clean(0)`` on dense tensors here,
+        :267-271, which would raise; zeroing is what that call means.)"""
+        if self.use_error_feedback:
+            for per_bucket in self.error_dict.values():
+                if isinstance(per_bucket, dict):
+                    for err in per_bucket.values():
+                        err.zero_()
+                else:
+                    per_bucket.zero_()
+
+
+def hpowerSGD_hook(state: hPowerSGDState, bucket) -> torch.futures.Future:
+    if not state.use_error_feedback:
+        mode = None
+    else:
+        mode = "topk" if state.use_error_compression else "ef"
+    return run_round(state, bucket, mode)

@@ -1,0 +1,182 @@
+/*
+ * conef_hip.h - C ABI of libconef_hip.so, the MI355X (gfx950) kernels behind the ConEF
+ * gradient-compression hooks.
+ *
+ * This is the boundary the reference crosses in communication/compressors/cupy_kernel.py:36-45
+ * (`func(grid, block, args, smem, stream=...)` with raw `tensor.data_ptr()` integers), widened to
+ * the torch-op sequences of the hooks that are fused into single kernels here.  Conventions:
+ *
+ *   - every pointer is a DEVICE pointer into memory the caller owns and keeps alive until the
+ *     stream has run the call (the one exception, conef_hash_table_host_i32, takes host memory);
+ *   - `stream` is a hipStream_t (NULL = the default stream); every call is asynchronous on it,
+ *     never synchronises the host, never allocates or frees, keeps no global or thread-local
+ *     state and may be called from any thread;
+ *   - scalars (alpha, beta, hash seeds) travel by value - the reference passes them as pointers
+ *     to 1-element device tensors it allocates per call (CountSketch.py:144,167);
+ *   - matrices are dense row-major fp32; a sketch is [n, w] row-major, fp32 unless the name says f16;
+ *   - return value: 0 = enqueued, -1 = invalid argument (nothing enqueued), > 0 = hipError_t.
+ *   - empty inputs (n == 0 or d == 0) are accepted and do nothing.
+ *
+ * Floating point: multiplications and additions are done in the order the reference's kernels
+ * write them, without contraction; only the order in which a sketch cell accumulates its terms is
+ * not fixed (the reference uses float atomicAdd and does not fix it either).
+ */
+#ifndef CONEF_HIP_H
+#define CONEF_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CONEF_OK 0
+#define CONEF_ERR_INVALID (-1)
+
+/* Library ABI version (1). */
+int conef_version(void);
+
+/* ---------------------------------------------------------------- hashing ---------------- */
+
+/* bucket[i] = hash(i, w, a, b), sign[i] = (hash(i, w, sa, sb) & 1) ? +1 : -1 for i in [0, d).
+ * Replaces: the `hash` device function and its two call sites, CountSketch.py:7-18,60-62.
+ * Exists so that buckets and signs can be checked bit for bit against the reference arithmetic. */
+int conef_hash_table_i32(int32_t* bucket, int32_t* sign, int64_t d, int32_t w, int32_t a, int32_t b,
+                         int32_t sa, int32_t sb, void* stream);
+
+/* Same table computed on the HOST by the host compilation of the same source (host pointers, no
+ * stream): lets a machine without a GPU check the shipped hash, fast modulo included. */
+int conef_hash_table_host_i32(int32_t* bucket, int32_t* sign, int64_t d, int32_t w, int32_t a, int32_t b,
+                              int32_t sa, int32_t sb);
+
+/* ------------------------------------------------------- one-hash count sketch ---------- */
+
+/* x[r,i] += (sign_i * cs[r, bucket_i]) * alpha, x is [n,d], cs is [n,w].
+ * Replaces: kernel dense_cs_query, CountSketch.py:70-98, launched from DenseCS.query :165-179. */
+int conef_cs_query_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
+                       int32_t b, void* stream);
+
+/* cs_out[r,j] = cs_in[r,j] + sum_{i: bucket_i = j} fl32( sign_i*(vec[r,i] - (1.-beta)*sign_i*cs_in[r,j]) ),
+ * the inner expression in double as in the reference.
+ * Replaces: kernel dense_cs_update, CountSketch.py:27-67, launched from DenseCS.update :143-158.
+ * cs_out may be the same buffer as cs_in only if conef_cs_update_inplace_ok(n,d,w) is 1 (a sketch
+ * row then fits LDS and is snapshotted there, as the reference does in shared memory :47-52);
+ * otherwise the snapshot is cs_in itself and cs_out must be a different buffer (-1 if not). */
+int conef_cs_update_f32(const float* vec, const float* cs_in, float* cs_out, int64_t n, int64_t d, int32_t w,
+                        float beta, int32_t a, int32_t b, void* stream);
+
+/* 1 if an update (or fused step) of this shape may run in place, else 0.  Pure host function. */
+int conef_cs_update_inplace_ok(int64_t n, int64_t d, int32_t w);
+
+/* fp16-storage variants: cells are read as fp16, all arithmetic is fp32, cells are rounded to
+ * nearest-even once when written.  Replaces: halfCountSketch.py:151-194, which casts the whole
+ * sketch to fp32 before and back to fp16 after each kernel.  The update requires
+ * conef_cs_update_inplace_ok(n,d,w) == 1 (larger sketches: convert, f32 update, convert back). */
+int conef_cs_query_f16(float* x, const void* cs_half, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
+                       int32_t b, void* stream);
+int conef_cs_update_f16(const float* vec, const void* cs_in_half, void* cs_out_half, int64_t n, int64_t d,
+                        int32_t w, float beta, int32_t a, int32_t b, void* stream);
+int conef_convert_f16_to_f32(float* dst, const void* src_half, int64_t count, void* stream);
+int conef_convert_f32_to_f16(void* dst_half, const float* src, int64_t count, void* stream);
+
+/* x *= alpha.  Replaces: DenseCS.clean, CountSketch.py:181-182 / halfCountSketch.py:196-197. */
+int conef_scale_f32(float* x, int64_t count, float alpha, void* stream);
+int conef_scale_f16(void* x_half, int64_t count, float alpha, void* stream);
+
+/* ----------------------------------------------------- three-hash count sketch ---------- */
+
+/* x[r,i] += median_k( sign_k,i * cs_k[r, bucket_k,i] * alpha ), k = 0..2, fixed hash constants.
+ * Replaces: CountSketchHash3.py:101-147 (query uses sign seed (a2+8, b2+7) for the third hash). */
+int conef_cs3_query_f32(float* x, const float* cs0, const float* cs1, const float* cs2, int64_t n, int64_t d,
+                        int32_t w, float alpha, void* stream);
+
+/* Median-coupled update of the three sketches.  Replaces: CountSketchHash3.py:27-98 (update uses
+ * sign seed (a2+8, b2+4) for the third hash).  out_k must differ from in_k. */
+int conef_cs3_update_f32(const float* vec, const float* in0, const float* in1, const float* in2, float* out0,
+                         float* out1, float* out2, int64_t n, int64_t d, int32_t w, float beta, void* stream);
+
+/* ------------------------------------------------------------ random block ------------- */
+/* The block is the wrap-around range [start, start+block) of the flat tensor: [start, end) with
+ * end = min(start+block, numel), then [0, block-(end-start)).  0 <= start < numel, 1 <= block <= numel. */
+
+/* One fused RandomBlock + count-sketch error-feedback step on one [n,m] gradient, in place:
+ *   xq = x + alpha*unsketch(cs_in);  payload = xq[block];  x = xq on the block, 0 elsewhere;
+ *   cs_out = update(cs_in, xq off the block / 0 on it, beta).
+ * Replaces, for one tensor: DenseCS.query, clone, slice copies, zero_ calls, DenseCS.update,
+ * tensor.zero_ and copies back of RandomBlock_hook.py:190,216-243,272-280 (world size 1).
+ * Aliasing of cs_out/cs_in as for conef_cs_update_f32. */
+int conef_randblock_conef_step_f32(float* x, const float* cs_in, float* cs_out, float* payload, int64_t n,
+                                   int64_t m, int32_t w, int64_t start, int64_t block, float alpha, float beta,
+                                   int32_t a, int32_t b, void* stream);
+
+/* Same step with a dense error tensor: xq = x + err; payload = xq[block]; x = xq on the block,
+ * 0 elsewhere; err = 0 on the block, xq elsewhere.
+ * Replaces: RandomBlock_hook.py:182-184,222,228,237,240,276-280. */
+int conef_randblock_ef_step_f32(float* x, float* err, float* payload, int64_t numel, int64_t start,
+                                int64_t block, void* stream);
+
+/* Unbiased variant: payload = x[block] / prob; x = payload on the block, 0 elsewhere.
+ * Replaces: UnbiasedRandomBlock_hook.py:155,161-167,200-204. */
+int conef_randblock_unbiased_step_f32(float* x, float* payload, int64_t numel, int64_t start, int64_t block,
+                                      float prob, void* stream);
+
+/* The two halves a multi-rank caller puts around its all-reduce of the payload:
+ * gather: payload[p] = x[(start+p) mod numel] / scale;  scatter: x = 0 except the block = payload.
+ * Replace: RandomBlock_hook.py:222,237 and :276-280. */
+int conef_randblock_gather_f32(const float* x, float* payload, int64_t numel, int64_t start, int64_t block,
+                               float scale, void* stream);
+int conef_randblock_scatter_f32(float* x, const float* payload, int64_t numel, int64_t start, int64_t block,
+                                void* stream);
+
+/* ------------------------------------------------------------------ PowerSGD ---------- */
+/* M is [n,m], Q is [m,r], P is [n,r], 1 <= r <= 32. */
+
+/* In-place Gram-Schmidt of a row-major [rows, r] matrix: column by column, col /= ||col|| (+ eps
+ * if eps != 0), then every later column loses its projection on col.
+ * Replaces: _orthogonalize, powerSGD_hook.py:12-44 (about 4r torch kernels per matrix). */
+int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* stream);
+
+/* P = M Q.  Replaces: torch.matmul(tensor, q, out=p), powerSGD_hook.py:498. */
+int conef_psgd_mq_f32(float* x, const float* q, float* p, int64_t n, int64_t m, int32_t r, void* stream);
+/* M += E (kept in M), then P = M Q.  Replaces: input_tensor.add_(error) :361 + :498 for one matrix
+ * (also hPowerSGD_hook.py:399). */
+int conef_psgd_mq_ef_f32(float* x, const float* err, const float* q, float* p, int64_t n, int64_t m, int32_t r,
+                         void* stream);
+/* M += alpha*unsketch(cs) (kept in M), then P = M Q.  Replaces: DenseCS.query :409 + :498. */
+int conef_psgd_mq_conef_f32(float* x, const float* cs, const float* q, float* p, int64_t n, int64_t m,
+                            int32_t r, int32_t w, float alpha, int32_t a, int32_t b, void* stream);
+
+/* Q = M^T P.  Replaces: torch.matmul(tensor.t(), p, out=q), powerSGD_hook.py:532. */
+int conef_psgd_mtp_f32(const float* x, const float* p, float* q, int64_t n, int64_t m, int32_t r, void* stream);
+
+/* M = P Q^T.  Replaces: torch.matmul(p, q.t(), out=tensor), powerSGD_hook.py:551. */
+int conef_psgd_pqt_f32(float* x, const float* p, const float* q, int64_t n, int64_t m, int32_t r, void* stream);
+/* E = M - P Q^T, then M = P Q^T.  Replaces: clone :375 + :551 + `input_tensor_cp - input_tensor` :558
+ * for one matrix (also hPowerSGD_hook.py:553). */
+int conef_psgd_pqt_ef_f32(float* x, float* err, const float* p, const float* q, int64_t n, int64_t m, int32_t r,
+                          void* stream);
+/* cs_out = update(cs_in, M - P Q^T, beta), then M = P Q^T.  Replaces: clone :410 + :551 +
+ * cp_tensor.add_(-1, tensor) :563 + DenseCS.update :564.  Aliasing as for conef_cs_update_f32. */
+int conef_psgd_pqt_conef_f32(float* x, const float* p, const float* q, const float* cs_in, float* cs_out,
+                             int64_t n, int64_t m, int32_t r, int32_t w, float beta, int32_t a, int32_t b,
+                             void* stream);
+
+/* Dense error feedback on a stretch of the bucket that is not compressed: x += err; err = 0
+ * (the copy-minus-result of powerSGD_hook.py:558 is exactly zero there). */
+int conef_ef_passthrough_f32(float* x, float* err, int64_t count, void* stream);
+
+/* ------------------------------------------------------------- magnitude top-k ---------- */
+
+/* Bytes of device workspace conef_topk_sparsify_f32 needs for `numel` elements (host function). */
+int64_t conef_topk_workspace_bytes(int64_t numel);
+
+/* Keeps the k entries of largest magnitude of x[0..numel) and zeroes the rest, in place; ties on
+ * the threshold magnitude keep the lowest indices.  k >= numel keeps everything.
+ * Replaces: _topk, hPowerSGD_hook.py:90-97 (torch.topk on |x|, zero_, scatter back). */
+int conef_topk_sparsify_f32(float* x, int64_t numel, int64_t k, void* workspace, int64_t workspace_bytes,
+                            void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CONEF_HIP_H */

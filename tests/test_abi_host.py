@@ -1,0 +1,143 @@
+"""CPU-only checks of the native boundary: the library is built in-tree, loads, exports every
+entry point include/conef_hip.h declares with the arity the Python binding uses, rejects bad
+arguments before touching a GPU, and its hash (compiled for the host from the same source the
+kernels use) agrees with the oracle bit for bit.  No device compute is called here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "conef_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for m in re.finditer(r"\b(?:int|int64_t)\s+(conef_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+        args = m.group(2).strip()
+        out[m.group(1)] = 0 if args == "void" else len([a for a in args.split(",") if a.strip()])
+    return out
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from conef_amd import _lib
+    return _lib.load()
+
+
+def test_header_library_and_binding_agree(lib):
+    from conef_amd import _lib
+    decl = declared_functions()
+    assert len(decl) >= 30
+    assert set(decl) == set(_lib.SIGNATURES), set(decl) ^ set(_lib.SIGNATURES)
+    raw = ctypes.CDLL(_lib.LIBPATH)
+    for name, nargs in decl.items():
+        assert hasattr(raw, name), "library does not export %s" % name
+        assert nargs == len(_lib.SIGNATURES[name]), name
+    assert lib.conef_version() == 1
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from conef_amd import _lib
+    monkeypatch.setattr(_lib, "_handle", None)
+    monkeypatch.setattr(_lib, "LIBPATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.ConefLibraryError, match="no CPU fallback"):
+        _lib.load()
+
+
+def test_argument_validation_without_gpu(lib):
+    # all of these are refused on the host before any launch
+    assert lib.conef_cs_query_f32(1, 1, 1, 1, 0, 0.1, 1, 1, 0) == -1            # w < 1
+    assert lib.conef_cs_query_f32(0, 0, 2, 2, 4, 0.1, 1, 1, 0) == -1            # null pointers
+    assert lib.conef_cs_update_f32(1, 1, 1, -1, 1, 1, 0.9, 1, 1, 0) == -1
+    assert lib.conef_randblock_ef_step_f32(1, 1, 1, 10, 10, 1, 0) == -1         # start == numel
+    assert lib.conef_randblock_ef_step_f32(1, 1, 1, 10, 0, 11, 0) == -1         # block > numel
+    assert lib.conef_randblock_unbiased_step_f32(1, 1, 10, 0, 1, 0.0, 0) == -1  # prob must be > 0
+    assert lib.conef_gram_schmidt_f32(1, 10, 33, 0.0, 0) == -1                  # rank above 32
+    assert lib.conef_psgd_mq_f32(1, 1, 1, 4, 4, 0, 0) == -1
+    assert lib.conef_topk_sparsify_f32(1, 100, 10, 0, 0, 0) == -1               # no workspace
+    assert lib.conef_topk_sparsify_f32(1, 100, 100, 0, 0, 0) == 0               # k >= numel: nothing to do
+    assert lib.conef_topk_workspace_bytes(1 << 20) >= 4 * 1024
+    # shapes: short rows may update in place, the flat 25 MB bucket may not
+    assert lib.conef_cs_update_inplace_ok(640, 5760, 1152) == 1
+    assert lib.conef_cs_update_inplace_ok(5, 1_300_000, 130_000) == 0
+
+
+@pytest.mark.parametrize("d,w", [(1, 1), (1000, 7), (70_000, 65), (5760, 1152), (200_000, 130_000),
+                                 (100_000, 1 << 30), (300_000, 3), (65_536, 2), (50_000, 99_991)])
+def test_shipped_hash_matches_oracle_on_host(lib, oracle, d, w):
+    for (a, b, sa, sb) in [(994443, 609478, 994445, 609481), (4113759, 2949676, 4113763, 2949681),
+                           (9171025, 2171464, 9171033, 2171468), (9171025, 2171464, 9171033, 2171471)]:
+        bucket = np.empty(d, np.int32)
+        sign = np.empty(d, np.int32)
+        assert lib.conef_hash_table_host_i32(bucket.ctypes.data, sign.ctypes.data, d, w, a, b, sa, sb) == 0
+        ob, osg = oracle.hash_table(d, w, a, b, sa, sb)
+        np.testing.assert_array_equal(bucket, ob)
+        np.testing.assert_array_equal(sign, osg)
+
+
+def test_fast_modulo_near_multiples(lib, oracle):
+    # widths chosen so that many hash values sit next to a multiple of w, where a quotient
+    # estimated in floating point is most likely to be off by one
+    for w in (1, 2, 3, 7, 1000, 65_535, 65_536, 65_537, (1 << 30) - 1, 1 << 30):
+        d = 20_000
+        bucket = np.empty(d, np.int32)
+        sign = np.empty(d, np.int32)
+        assert lib.conef_hash_table_host_i32(bucket.ctypes.data, sign.ctypes.data, d, w, 1, 0, 3, 5) == 0
+        ob, osg = oracle.hash_table(d, w, 1, 0, 3, 5)
+        np.testing.assert_array_equal(bucket, ob)
+        np.testing.assert_array_equal(sign, osg)
+
+
+def test_states_and_host_logic_need_no_gpu():
+    from conef_amd.RandomBlock_hook import RandomBlockState
+    from conef_amd.UnbiasedRandomBlock_hook import UnbiasedRandomBlockState
+    from conef_amd.hPowerSGD_hook import hPowerSGDState
+    from conef_amd.powerSGD_hook import PowerSGDState, _should_compress
+    with pytest.raises(ValueError, match="Expect `start_compression_iter` > 1"):
+        RandomBlockState(None, start_compression_iter=1)
+    with pytest.raises(ValueError, match="Expect `use_error_feedback` = True if `use_error_compression`"):
+        RandomBlockState(None, start_compression_iter=2, use_error_feedback=False, use_error_compression=True)
+    with pytest.raises(ValueError, match="Expect `start_compression_iter` > 1"):
+        UnbiasedRandomBlockState(None, start_compression_iter=1)
+    for cls in (PowerSGDState, hPowerSGDState):
+        with pytest.raises(ValueError, match="Expect `start_powerSGD_iter` > 1"):
+            cls(None, start_powerSGD_iter=1)
+        cls(None, start_powerSGD_iter=1, use_error_feedback=False, warm_start=False)
+    s = RandomBlockState(None, start_compression_iter=2)
+    assert (s.compression_ratio, s.beta, s.sketch_size, s.use_error_feedback, s.use_error_compression) == \
+        (0.1, 0.9, 0.5, True, False)
+    assert [int(s.rng.choice(6_500_000)) for _ in range(2)] == [6413414, 6423388]
+    p = PowerSGDState(None, start_powerSGD_iter=2)
+    assert (p.matrix_approximation_rank, p.min_compression_rate, p.warm_start, p.beta, p.sketch_size) == \
+        (1, 2, True, 0.9, 0.5)
+    assert int(p.rng.randint(1_000_000_000)) == 209652396
+    assert hPowerSGDState(None, start_powerSGD_iter=2).topk_ratio == 0.4
+    # BERT's [2,1024] pooler-adjacent weight is not worth compressing at rank 8, [1024,1024] is
+    assert _should_compress(2, 1024, 2, 2) == (False, 2048, 2052)
+    assert _should_compress(1024, 1024, 8, 2)[0] is True
+    assert p.compression_stats() == (0, 0, 0)
+
+
+def test_hooks_refuse_host_tensors():
+    import torch
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from _helpers import FakeGradBucket
+    from conef_amd.RandomBlock_hook import RandomBlock_hook, RandomBlockState
+    from conef_amd.powerSGD_hook import PowerSGDState, powerSGD_hook
+    st = RandomBlockState(None, start_compression_iter=2)
+    g = torch.zeros(40)
+    out = RandomBlock_hook(st, FakeGradBucket(g, [(4, 10)])).wait()      # warm-up: identity all-reduce
+    assert out is g and st.iter == 1
+    st.iter = 2
+    with pytest.raises(ValueError, match="no CPU path"):
+        RandomBlock_hook(st, FakeGradBucket(g, [(4, 10)]))
+    ps = PowerSGDState(None, start_powerSGD_iter=2)
+    ps.iter = 2
+    with pytest.raises(ValueError, match="no CPU path"):
+        powerSGD_hook(ps, FakeGradBucket(g, [(4, 10)]))

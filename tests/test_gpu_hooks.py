@@ -1,0 +1,269 @@
+"""GPU parity of the communication hooks against the CPU oracle's restatement of the reference
+hooks, on the same seeded gradients with state carried across steps."""
+import numpy as np
+import pytest
+import torch
+
+from _helpers import FakeGradBucket, OldApiGradBucket, assert_close, heavy_tail_gradient, to_np
+
+pytestmark = pytest.mark.gpu
+
+RESNET20_SHAPES = ([(16, 3, 3, 3), (16,), (16,)] + [(16, 16, 3, 3), (16,), (16,)] * 6 +
+                   [(32, 16, 3, 3), (32,), (32,)] + [(32, 32, 3, 3), (32,), (32,)] * 5 +
+                   [(64, 32, 3, 3), (64,), (64,)] + [(64, 64, 3, 3), (64,), (64,)] * 5 + [(10, 64), (10,)])
+
+
+def numel_of(shapes):
+    return sum(int(np.prod(s)) for s in shapes)
+
+
+def grads(total, seed, sigma=1e-3):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(total, generator=g) * sigma).float()
+
+
+def run_steps(hook, state, ostate, shapes, steps, bucket_cls=FakeGradBucket, seed0=100, check=None):
+    total = numel_of(shapes)
+    state.iter = getattr(state, "start_compression_iter", None) or state.start_powerSGD_iter
+    for step in range(steps):
+        g = grads(total, seed0 + step)
+        gd = g.cuda()
+        out = hook(state, bucket_cls(gd, shapes)).wait()
+        assert out.data_ptr() == gd.data_ptr()        # in place, same buffer back
+        og = g.numpy().copy()
+        ostate.step(0, og, shapes)
+        check(step, gd, og)
+    return state
+
+
+# ------------------------------------------------------------- RandomBlock --
+
+@pytest.mark.parametrize("shapes,ratio", [([(6, 5, 3), (7,), (4, 9)], 0.3), (RESNET20_SHAPES, 0.1),
+                                          ([(5, 26_000)], 0.1), ([(3, 4), (1,)], 0.01)])
+def test_randomblock_dense_ef_bit_exact(oracle, shapes, ratio):
+    from conef_amd.RandomBlock_hook import RandomBlock_hook, RandomBlockState
+    st = RandomBlockState(None, compression_ratio=ratio, start_compression_iter=2)
+    ost = oracle.RandomBlockOracle(compression_ratio=ratio)
+
+    def check(step, gd, og):
+        np.testing.assert_array_equal(to_np(gd), og)                       # adds, copies and zeros only
+        for e, oe in zip(st.error_dict[0], ost.error_dict[0]):
+            np.testing.assert_array_equal(to_np(e), oe)
+        np.testing.assert_array_equal(to_np(st.compressed_tensor_memory[0]), ost.compressed_tensor_memory[0])
+
+    run_steps(RandomBlock_hook, st, ost, shapes, 4, check=check)
+    assert st.iter == 2 + 4
+
+
+@pytest.mark.parametrize("shapes,ratio,ss", [([(6, 5, 3), (7,), (4, 9)], 0.3, 0.5), (RESNET20_SHAPES, 0.1, 0.2),
+                                             ([(5, 26_000)], 0.1, 0.1), ([(40, 650), (650,), (26, 650)], 0.05, 0.1)])
+@pytest.mark.parametrize("bucket_cls", [FakeGradBucket, OldApiGradBucket])
+def test_randomblock_conef_parity(oracle, shapes, ratio, ss, bucket_cls):
+    from conef_amd.RandomBlock_hook import RandomBlock_hook, RandomBlockState
+    st = RandomBlockState(None, compression_ratio=ratio, start_compression_iter=2, use_error_compression=True,
+                          sketch_size=ss, beta=0.9)
+    ost = oracle.RandomBlockOracle(compression_ratio=ratio, use_error_compression=True, sketch_size=ss, beta=0.9)
+
+    def check(step, gd, og):
+        assert_close(gd, og, what="decompressed gradient, step %d" % step)
+        np.testing.assert_array_equal(to_np(gd) != 0, og != 0)             # same selected indices
+        assert_close(st.compressed_tensor_memory[0], ost.compressed_tensor_memory[0], what="payload")
+        for k, (cs, ocs) in enumerate(zip(st.error_dict[0], ost.error_dict[0])):
+            assert_close(cs.cs, ocs.cs, what="sketch %d, step %d" % (k, step))
+
+    run_steps(RandomBlock_hook, st, ost, shapes, 5, bucket_cls=bucket_cls, check=check)
+
+
+def test_randomblock_warmup_and_errors():
+    from conef_amd.RandomBlock_hook import RandomBlock_hook, RandomBlockState
+    with pytest.raises(ValueError, match="Expect `start_compression_iter` > 1"):
+        RandomBlockState(None, start_compression_iter=1)
+    with pytest.raises(ValueError, match="Expect `use_error_feedback` = True if `use_error_compression`"):
+        RandomBlockState(None, start_compression_iter=2, use_error_feedback=False, use_error_compression=True)
+    st = RandomBlockState(None, start_compression_iter=2)
+    g = torch.randn(40, device="cuda")
+    before = g.clone()
+    for it in range(2):                                   # plain all-reduce phase: identity at world size 1
+        out = RandomBlock_hook(st, FakeGradBucket(g, [(4, 10)])).wait()
+        assert torch.equal(out, before)
+    assert st.iter == 2
+    RandomBlock_hook(st, FakeGradBucket(g, [(4, 10)], is_last=False)).wait()
+    assert st.iter == 2                                   # only the last bucket closes an iteration
+    assert int((g != 0).sum()) == 4
+    st2 = RandomBlockState(None, start_compression_iter=2, use_error_feedback=False)
+    st2.iter = 2
+    with pytest.raises(KeyError):
+        RandomBlock_hook(st2, FakeGradBucket(g, [(4, 10)]))
+    with pytest.raises(ValueError, match="no CPU path"):
+        RandomBlock_hook(st, FakeGradBucket(torch.zeros(40), [(4, 10)]))
+
+
+def test_randomblock_two_buckets_share_one_rng(oracle):
+    from conef_amd.RandomBlock_hook import RandomBlock_hook, RandomBlockState
+    st = RandomBlockState(None, compression_ratio=0.2, start_compression_iter=2)
+    st.iter = 2
+    ost = oracle.RandomBlockOracle(compression_ratio=0.2)
+    layout = {1: [(8, 9), (3,)], 0: [(5, 5), (6, 7)]}
+    for step in range(3):
+        for bi in (1, 0):                                 # buckets arrive in reverse order, 0 last
+            g = grads(numel_of(layout[bi]), 10 * step + bi)
+            gd = g.cuda()
+            RandomBlock_hook(st, FakeGradBucket(gd, layout[bi], index=bi, is_last=(bi == 0))).wait()
+            og = g.numpy().copy()
+            ost.step(bi, og, layout[bi])
+            np.testing.assert_array_equal(to_np(gd), og)
+    assert st.iter == 5
+
+
+# ------------------------------------------------------------------ Unbiased --
+
+@pytest.mark.parametrize("shapes,ratio", [([(6, 5, 3), (7,), (4, 9)], 0.3), ([(700, 650), (650,), (26, 650)], 0.05)])
+def test_unbiased_randomblock_bit_exact(oracle, shapes, ratio):
+    from conef_amd.UnbiasedRandomBlock_hook import UnbiasedRandomBlock_hook, UnbiasedRandomBlockState
+    st = UnbiasedRandomBlockState(None, compression_ratio=ratio, start_compression_iter=2)
+    ost = oracle.UnbiasedRandomBlockOracle(compression_ratio=ratio)
+
+    def check(step, gd, og):
+        np.testing.assert_array_equal(to_np(gd), og)
+        np.testing.assert_array_equal(to_np(st.compressed_tensor_memory[0]), ost.compressed_tensor_memory[0])
+
+    run_steps(UnbiasedRandomBlock_hook, st, ost, shapes, 4, check=check)
+    with pytest.raises(ValueError):
+        UnbiasedRandomBlockState(None, start_compression_iter=0)
+
+
+# ------------------------------------------------------------------ PowerSGD --
+
+def test_gram_schmidt_parity(oracle):
+    from conef_amd.powerSGD_hook import _orthogonalize
+    for rows, r, eps in [(27, 1, 0.0), (576, 2, 0.0), (5760, 4, 0.0), (1024, 8, 0.0), (4096, 32, 0.0),
+                         (300, 3, 1e-8), (33278, 4, 0.0), (2000, 13, 0.0)]:
+        g = torch.Generator().manual_seed(rows + r)
+        a = torch.randn(rows, r, generator=g)
+        want = a.numpy().copy()
+        oracle.gram_schmidt(want, eps)
+        got = a.cuda()
+        _orthogonalize(got, eps)
+        assert_close(got, want, what="gram-schmidt %dx%d" % (rows, r))
+        gg = to_np(got).astype(np.float64)
+        np.testing.assert_allclose(gg.T @ gg, np.eye(r), atol=2e-5)
+
+
+def test_products_parity(oracle):
+    from conef_amd import _lib
+    lib = _lib.load()
+    rng = np.random.RandomState(0)
+    for n, m, r in [(16, 27, 2), (64, 576, 2), (640, 5760, 4), (13, 29, 3), (1024, 1024, 8), (300, 4096, 32),
+                    (1000, 77, 1), (9, 4100, 16)]:
+        M = rng.randn(n, m).astype(np.float32)
+        Q = rng.randn(m, r).astype(np.float32)
+        P = rng.randn(n, r).astype(np.float32)
+        Md, Qd, Pd = (torch.from_numpy(t).cuda() for t in (M, Q, P))
+        out = torch.empty(n, r, device="cuda")
+        assert lib.conef_psgd_mq_f32(Md.data_ptr(), Qd.data_ptr(), out.data_ptr(), n, m, r, 0) == 0
+        assert_close(out, oracle.mq(M, Q), what="MQ %s" % ((n, m, r),))
+        outq = torch.empty(m, r, device="cuda")
+        assert lib.conef_psgd_mtp_f32(Md.data_ptr(), Pd.data_ptr(), outq.data_ptr(), n, m, r, 0) == 0
+        assert_close(outq, oracle.mtp(M, P), what="MtP %s" % ((n, m, r),))
+        outm = torch.empty(n, m, device="cuda")
+        assert lib.conef_psgd_pqt_f32(outm.data_ptr(), Pd.data_ptr(), Qd.data_ptr(), n, m, r, 0) == 0
+        assert_close(outm, oracle.pqt(P, Q), what="PQt %s" % ((n, m, r),))
+
+
+def psgd_check_factory(st, ost, mode):
+    def check(step, gd, og):
+        assert_close(gd, og, what="%s: decompressed bucket, step %d" % (mode, step))
+        for p, op in zip(_views(st.p_memory_dict[0], ost.p_memory_dict[0]), ost.p_memory_dict[0]):
+            assert_close(p, op, what="P")
+        for q, oq in zip(_views(st.q_memory_dict[0], ost.q_memory_dict[0]), ost.q_memory_dict[0]):
+            assert_close(q, oq, what="Q")
+        if mode == "ef":
+            assert_close(st.error_dict[0], ost.error_dict[0], what="dense error, step %d" % step)
+        elif mode == "conef":
+            for k in ost.error_dict[0]:
+                assert_close(st.error_dict[0][k].cs, ost.error_dict[0][k].cs, what="sketch %d step %d" % (k, step))
+        elif mode == "topk":
+            for k in ost.error_dict[0]:
+                got, want = to_np(st.error_dict[0][k]), ost.error_dict[0][k]
+                # the kept set may differ where two magnitudes are within rounding of the threshold
+                assert (np.count_nonzero(got) == np.count_nonzero(want))
+                same = (got != 0) == (want != 0)
+                assert same.mean() > 0.999
+                assert_close(np.where(same, got, 0), np.where(same, want, 0), what="top-k error %d" % k)
+    return check
+
+
+def _views(flat, like):
+    out, off = [], 0
+    for arr in like:
+        out.append(flat[off: off + arr.size].view(*arr.shape))
+        off += arr.size
+    return out
+
+
+PSGD_CASES = [
+    (RESNET20_SHAPES, 2, 0.5),
+    ([(640, 1440), (640,), (320, 2880), (40, 33)], 4, 0.2),
+    ([(1024, 1024), (1024,), (512, 1024), (2, 1024)], 8, 0.1),
+    ([(256, 1024), (1024, 256)], 32, 0.1),
+]
+
+
+@pytest.mark.parametrize("shapes,rank,ss", PSGD_CASES)
+@pytest.mark.parametrize("mode", [None, "ef", "conef"])
+def test_powersgd_hook_parity(oracle, shapes, rank, ss, mode):
+    from conef_amd.powerSGD_hook import PowerSGDState, powerSGD_hook
+    st = PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2,
+                       use_error_feedback=mode is not None, use_error_compression=mode == "conef",
+                       sketch_size=ss, beta=0.9)
+    ost = oracle.PowerSGDOracle(matrix_approximation_rank=rank, error_mode=mode, sketch_size=ss, beta=0.9)
+    run_steps(powerSGD_hook, st, ost, shapes, 4, check=psgd_check_factory(st, ost, mode))
+    rate, before, after = st.compression_stats()
+    assert before == 4 * numel_of(shapes) and 0 < after < before and rate > 1
+
+
+def test_hpowersgd_topk_parity(oracle):
+    from conef_amd.hPowerSGD_hook import hPowerSGDState, hpowerSGD_hook
+    shapes, rank = [(640, 1440), (640,), (320, 2880), (40, 33)], 4
+    st = hPowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, use_error_compression=True,
+                        topk_ratio=0.4)
+    ost = oracle.PowerSGDOracle(matrix_approximation_rank=rank, error_mode="topk", topk_ratio=0.4)
+    run_steps(hpowerSGD_hook, st, ost, shapes, 4, check=psgd_check_factory(st, ost, "topk"))
+    st.clean_error()
+    assert all(float(e.abs().max()) == 0 for e in st.error_dict[0].values())
+
+
+def test_topk_exact(oracle):
+    from conef_amd.hPowerSGD_hook import _topk
+    for numel, ratio, seed in [(11, 0.4, 0), (1025, 0.4, 1), (1_048_576, 0.4, 2), (100_000, 0.01, 3), (7, 2.0, 4)]:
+        g = torch.Generator().manual_seed(seed)
+        x = torch.randn(numel, generator=g)
+        want = x.numpy().copy()
+        oracle.topk_sparsify(want, ratio)
+        xd = x.cuda()
+        _topk(xd, ratio)
+        np.testing.assert_array_equal(to_np(xd), want)
+    # ties, zeros and a threshold of zero
+    x = torch.tensor([1.0, -1.0, 1.0, 0.5, 0.0, 0.0, -1.0, 2.0] * 300)
+    for ratio in (0.25, 0.5, 1.0, 1.9):
+        want = x.numpy().copy()
+        oracle.topk_sparsify(want, ratio)
+        xd = x.cuda()
+        _topk(xd, ratio)
+        np.testing.assert_array_equal(to_np(xd), want)
+
+
+def test_powersgd_state_errors_and_warmup():
+    from conef_amd.powerSGD_hook import PowerSGDState, _should_compress, powerSGD_hook
+    with pytest.raises(ValueError, match="Expect `start_powerSGD_iter` > 1"):
+        PowerSGDState(None, start_powerSGD_iter=1)
+    PowerSGDState(None, start_powerSGD_iter=1, use_error_feedback=False, warm_start=False)
+    assert _should_compress(2, 1024, 2, 2)[0] is False and _should_compress(1024, 1024, 8, 2)[0] is True
+    st = PowerSGDState(None, matrix_approximation_rank=2, start_powerSGD_iter=3)
+    g = torch.randn(64 * 64, device="cuda")
+    ref = g.clone()
+    for _ in range(3):
+        assert torch.equal(powerSGD_hook(st, FakeGradBucket(g, [(64, 64)])).wait(), ref)
+    powerSGD_hook(st, FakeGradBucket(g, [(64, 64)])).wait()
+    assert st.iter == 4 and not torch.equal(g, ref)
+    assert torch.linalg.matrix_rank(g.view(64, 64).cpu().double(), tol=1e-4) <= 2

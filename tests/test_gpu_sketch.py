@@ -1,0 +1,178 @@
+"""GPU parity of the count-sketch kernels against the CPU oracle, through the C-ABI library
+(ctypes) and the product classes that wrap it.  Buckets, signs and query results must be bit
+exact; update results are compared at 1e-5 relative because the reference accumulates with float
+atomics in no fixed order."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from _helpers import assert_close, to_np
+
+pytestmark = pytest.mark.gpu
+
+A, B = 994443, 609478
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from conef_amd import _lib
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return _lib.load()
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.mark.parametrize("d,w", [(1, 1), (700, 65), (5760, 1152), (4096, 409), (200_000, 130_000),
+                                 (1_300_000, 130_000), (100_000, 1), (300_000, 2 ** 30), (1000, 3)])
+def test_device_hash_bit_exact(lib, oracle, d, w):
+    bucket = torch.empty(d, dtype=torch.int32, device="cuda")
+    sign = torch.empty(d, dtype=torch.int32, device="cuda")
+    for (a, b, sa, sb) in [(A, B, A + 2, B + 3), (9171025, 2171464, 9171025 + 8, 2171464 + 7)]:
+        rc = lib.conef_hash_table_i32(bucket.data_ptr(), sign.data_ptr(), d, w, a, b, sa, sb, 0)
+        assert rc == 0
+        torch.cuda.synchronize()
+        ob, osg = oracle.hash_table(d, w, a, b, sa, sb)
+        np.testing.assert_array_equal(to_np(bucket), ob)
+        np.testing.assert_array_equal(to_np(sign), osg)
+
+
+SHAPES = [  # n, d, sketch_size   (row shape: short rows;  tile shape: long rows)
+    (1, 1, 0.5), (3, 17, 0.3), (16, 27, 0.5), (64, 576, 0.2), (7, 650, 0.1), (33, 1024, 0.1),
+    (40, 5760, 0.2), (5, 40_003, 0.1), (5, 100_000, 0.1), (2, 65_537, 0.5), (3, 8191, 1.0),
+]
+
+
+@pytest.mark.parametrize("n,d,ss", SHAPES)
+def test_query_bit_exact(oracle, n, d, ss):
+    from conef_amd.compressors.CountSketch import DenseCS
+    rng = np.random.RandomState(n * 7 + d)
+    cs = DenseCS(n, d, ss)
+    o = oracle.DenseCS(n, d, ss)
+    assert cs.range == o.range
+    o.cs[:] = rng.randn(n, o.range).astype(np.float32)
+    cs.cs.copy_(dev(o.cs))
+    x = (rng.randn(n, d) * 1e-3).astype(np.float32)
+    xd = dev(x)
+    cs.query(xd, 1 - 0.9)
+    o.query(x, 1 - 0.9)
+    np.testing.assert_array_equal(to_np(xd), x)
+
+
+@pytest.mark.parametrize("n,d,ss", SHAPES)
+@pytest.mark.parametrize("beta", [0.9, 1.0])
+def test_update_parity(oracle, n, d, ss, beta):
+    from conef_amd.compressors.CountSketch import DenseCS
+    rng = np.random.RandomState(n * 11 + d)
+    cs = DenseCS(n, d, ss)
+    o = oracle.DenseCS(n, d, ss)
+    for step in range(3):                      # state carried across steps
+        v = (rng.randn(n, d) * 1e-3).astype(np.float32)
+        cs.update(dev(v), beta)
+        o.update(v, beta)
+        assert_close(cs.cs, o.cs, what="sketch after update %d" % step)
+    cs.clean(0.5)
+    o.clean(0.5)
+    assert_close(cs.cs, o.cs, what="clean")
+    cs.clean(0)
+    assert float(cs.cs.abs().max()) == 0.0
+
+
+def test_update_raw_abi_aliasing_rules(lib):
+    n, d, w = 4, 100_000, 10_000           # tile shape: in place is refused
+    assert lib.conef_cs_update_inplace_ok(n, d, w) == 0
+    v = torch.zeros(n, d, device="cuda")
+    cs = torch.zeros(n, w, device="cuda")
+    assert lib.conef_cs_update_f32(v.data_ptr(), cs.data_ptr(), cs.data_ptr(), n, d, w, 0.9, A, B, 0) == -1
+    assert lib.conef_cs_update_inplace_ok(64, 576, 115) == 1
+    assert lib.conef_cs_update_f32(v.data_ptr(), cs.data_ptr(), cs.data_ptr(), n, d, 0, 0.9, A, B, 0) == -1
+    assert lib.conef_cs_query_f32(0, cs.data_ptr(), n, d, w, 0.1, A, B, 0) == -1
+    assert lib.conef_cs_query_f32(v.data_ptr(), cs.data_ptr(), 0, d, w, 0.1, A, B, 0) == 0   # empty input
+
+
+def test_exact_recovery_on_device(oracle):
+    # W >= m with an injective hash sample: unsketch(sketch(v)) == v bit for bit
+    from conef_amd.compressors.CountSketch import DenseCS
+    w = 4096
+    bucket, _ = oracle.hash_table(600, w)
+    d, seen = 0, set()
+    while int(bucket[d]) not in seen:
+        seen.add(int(bucket[d]))
+        d += 1
+    cs = DenseCS(2, d, w / d + 1e-9)
+    assert cs.range == w
+    v = torch.randn(2, d, device="cuda")
+    cs.update(v, 1.0)
+    x = torch.zeros_like(v)
+    cs.query(x, 1.0)
+    assert torch.equal(x, v)
+
+
+@pytest.mark.parametrize("n,d,ss", [(3, 17, 0.3), (64, 576, 0.2), (5, 100_000, 0.1)])
+def test_half_sketch_parity(oracle, n, d, ss):
+    from conef_amd.compressors.halfCountSketch import DenseCS as HalfCS
+    rng = np.random.RandomState(d)
+    cs = HalfCS(n, d, ss)
+    o = oracle.HalfDenseCS(n, d, ss)
+    for step in range(3):
+        v = (rng.randn(n, d) * 1e-2).astype(np.float32)
+        cs.update(dev(v), 0.9)
+        o.update(v, 0.9)
+        got, want = to_np(cs.cs).astype(np.float32), o.cs.astype(np.float32)
+        # one fp16 ulp of slack on top of the fp32 tolerance: a value on a rounding boundary may
+        # land either side when the fp32 accumulation order differs
+        assert np.abs(got - want).max() <= 2 ** -10 * np.abs(want).max()
+        o.cs = to_np(cs.cs).copy()           # keep both on the same fp16 state for the next step
+    x = (rng.randn(n, d) * 1e-2).astype(np.float32)
+    xd = dev(x)
+    cs.query(xd, 0.1)
+    o.query(x, 0.1)
+    np.testing.assert_array_equal(to_np(xd), x)
+    cs.clean(0.5)
+    o.clean(0.5)
+    np.testing.assert_array_equal(to_np(cs.cs), o.cs)
+
+
+@pytest.mark.parametrize("n,d,ss", [(3, 17, 0.3), (64, 576, 0.2), (5, 50_000, 0.1)])
+def test_hash3_parity(oracle, n, d, ss):
+    from conef_amd.compressors.CountSketchHash3 import DenseCSHash3
+    rng = np.random.RandomState(d + 1)
+    cs = DenseCSHash3(n, d, ss)
+    o = oracle.DenseCSHash3(n, d, ss)
+    for step in range(3):
+        v = (rng.randn(n, d) * 1e-3).astype(np.float32)
+        cs.update(dev(v), 0.9)
+        o.update(v, 0.9)
+        for k, (g, want) in enumerate(zip((cs.cs0, cs.cs1, cs.cs2), (o.cs0, o.cs1, o.cs2))):
+            assert_close(g, want, what="cs%d step %d" % (k, step))
+        for g, want in zip((cs.cs0, cs.cs1, cs.cs2), (o.cs0, o.cs1, o.cs2)):
+            want[:] = to_np(g)                 # same state on both sides before the query
+    x = (rng.randn(n, d) * 1e-3).astype(np.float32)
+    xd = dev(x)
+    cs.query(xd, 0.1)
+    o.query(x, 0.1)
+    np.testing.assert_array_equal(to_np(xd), x)
+
+
+def test_state_dict_round_trip():
+    from conef_amd.compressors.CountSketch import DenseCS
+    cs = DenseCS(4, 100, 0.2)
+    cs.update(torch.randn(4, 100, device="cuda"), 0.9)
+    sd = cs.state_dict()
+    other = DenseCS(4, 100, 0.2)
+    other.load_state_dict(sd)
+    assert torch.equal(other.cs, cs.cs)
+    with pytest.raises(ValueError):
+        DenseCS(4, 101, 0.2).load_state_dict(sd)
+
+
+def test_rejects_host_tensors():
+    from conef_amd.compressors.CountSketch import DenseCS
+    cs = DenseCS(2, 10, 0.5)
+    with pytest.raises(ValueError):
+        cs.update(torch.zeros(2, 10), 0.9)
+    with pytest.raises(ValueError):
+        cs.query(torch.zeros(2, 11, device="cuda"), 0.1)
