@@ -6,7 +6,7 @@ contiguous block, with a count-sketch error compressor at 10 % memory, on one fl
 6.5 M elements viewed [5, 1_300_000] (sketch [5, 130_000]); gradients N(0, 1e-6) with 1 % heavy-tail
 entries Laplace(0, 1e-2); synthetic, seeded.
 
-A "step" is one call of the fused C-ABI entry point `conef_randblock_conef_step_f32` on one
+A "step" is one call of the fused C-ABI entry point `conef_randblock_conef_step_planned_f32` on one
 bucket whose gradient already sits in HBM: it adds the unsketched error, extracts the payload
 block, leaves the decompressed gradient in place and writes the new sketch.  Every timed step gets a gradient buffer
 no earlier step has touched and one of a rotating set of sketch states, so nothing it reads is left
@@ -91,15 +91,28 @@ def main():
     starts = [int(rng.choice(L)) for _ in range(total_steps + 64)]
     stream = torch.cuda.current_stream().cuda_stream
 
+    plans = [cs.plan() for cs in sketches]
+    planned = plans[0] is not None
+    entry = "conef_randblock_conef_step_planned_f32" if planned else "conef_randblock_conef_step_f32"
+
     def one_step(i, g, b):
         cs = sketches[b]
-        out = cs.next_buffer()
-        rc = lib.conef_randblock_conef_step_f32(g.data_ptr(), cs.cs.data_ptr(), out.data_ptr(),
-                                                payloads[b].data_ptr(), N_ROWS, N_COLS, W, starts[i], block,
-                                                alpha, BETA, cs.a, cs.b, stream)
+        if planned:
+            pl = plans[b]
+            out = cs.spare_buffer()
+            rc = lib.conef_randblock_conef_step_planned_f32(
+                g.data_ptr(), cs.cs.data_ptr(), out.data_ptr(), payloads[b].data_ptr(), pl.host_ptr,
+                pl.device.data_ptr(), pl.workspace.data_ptr(), N_ROWS, N_COLS, W, starts[i], block, alpha, BETA,
+                cs.a, cs.b, stream)
+            cs.commit(out)
+        else:
+            out = cs.next_buffer()
+            rc = lib.conef_randblock_conef_step_f32(g.data_ptr(), cs.cs.data_ptr(), out.data_ptr(),
+                                                    payloads[b].data_ptr(), N_ROWS, N_COLS, W, starts[i], block,
+                                                    alpha, BETA, cs.a, cs.b, stream)
+            cs.commit(out)
         if rc != 0:
-            raise RuntimeError("conef_randblock_conef_step_f32 returned %d" % rc)
-        cs.commit(out)
+            raise RuntimeError("%s returned %d" % (entry, rc))
 
     torch.cuda.synchronize()
     for i in range(args.warmup):
@@ -163,7 +176,7 @@ def main():
         "config": {
             "workload": "RandomBlock 10% + count-sketch ConEF 10%, flat fp32 bucket [5,1300000] (26 MB), "
                         "sketch [5,130000], block 650000, beta 0.9",
-            "entry_point": "conef_randblock_conef_step_f32",
+            "entry_point": entry,
             "gradient_buffers": n_grads,
             "sketch_states_rotated": N_BUCKETS,
             "working_set_mb": round((n_grads * 4 * L + N_BUCKETS * (4 * block + 8 * N_ROWS * W)) / 1e6, 1),

@@ -147,12 +147,7 @@ def RandomBlock_hook(state: RandomBlockState, bucket) -> torch.futures.Future:
         payload = payload_all[idx: idx + block]
         n, m = matrix.shape
         if state.use_error_compression:
-            out = error.next_buffer()
-            rc = lib.conef_randblock_conef_step_f32(
-                matrix.data_ptr(), error.cs.data_ptr(), out.data_ptr(), payload.data_ptr(), n, m, error.range,
-                start, block, float(alpha), float(state.beta), error.a, error.b, stream)
-            _lib.check(rc, "conef_randblock_conef_step_f32")
-            error.commit(out)
+            error.randblock_step(matrix, payload, start, block, alpha, state.beta)
         else:
             rc = lib.conef_randblock_ef_step_f32(matrix.data_ptr(), error.data_ptr(), payload.data_ptr(), numel,
                                                  start, block, stream)

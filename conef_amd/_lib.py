@@ -20,7 +20,7 @@ _I32 = ctypes.c_int32
 _F32 = ctypes.c_float
 
 # name -> argtypes; every function returns int (0 = ok, >0 hipError_t, -1 invalid argument),
-# except conef_topk_workspace_bytes which returns a byte count as int64
+# except the *_bytes functions, which return a byte count as int64
 SIGNATURES = {
     "conef_version": [],
     "conef_hash_table_i32": [_P, _P, _I64, _I32, _I32, _I32, _I32, _I32, _P],
@@ -50,9 +50,17 @@ SIGNATURES = {
     "conef_psgd_pqt_conef_f32": [_P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P],
     "conef_gram_schmidt_f32": [_P, _I64, _I32, _F32, _P],
     "conef_ef_passthrough_f32": [_P, _P, _I64, _P],
+    "conef_plan_bytes": [_I64, _I64, _I32, _I32, _I32],
+    "conef_plan_build_host": [_P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32],
+    "conef_plan_workspace_bytes": [_P],
+    "conef_cs_update_planned_f32": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],
+    "conef_randblock_conef_step_planned_f32": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I32, _I64, _I64, _F32, _F32,
+                                               _I32, _I32, _P],
     "conef_topk_workspace_bytes": [_I64],
     "conef_topk_sparsify_f32": [_P, _I64, _I64, _P, _I64, _P],
 }
+
+_RETURNS_I64 = ("conef_topk_workspace_bytes", "conef_plan_bytes", "conef_plan_workspace_bytes")
 
 _handle = None
 
@@ -74,7 +82,7 @@ def load():
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)      # AttributeError here means header and library disagree
         fn.argtypes = argtypes
-        fn.restype = _I64 if name == "conef_topk_workspace_bytes" else ctypes.c_int
+        fn.restype = _I64 if name in _RETURNS_I64 else ctypes.c_int
     _handle = lib
     return lib
 

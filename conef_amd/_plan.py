@@ -1,0 +1,48 @@
+"""Host/device holder of an accumulation plan for sketches whose rows do not fit LDS.
+
+The plan (built once per sketch by ``conef_plan_build_host``) lists where every column's record
+goes, so that the count-sketch update of a long row runs as two streaming passes without
+atomics and adds each bucket's terms in ascending column order.
+"""
+import numpy as np
+import torch
+
+from . import _lib
+
+
+class SketchPlan:
+    """plan bytes on the host (read for launch geometry), the same bytes on the device, and the
+    staging buffer the two passes hand records through."""
+
+    def __init__(self, n, d, w, a, b, device, chunk_cols=0, bin_buckets=0):
+        lib = _lib.load()
+        nbytes = lib.conef_plan_bytes(n, d, w, chunk_cols, bin_buckets)
+        if nbytes <= 0:
+            raise ValueError("no plan for shape n=%d d=%d w=%d" % (n, d, w))
+        self.host = np.zeros(nbytes, dtype=np.uint8)
+        rc = lib.conef_plan_build_host(self.host.ctypes.data, nbytes, n, d, w, a, b, chunk_cols, bin_buckets)
+        _lib.check(rc, "conef_plan_build_host")
+        self.device = torch.from_numpy(self.host).to(device)
+        ws = lib.conef_plan_workspace_bytes(self.host.ctypes.data)
+        self.workspace = torch.empty(ws, dtype=torch.uint8, device=device)
+        self.key = (n, d, w, a, b)
+
+    @property
+    def host_ptr(self):
+        return self.host.ctypes.data
+
+    @staticmethod
+    def applicable(n, d, w):
+        lib = _lib.load()
+        return n <= 8 and not lib.conef_cs_update_inplace_ok(n, d, w)
+
+    def header(self):
+        """Decoded header fields (for tests and diagnostics)."""
+        h = self.host
+        i32 = h[:128].view(np.int32)
+        i64 = h[:128].view(np.int64)
+        return {"n": int(i64[1]), "d": int(i64[2]), "w": int(i32[6]), "a": int(i32[7]), "b": int(i32[8]),
+                "chunk_cols": int(i32[9]), "nchunks": int(i32[10]), "bin_buckets": int(i32[11]),
+                "nbins": int(i32[12]), "max_bin_records": int(i32[13]), "off_pos": int(i64[7]),
+                "off_seg": int(i64[8]), "off_csr": int(i64[9]), "off_ent": int(i64[10]),
+                "total_bytes": int(i64[11]), "workspace_bytes": int(i64[12])}

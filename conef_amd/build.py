@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBPATH = os.path.join(LIBDIR, "libconef_hip.so")
 
-SOURCES = ["conef_sketch.hip", "conef_randblock.hip", "conef_psgd.hip", "conef_topk.hip"]
+SOURCES = ["conef_sketch.hip", "conef_randblock.hip", "conef_psgd.hip", "conef_topk.hip", "conef_plan.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -4,13 +4,17 @@ Same constructor, attributes (N, D, blk_size, range, cs, a, b) and methods as th
 Differences a maintainer should know about:
   * the kernels are precompiled gfx950 code reached through libconef_hip.so, not CuPy/NVRTC;
   * alpha, beta, a, b travel by value, so ``a``/``b`` are Python ints, not 1-element device tensors;
-  * when a sketch row does not fit LDS (W above a few thousand) ``update`` writes into a second
-    buffer and ``self.cs`` is rebound to it, so do not keep a stale reference to ``cs`` across updates;
+  * when a sketch row does not fit LDS (W above a few thousand) and the tensor has at most 8 rows,
+    updates run on a precomputed plan (two streaming passes, no atomics, deterministic); with more
+    rows ``update`` writes into a second buffer and ``self.cs`` is rebound to it;
   * ``state_dict``/``load_state_dict`` round-trip (the reference's __setstate__ loses a, b).
 """
+import os
+
 import torch
 
 from .. import _lib
+from .._plan import SketchPlan
 
 HASH_A = 994443   # CountSketch.py:112
 HASH_B = 609478   # CountSketch.py:113
@@ -30,6 +34,7 @@ class DenseCS:
         self._lib = _lib.load()
         self._inplace = bool(self._lib.conef_cs_update_inplace_ok(self.N, self.D, self.range))
         self._spare = None
+        self._plan = None
 
     # -- persistence ---------------------------------------------------------------------------
     def state_dict(self):
@@ -54,6 +59,7 @@ class DenseCS:
         self._lib = _lib.load()
         self._inplace = bool(self._lib.conef_cs_update_inplace_ok(self.N, self.D, self.range))
         self._spare = None
+        self._plan = None
 
     # -- kernels -------------------------------------------------------------------------------
     def _check(self, t, name):
@@ -64,13 +70,28 @@ class DenseCS:
         if t.device != self.cs.device:
             raise ValueError("%s is on %s, the sketch on %s" % (name, t.device, self.cs.device))
 
-    def next_buffer(self):
-        """Buffer the next update writes into: ``cs`` itself when a row fits LDS, else a spare."""
-        if self._inplace:
-            return self.cs
+    def plan(self):
+        """Accumulation plan for long rows (built on first use), or None when a row fits LDS or the
+        tensor has more than 8 rows.  CONEF_PLAN_CHUNK / CONEF_PLAN_BIN override the tile sizes and
+        CONEF_PLAN=0 disables the planned path (the kernels then accumulate with float atomics)."""
+        if self._plan is None and not self._inplace and os.environ.get("CONEF_PLAN", "1") != "0":
+            if SketchPlan.applicable(self.N, self.D, self.range):
+                self._plan = SketchPlan(self.N, self.D, self.range, self.a, self.b, self.cs.device,
+                                        int(os.environ.get("CONEF_PLAN_CHUNK", "0")),
+                                        int(os.environ.get("CONEF_PLAN_BIN", "0")))
+        if self._plan is not None and self._plan.key != (self.N, self.D, self.range, self.a, self.b):
+            self._plan = None
+            return self.plan()
+        return self._plan
+
+    def spare_buffer(self):
         if self._spare is None:
             self._spare = torch.empty_like(self.cs)
         return self._spare
+
+    def next_buffer(self):
+        """Buffer the next update writes into: ``cs`` itself when a row fits LDS, else a spare."""
+        return self.cs if self._inplace else self.spare_buffer()
 
     def commit(self, written):
         """Makes the buffer an update wrote into the current sketch."""
@@ -80,10 +101,41 @@ class DenseCS:
     def update(self, vec, beta):
         """cs <- cs + sketch-accumulate(vec) with the reference's per-element decay (CountSketch.py:27-67)."""
         self._check(vec, "vec")
+        plan = self.plan()
+        if plan is not None:
+            rc = self._lib.conef_cs_update_planned_f32(vec.data_ptr(), self.cs.data_ptr(), self.cs.data_ptr(),
+                                                       plan.host_ptr, plan.device.data_ptr(),
+                                                       plan.workspace.data_ptr(), self.N, self.D, self.range,
+                                                       float(beta), self.a, self.b, _lib.stream_ptr(vec))
+            _lib.check(rc, "conef_cs_update_planned_f32")
+            return
         out = self.next_buffer()
         rc = self._lib.conef_cs_update_f32(vec.data_ptr(), self.cs.data_ptr(), out.data_ptr(), self.N, self.D,
                                            self.range, float(beta), self.a, self.b, _lib.stream_ptr(vec))
         _lib.check(rc, "conef_cs_update_f32")
+        self.commit(out)
+
+    def randblock_step(self, x, payload, start, block, alpha, beta):
+        """One fused RandomBlock + ConEF step on the [N,D] gradient ``x`` (in place): adds the
+        unsketched error, moves the wrap-around block [start, start+block) to ``payload``, leaves
+        zeros + block in ``x`` and sketches the rest."""
+        self._check(x, "x")
+        stream = _lib.stream_ptr(x)
+        plan = self.plan()
+        if plan is not None:
+            out = self.spare_buffer()      # the planned step reads the old sketch while it writes the new one
+            rc = self._lib.conef_randblock_conef_step_planned_f32(
+                x.data_ptr(), self.cs.data_ptr(), out.data_ptr(), payload.data_ptr(), plan.host_ptr,
+                plan.device.data_ptr(), plan.workspace.data_ptr(), self.N, self.D, self.range, start, block,
+                float(alpha), float(beta), self.a, self.b, stream)
+            _lib.check(rc, "conef_randblock_conef_step_planned_f32")
+            self.commit(out)
+            return
+        out = self.next_buffer()
+        rc = self._lib.conef_randblock_conef_step_f32(
+            x.data_ptr(), self.cs.data_ptr(), out.data_ptr(), payload.data_ptr(), self.N, self.D, self.range,
+            start, block, float(alpha), float(beta), self.a, self.b, stream)
+        _lib.check(rc, "conef_randblock_conef_step_f32")
         self.commit(out)
 
     def query(self, grad_plus_error, alpha):

@@ -1,0 +1,75 @@
+// Entry points of the planned (atomic-free, deterministic) sketch accumulation for long rows;
+// the scheme is described at the top of conef_plan.h.
+#include "conef_plan.h"
+
+namespace {
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+}  // namespace
+
+extern "C" {
+
+// Bytes of a plan for an [n,d] tensor sketched at width w; 0 when the planned path does not apply
+// (more than 8 rows), -1 on invalid arguments.  chunk_cols / bin_buckets = 0 pick defaults.
+int64_t conef_plan_bytes(int64_t n, int64_t d, int32_t w, int32_t chunk_cols, int32_t bin_buckets)
+{
+    if (n < 1 || d < 1 || w < 1 || w > (1 << 30) || d > 0x7fffffffLL) return -1;
+    if (n > kConefPlanMaxRows) return 0;
+    ConefPlanHeader h;
+    if (!conef_plan_shape(n, d, w, chunk_cols, bin_buckets, &h)) return -1;
+    return h.total_bytes;
+}
+
+// Builds the plan into HOST memory.  The caller copies the same bytes to the device and passes
+// both copies to the *_planned entry points (the host copy is read for launch geometry only).
+int conef_plan_build_host(void* plan_host, int64_t plan_bytes, int64_t n, int64_t d, int32_t w, int32_t a, int32_t b,
+                          int32_t chunk_cols, int32_t bin_buckets)
+{
+    ConefPlanHeader h;
+    if (!plan_host || !conef_plan_shape(n, d, w, chunk_cols, bin_buckets, &h)) return CONEF_ERR_INVALID;
+    if (plan_bytes < h.total_bytes) return CONEF_ERR_INVALID;
+    if (!conef_plan_fill(plan_host, h, a, b)) return CONEF_ERR_INVALID;
+    const ConefPlanHeader* built = (const ConefPlanHeader*)plan_host;
+    if (conef_binned_lds_b(built, (int)n) > 160 * 1024) return CONEF_ERR_INVALID;
+    return CONEF_OK;
+}
+
+int64_t conef_plan_workspace_bytes(const void* plan_host)
+{
+    const ConefPlanHeader* h = (const ConefPlanHeader*)plan_host;
+    if (!h || h->magic != kConefPlanMagic) return -1;
+    return h->workspace_bytes;
+}
+
+int conef_cs_update_planned_f32(const float* vec, const float* cs_in, float* cs_out, const void* plan_host,
+                                const void* plan_dev, void* workspace, int64_t n, int64_t d, int32_t w, float beta,
+                                int32_t a, int32_t b, void* stream)
+{
+    const ConefPlanHeader* hp = (const ConefPlanHeader*)plan_host;
+    if (!conef_plan_matches(hp, n, d, w, a, b) || !plan_dev || !workspace || !vec || !cs_in || !cs_out)
+        return CONEF_ERR_INVALID;
+    ConefStageVec stage = {vec, d};
+    ConefBlockWork none = {};
+    return conef_launch_binned(stage, hp, plan_dev, (float*)workspace, cs_in, cs_out, 0.f, beta, aligned16(vec), none,
+                               (hipStream_t)stream);
+}
+
+int conef_randblock_conef_step_planned_f32(float* x, const float* cs_in, float* cs_out, float* payload,
+                                           const void* plan_host, const void* plan_dev, void* workspace, int64_t n,
+                                           int64_t m, int32_t w, int64_t start, int64_t block, float alpha,
+                                           float beta, int32_t a, int32_t b, void* stream)
+{
+    const ConefPlanHeader* hp = (const ConefPlanHeader*)plan_host;
+    if (!conef_plan_matches(hp, n, m, w, a, b) || !plan_dev || !workspace || !x || !cs_in || !cs_out || !payload)
+        return CONEF_ERR_INVALID;
+    int64_t numel = n * m;
+    if (!(start >= 0 && start < numel && block >= 1 && block <= numel)) return CONEF_ERR_INVALID;
+    if (cs_in == cs_out) return CONEF_ERR_INVALID;   // the block is finished while buckets are being rewritten
+    ConefBlock blk = conef_make_block(numel, start, block);
+    ConefSeeds hs = {a, b, a + 2, b + 3};
+    ConefStageRandBlock stage = {x, m, blk};
+    ConefBlockWork bw = {x, payload, numel, m, block, blk, conef_make_mod(w), hs, alpha};
+    return conef_launch_binned(stage, hp, plan_dev, (float*)workspace, cs_in, cs_out, alpha, beta, aligned16(x), bw,
+                               (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -9,8 +9,8 @@
  *   - every pointer is a DEVICE pointer into memory the caller owns and keeps alive until the
  *     stream has run the call (the one exception, conef_hash_table_host_i32, takes host memory);
  *   - `stream` is a hipStream_t (NULL = the default stream); every call is asynchronous on it,
- *     never synchronises the host, never allocates or frees, keeps no global or thread-local
- *     state and may be called from any thread;
+ *     never synchronises the host, never allocates or frees device memory, keeps no global or
+ *     thread-local state and may be called from any thread;
  *   - scalars (alpha, beta, hash seeds) travel by value - the reference passes them as pointers
  *     to 1-element device tensors it allocates per call (CountSketch.py:144,167);
  *   - matrices are dense row-major fp32; a sketch is [n, w] row-major, fp32 unless the name says f16;
@@ -95,6 +95,32 @@ int conef_cs3_query_f32(float* x, const float* cs0, const float* cs1, const floa
 int conef_cs3_update_f32(const float* vec, const float* in0, const float* in1, const float* in2, float* out0,
                          float* out1, float* out2, int64_t n, int64_t d, int32_t w, float beta, void* stream);
 
+/* ------------------------------------------- planned accumulation for long rows -------- */
+/* When a sketch row does not fit LDS (W above a few thousand) the update has no locality and
+ * float atomics on global memory are far too slow.  The hash is a fixed function of (column, w,
+ * a, b), so a plan built once per sketch turns the update into two streaming passes through a
+ * staging buffer, without atomics, adding each bucket's terms in ascending column order (the
+ * CPU restatement's order, so results match it bit for bit).  Applies to tensors of <= 8 rows.
+ * No counterpart in the reference, whose kernel cannot launch at all for such widths (it asks
+ * for 8*W bytes of shared memory, CountSketch.py:158). */
+
+/* Size in bytes of the plan for an [n,d] tensor at width w; 0 = not applicable (n > 8),
+ * -1 = invalid.  chunk_cols / bin_buckets tune the tile sizes, 0 = default.  Host function. */
+int64_t conef_plan_bytes(int64_t n, int64_t d, int32_t w, int32_t chunk_cols, int32_t bin_buckets);
+/* Builds the plan into HOST memory (plan_bytes >= conef_plan_bytes(...)).  The caller copies the
+ * same bytes to the device and hands both copies to the *_planned entry points; the host copy
+ * is only read for the launch geometry.  Host function, O(d). */
+int conef_plan_build_host(void* plan_host, int64_t plan_bytes, int64_t n, int64_t d, int32_t w, int32_t a,
+                          int32_t b, int32_t chunk_cols, int32_t bin_buckets);
+/* Bytes of device staging memory the planned entry points need (n*d floats, rounded up). */
+int64_t conef_plan_workspace_bytes(const void* plan_host);
+
+/* conef_cs_update_f32 on a plan.  cs_out may be the same buffer as cs_in.  Calls that share a
+ * workspace must be ordered on one stream. */
+int conef_cs_update_planned_f32(const float* vec, const float* cs_in, float* cs_out, const void* plan_host,
+                                const void* plan_dev, void* workspace, int64_t n, int64_t d, int32_t w, float beta,
+                                int32_t a, int32_t b, void* stream);
+
 /* ------------------------------------------------------------ random block ------------- */
 /* The block is the wrap-around range [start, start+block) of the flat tensor: [start, end) with
  * end = min(start+block, numel), then [0, block-(end-start)).  0 <= start < numel, 1 <= block <= numel. */
@@ -108,6 +134,13 @@ int conef_cs3_update_f32(const float* vec, const float* in0, const float* in1, c
 int conef_randblock_conef_step_f32(float* x, const float* cs_in, float* cs_out, float* payload, int64_t n,
                                    int64_t m, int32_t w, int64_t start, int64_t block, float alpha, float beta,
                                    int32_t a, int32_t b, void* stream);
+
+/* conef_randblock_conef_step_f32 on a plan (see above).  cs_out must NOT be cs_in here (-1): the
+ * selected block is finished from the old sketch while the new one is being written. */
+int conef_randblock_conef_step_planned_f32(float* x, const float* cs_in, float* cs_out, float* payload,
+                                           const void* plan_host, const void* plan_dev, void* workspace, int64_t n,
+                                           int64_t m, int32_t w, int64_t start, int64_t block, float alpha,
+                                           float beta, int32_t a, int32_t b, void* stream);
 
 /* Same step with a dense error tensor: xq = x + err; payload = xq[block]; x = xq on the block,
  * 0 elsewhere; err = 0 on the block, xq elsewhere.

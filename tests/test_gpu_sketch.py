@@ -176,3 +176,61 @@ def test_rejects_host_tensors():
         cs.update(torch.zeros(2, 10), 0.9)
     with pytest.raises(ValueError):
         cs.query(torch.zeros(2, 11, device="cuda"), 0.1)
+
+
+# ---- long rows: the planned (atomic-free) path is deterministic and follows the oracle's order ----
+
+PLANNED_SHAPES = [(5, 40_003, 0.1), (5, 100_000, 0.1), (2, 65_537, 0.5), (3, 8191, 1.0), (1, 300_001, 0.05),
+                  (8, 20_000, 0.9)]
+
+
+@pytest.mark.parametrize("n,d,ss", PLANNED_SHAPES)
+def test_planned_update_bit_exact(oracle, n, d, ss):
+    from conef_amd.compressors.CountSketch import DenseCS
+    rng = np.random.RandomState(d)
+    cs = DenseCS(n, d, ss)
+    assert cs.plan() is not None
+    o = oracle.DenseCS(n, d, ss)
+    for step in range(3):
+        v = (rng.randn(n, d) * 1e-3).astype(np.float32)
+        cs.update(dev(v), 0.9)
+        o.update(v, 0.9)
+        np.testing.assert_array_equal(to_np(cs.cs), o.cs)
+
+
+@pytest.mark.parametrize("chunk,tbin", [(1024, 64), (2048, 512), (8192, 256), (4096, 128)])
+def test_planned_update_any_tiling(oracle, monkeypatch, chunk, tbin):
+    from conef_amd.compressors.CountSketch import DenseCS
+    monkeypatch.setenv("CONEF_PLAN_CHUNK", str(chunk))
+    monkeypatch.setenv("CONEF_PLAN_BIN", str(tbin))
+    n, d, ss = 5, 130_001, 0.1
+    cs = DenseCS(n, d, ss)
+    h = cs.plan().header()
+    assert (h["chunk_cols"], h["bin_buckets"]) == (chunk, tbin)
+    o = oracle.DenseCS(n, d, ss)
+    v = (np.random.RandomState(1).randn(n, d) * 1e-3).astype(np.float32)
+    for _ in range(2):
+        cs.update(dev(v), 0.9)
+        o.update(v, 0.9)
+    np.testing.assert_array_equal(to_np(cs.cs), o.cs)
+
+
+def test_atomic_fallback_still_matches(oracle, monkeypatch):
+    from conef_amd.compressors.CountSketch import DenseCS
+    monkeypatch.setenv("CONEF_PLAN", "0")
+    n, d, ss = 5, 100_000, 0.1
+    cs = DenseCS(n, d, ss)
+    assert cs.plan() is None
+    o = oracle.DenseCS(n, d, ss)
+    v = (np.random.RandomState(2).randn(n, d) * 1e-3).astype(np.float32)
+    cs.update(dev(v), 0.9)
+    o.update(v, 0.9)
+    assert_close(cs.cs, o.cs, what="atomic path")
+    big = DenseCS(12, 100_000, 0.1)          # more than 8 rows: no plan, atomics
+    monkeypatch.delenv("CONEF_PLAN")
+    assert big.plan() is None
+    ob = oracle.DenseCS(12, 100_000, 0.1)
+    v = (np.random.RandomState(3).randn(12, 100_000) * 1e-3).astype(np.float32)
+    big.update(dev(v), 0.9)
+    ob.update(v, 0.9)
+    assert_close(big.cs, ob.cs, what="atomic path, 12 rows")

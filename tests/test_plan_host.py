@@ -1,0 +1,102 @@
+"""CPU-only check of the accumulation plan the long-row sketch kernels run on.
+
+The two GPU passes are replayed here in numpy, reading only the plan's tables: pass A permutes
+each chunk's records into its image, pass B collects a bin's segments and adds every bucket's
+terms in the order the plan lists them.  If the tables are right this reproduces the oracle's
+update bit for bit (same terms, same ascending-column order)."""
+import numpy as np
+import pytest
+
+A, B = 994443, 609478
+
+
+def build_plan(n, d, w, chunk=0, tbin=0):
+    from conef_amd import _lib
+    lib = _lib.load()
+    nb = lib.conef_plan_bytes(n, d, w, chunk, tbin)
+    assert nb > 0
+    buf = np.zeros(nb, np.uint8)
+    assert lib.conef_plan_build_host(buf.ctypes.data, nb, n, d, w, A, B, chunk, tbin) == 0
+    i32, i64 = buf[:128].view(np.int32), buf[:128].view(np.int64)
+    h = {"C": int(i32[9]), "nchunks": int(i32[10]), "T": int(i32[11]), "nbins": int(i32[12]),
+         "maxrec": int(i32[13])}
+    h["pos"] = buf[int(i64[7]):int(i64[7]) + 2 * d].view(np.uint16)
+    h["seg"] = buf[int(i64[8]):int(i64[8]) + 4 * h["nbins"] * (h["nchunks"] + 1)].view(np.uint32).reshape(
+        h["nbins"], h["nchunks"] + 1)
+    h["csr"] = buf[int(i64[9]):int(i64[9]) + 4 * (w + 1)].view(np.uint32)
+    h["ent"] = buf[int(i64[10]):int(i64[10]) + 2 * d].view(np.uint16)
+    assert int(i64[12]) >= 4 * n * d
+    return h
+
+
+def replay(h, vec, cs, beta, oracle):
+    n, d = vec.shape
+    w = cs.shape[1]
+    C, T = h["C"], h["T"]
+    staging = np.full(n * d, np.nan, np.float32)
+    for c in range(h["nchunks"]):                                   # pass A
+        c0, c1 = c * C, min(d, (c + 1) * C)
+        img = np.full((c1 - c0, n), np.nan, np.float32)
+        p = h["pos"][c0:c1].astype(np.int64)
+        assert sorted(p.tolist()) == list(range(c1 - c0))           # a permutation of the chunk
+        img[p, :] = vec[:, c0:c1].T
+        staging[c0 * n:c1 * n] = img.reshape(-1)
+    out = cs.copy()
+    omb = 1.0 - float(np.float32(beta))
+    for bn in range(h["nbins"]):                                    # pass B
+        seg = h["seg"][bn]
+        total = int(seg[-1] >> 16)
+        assert total <= h["maxrec"]
+        img = np.empty((total, n), np.float32)
+        for c in range(h["nchunks"]):
+            start, off = int(seg[c] & 0xffff), int(seg[c] >> 16)
+            ln = int(seg[c + 1] >> 16) - off
+            src = (c * C + start) * n
+            img[off:off + ln] = staging[src:src + ln * n].reshape(ln, n)
+        for j in range(bn * T, min(w, (bn + 1) * T)):
+            for e in range(int(h["csr"][j]), int(h["csr"][j + 1])):
+                en = int(h["ent"][e])
+                sign = 1.0 if en >> 15 else -1.0
+                for r in range(n):
+                    v = float(img[en & 0x7fff, r])
+                    term = np.float32(sign * v - omb * float(cs[r, j]))
+                    out[r, j] = np.float32(out[r, j] + term)
+    assert not np.isnan(out).any()
+    return out
+
+
+@pytest.mark.parametrize("n,d,w,chunk,tbin", [(5, 9000, 900, 1024, 64), (1, 5000, 5000, 2048, 128),
+                                              (8, 3001, 77, 1024, 64), (3, 12345, 4000, 0, 0)])
+def test_plan_replay_matches_oracle_bit_for_bit(oracle, n, d, w, chunk, tbin):
+    rng = np.random.RandomState(d)
+    h = build_plan(n, d, w, chunk, tbin)
+    vec = rng.randn(n, d).astype(np.float32)
+    cs0 = rng.randn(n, w).astype(np.float32)
+    got = replay(h, vec, cs0, 0.9, oracle)
+    want = cs0.copy()
+    oracle.cs_update(vec, want, 0.9)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_plan_tables_are_consistent(oracle):
+    n, d, w = 5, 50_000, 5_000
+    h = build_plan(n, d, w)
+    bucket, sign = oracle.hash_table(d, w)
+    assert h["csr"][0] == 0 and h["csr"][-1] == d
+    np.testing.assert_array_equal(np.diff(h["csr"].astype(np.int64)), np.bincount(bucket, minlength=w))
+    bins = bucket // h["T"]
+    np.testing.assert_array_equal(h["seg"][:, -1] >> 16, np.bincount(bins, minlength=h["nbins"]))
+    assert h["maxrec"] == np.bincount(bins, minlength=h["nbins"]).max()
+    # entries of a bucket carry that bucket's signs, in ascending column order
+    order = np.lexsort((np.arange(d), bucket))
+    np.testing.assert_array_equal(h["ent"] >> 15, (sign[order] > 0).astype(np.uint16))
+
+
+def test_plan_argument_checks():
+    from conef_amd import _lib
+    lib = _lib.load()
+    assert lib.conef_plan_bytes(9, 1000, 100, 0, 0) == 0          # more than 8 rows: not applicable
+    assert lib.conef_plan_bytes(0, 1000, 100, 0, 0) == -1
+    buf = np.zeros(64, np.uint8)
+    assert lib.conef_plan_build_host(buf.ctypes.data, 64, 5, 1000, 100, A, B, 0, 0) == -1   # buffer too small
+    assert lib.conef_plan_workspace_bytes(buf.ctypes.data) == -1                            # not a plan
