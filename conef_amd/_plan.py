@@ -44,5 +44,5 @@ class SketchPlan:
         return {"n": int(i64[1]), "d": int(i64[2]), "w": int(i32[6]), "a": int(i32[7]), "b": int(i32[8]),
                 "chunk_cols": int(i32[9]), "nchunks": int(i32[10]), "bin_buckets": int(i32[11]),
                 "nbins": int(i32[12]), "max_bin_records": int(i32[13]), "off_pos": int(i64[7]),
-                "off_seg": int(i64[8]), "off_csr": int(i64[9]), "off_ent": int(i64[10]),
-                "total_bytes": int(i64[11]), "workspace_bytes": int(i64[12])}
+                "off_seg": int(i64[8]), "off_csr": int(i64[9]), "off_ent": int(i64[10]), "off_pk": int(i64[11]),
+                "total_bytes": int(i64[12]), "workspace_bytes": int(i64[13])}

@@ -58,9 +58,10 @@ struct ConefPlanHeader {
                                // entry [nchunks] holds the bin's record count in the high half
     int64_t off_csr;           // uint32[w+1]: first entry of bucket j
     int64_t off_ent;           // uint16[d]: (slot inside bin image) | (sign bit << 15), buckets ascending, columns ascending
+    int64_t off_pk;            // uint32[d]: bucket | (sign bit << 31) of every column, for the column-order work
     int64_t total_bytes;
     int64_t workspace_bytes;   // staging buffer: n * d floats, rounded up
-    int64_t reserved[4];
+    int64_t reserved[3];
 };
 
 inline int64_t conef_align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
@@ -71,7 +72,7 @@ inline bool conef_plan_shape(int64_t n, int64_t d, int32_t w, int32_t hint_chunk
 {
     if (n < 1 || n > kConefPlanMaxRows || d < 1 || d > 0x7fffffffLL || w < 1 || w > (1 << 30)) return false;
     memset(h, 0, sizeof(*h));
-    int64_t c = hint_chunk > 0 ? hint_chunk : (80 * 1024) / (4 * n);
+    int64_t c = hint_chunk > 0 ? hint_chunk : (100 * 1024) / (4 * n);   // a 100 KB chunk image: one workgroup per CU
     if (c > 16384) c = 16384;
     c = c / 1024 * 1024;
     if (c < 1024) c = 1024;
@@ -79,8 +80,9 @@ inline bool conef_plan_shape(int64_t n, int64_t d, int32_t w, int32_t hint_chunk
     if (hint_bin > 0) {
         t = hint_bin;
     } else {
-        // aim at a bin image of about 48 KB: records = 48K / (4n), buckets = records * w / d
-        double records = 48.0 * 1024 / (4.0 * n);
+        // aim at a bin image of about 52 KB (two workgroups per CU): records = 52K / (4n),
+        // buckets = records * w / d
+        double records = 52.0 * 1024 / (4.0 * n);
         t = (int64_t)(records * (double)w / (double)d);
         t = t / 64 * 64;
     }
@@ -104,6 +106,8 @@ inline bool conef_plan_shape(int64_t n, int64_t d, int32_t w, int32_t hint_chunk
     off += conef_align256(4 * ((int64_t)w + 1));
     h->off_ent = off;
     off += conef_align256(2 * d);
+    h->off_pk = off;
+    off += conef_align256(4 * d);
     h->total_bytes = off;
     h->workspace_bytes = conef_align256(4 * n * d);
     return true;
@@ -124,7 +128,7 @@ inline bool conef_plan_fill(void* buf, const ConefPlanHeader& shape, int32_t a, 
     uint32_t* csr = (uint32_t*)(base + h.off_csr);
     uint16_t* ent = (uint16_t*)(base + h.off_ent);
     ConefMod mod = conef_make_mod(w);
-    std::vector<uint32_t> packed((size_t)d);
+    uint32_t* packed = (uint32_t*)(base + h.off_pk);
     for (int64_t i = 0; i < d; ++i) packed[(size_t)i] = conef_bucket_sign((int32_t)i, mod, a, b, a + 2, b + 3);
 
     // pass-A side: inside every chunk, records grouped by bin (stable in column order)
@@ -180,6 +184,7 @@ struct ConefPlanView {
     const uint32_t* seg;
     const uint32_t* csr;
     const uint16_t* ent;
+    const uint32_t* pk;
     int32_t chunk_cols, nchunks, bin_buckets, nbins;
     int32_t flags;   // bit 0: XCD-major work mapping, bit 1: streaming (nontemporal) stores
 };
@@ -202,6 +207,7 @@ inline ConefPlanView conef_plan_view(const ConefPlanHeader* host, const void* de
     v.seg = (const uint32_t*)(b + host->off_seg);
     v.csr = (const uint32_t*)(b + host->off_csr);
     v.ent = (const uint16_t*)(b + host->off_ent);
+    v.pk = (const uint32_t*)(b + host->off_pk);
     v.chunk_cols = host->chunk_cols;
     v.nchunks = host->nchunks;
     v.bin_buckets = host->bin_buckets;
@@ -377,17 +383,21 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
             int n = bw.block - p0 < 4 ? (int)(bw.block - p0) : 4;
             int64_t f = bw.blk.start + p0;
             if (f >= bw.numel) f -= bw.numel;
-            int64_t r = f / bw.m;
-            int64_t col = f - r * bw.m;
+            int64_t r = 0, col = f;                 // at most 8 rows: no 64-bit division needed
+            while (col >= bw.m) {
+                col -= bw.m;
+                ++r;
+            }
             float* px[4];
             float g[4], cell[4];
             uint32_t pk[4];
+            int64_t rr[4];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 px[k] = bw.x + r * bw.m + col;
-                pk[k] = conef_bucket_sign((int32_t)col, bw.mod, bw.hs.a, bw.hs.b, bw.hs.sa, bw.hs.sb);
+                rr[k] = r;
+                pk[k] = plan.pk[col];
                 g[k] = *px[k];
-                cell[k] = cs_in[r * (int64_t)bw.mod.w + (pk[k] & 0x7fffffffu)];
                 if (k + 1 < n) {      // next element of the wrap-around block (else stay on a valid address)
                     ++col;
                     if (col == bw.m) {
@@ -396,6 +406,8 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
                     }
                 }
             }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) cell[k] = cs_in[rr[k] * (int64_t)w + (pk[k] & 0x7fffffffu)];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 if (k < n) {
@@ -569,7 +581,8 @@ int conef_launch_binned_rows(Stage stage, const ConefPlanHeader* hp, const void*
     int threads_a = (hp->chunk_cols / 4 + 63) & ~63;
     if (threads_a > 1024) threads_a = 1024;
     int tpad = (hp->bin_buckets + 63) & ~63;
-    int col_threads = bw.x ? 256 : 0;                   // waves of pass B that do the fused step's column work
+    static int col_env = getenv("CONEF_COL_THREADS") ? atoi(getenv("CONEF_COL_THREADS")) : 256;
+    int col_threads = bw.x ? col_env : 0;               // waves of pass B that do the fused step's column work
     if (tpad + col_threads > 1024) col_threads = 1024 - tpad;
     if (bw.x && col_threads < 64) return CONEF_ERR_INVALID;
     int threads_b = (1024 - col_threads) / tpad * tpad + col_threads;

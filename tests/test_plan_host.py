@@ -25,7 +25,8 @@ def build_plan(n, d, w, chunk=0, tbin=0):
         h["nbins"], h["nchunks"] + 1)
     h["csr"] = buf[int(i64[9]):int(i64[9]) + 4 * (w + 1)].view(np.uint32)
     h["ent"] = buf[int(i64[10]):int(i64[10]) + 2 * d].view(np.uint16)
-    assert int(i64[12]) >= 4 * n * d
+    assert int(i64[13]) >= 4 * n * d
+    h["pk"] = buf[int(i64[11]):int(i64[11]) + 4 * d].view(np.uint32)
     return h
 
 
@@ -87,6 +88,8 @@ def test_plan_tables_are_consistent(oracle):
     bins = bucket // h["T"]
     np.testing.assert_array_equal(h["seg"][:, -1] >> 16, np.bincount(bins, minlength=h["nbins"]))
     assert h["maxrec"] == np.bincount(bins, minlength=h["nbins"]).max()
+    np.testing.assert_array_equal(h["pk"] & 0x7fffffff, bucket.astype(np.uint32))
+    np.testing.assert_array_equal(h["pk"] >> 31, (sign > 0).astype(np.uint32))
     # entries of a bucket carry that bucket's signs, in ascending column order
     order = np.lexsort((np.arange(d), bucket))
     np.testing.assert_array_equal(h["ent"] >> 15, (sign[order] > 0).astype(np.uint16))
