@@ -44,15 +44,20 @@ SIGNATURES = {
     "conef_psgd_mq_f32": [_P, _P, _P, _I64, _I64, _I32, _P],
     "conef_psgd_mq_ef_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _P],
     "conef_psgd_mq_conef_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P],
-    "conef_psgd_mtp_f32": [_P, _P, _P, _I64, _I64, _I32, _P],
+    "conef_psgd_mq_conef_planned_f32": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P],
+    "conef_psgd_workspace_bytes": [_I64, _I64, _I32],
+    "conef_psgd_mtp_f32": [_P, _P, _P, _I64, _I64, _I32, _P, _I64, _P],
     "conef_psgd_pqt_f32": [_P, _P, _P, _I64, _I64, _I32, _P],
     "conef_psgd_pqt_ef_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _P],
     "conef_psgd_pqt_conef_f32": [_P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P],
-    "conef_gram_schmidt_f32": [_P, _I64, _I32, _F32, _P],
+    "conef_psgd_pqt_conef_planned_f32": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P],
+    "conef_gram_schmidt_f32": [_P, _I64, _I32, _F32, _P, _I64, _P],
     "conef_ef_passthrough_f32": [_P, _P, _I64, _P],
     "conef_plan_bytes": [_I64, _I64, _I32, _I32, _I32],
     "conef_plan_build_host": [_P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32],
     "conef_plan_workspace_bytes": [_P],
+    "conef_plan_kind": [_P],
+    "conef_cs_update_planned_f16": [_P, _P, _P, _P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],
     "conef_cs_update_planned_f32": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],
     "conef_randblock_conef_step_planned_f32": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I32, _I64, _I64, _F32, _F32,
                                                _I32, _I32, _P],
@@ -60,7 +65,8 @@ SIGNATURES = {
     "conef_topk_sparsify_f32": [_P, _I64, _I64, _P, _I64, _P],
 }
 
-_RETURNS_I64 = ("conef_topk_workspace_bytes", "conef_plan_bytes", "conef_plan_workspace_bytes")
+_RETURNS_I64 = ("conef_topk_workspace_bytes", "conef_plan_bytes", "conef_plan_workspace_bytes",
+                "conef_psgd_workspace_bytes")
 
 _handle = None
 

@@ -1,8 +1,9 @@
-"""Host/device holder of an accumulation plan for sketches whose rows do not fit LDS.
+"""Host/device holder of an accumulation plan of a count sketch.
 
-The plan (built once per sketch by ``conef_plan_build_host``) lists where every column's record
-goes, so that the count-sketch update of a long row runs as two streaming passes without
-atomics and adds each bucket's terms in ascending column order.
+The plan (built once per sketch by ``conef_plan_build_host``) lists where every column goes, so
+that the count-sketch update runs without atomics and adds each bucket's terms in ascending
+column order: per-bucket column lists when a row fits LDS (``kind`` 1), two binned streaming
+passes through a staging buffer for a few long rows (``kind`` 0).
 """
 import numpy as np
 import torch
@@ -24,17 +25,24 @@ class SketchPlan:
         _lib.check(rc, "conef_plan_build_host")
         self.device = torch.from_numpy(self.host).to(device)
         ws = lib.conef_plan_workspace_bytes(self.host.ctypes.data)
-        self.workspace = torch.empty(ws, dtype=torch.uint8, device=device)
+        self.workspace = torch.empty(max(ws, 16), dtype=torch.uint8, device=device)
+        self.kind = lib.conef_plan_kind(self.host.ctypes.data)
         self.key = (n, d, w, a, b)
 
     @property
     def host_ptr(self):
         return self.host.ctypes.data
 
+    BINNED, ROWLIST = 0, 1
+
+    @property
+    def in_place(self):
+        """Whether the fused steps may write the sketch they read (row lists) or need a second buffer."""
+        return self.kind == self.ROWLIST
+
     @staticmethod
-    def applicable(n, d, w):
-        lib = _lib.load()
-        return n <= 8 and not lib.conef_cs_update_inplace_ok(n, d, w)
+    def applicable(n, d, w, chunk_cols=0, bin_buckets=0):
+        return _lib.load().conef_plan_bytes(n, d, w, chunk_cols, bin_buckets) > 0
 
     def header(self):
         """Decoded header fields (for tests and diagnostics)."""
@@ -45,4 +53,4 @@ class SketchPlan:
                 "chunk_cols": int(i32[9]), "nchunks": int(i32[10]), "bin_buckets": int(i32[11]),
                 "nbins": int(i32[12]), "max_bin_records": int(i32[13]), "off_pos": int(i64[7]),
                 "off_seg": int(i64[8]), "off_csr": int(i64[9]), "off_ent": int(i64[10]), "off_pk": int(i64[11]),
-                "total_bytes": int(i64[12]), "workspace_bytes": int(i64[13])}
+                "total_bytes": int(i64[12]), "workspace_bytes": int(i64[13]), "kind": int(i64[14])}

@@ -23,12 +23,32 @@ def should_compress(num_rows, num_cols, matrix_approximation_rank, min_compressi
     return (compressed_size * min_compression_rate < uncompressed_size, uncompressed_size, compressed_size)
 
 
-def orthogonalize(matrix, epsilon=0):
+def orthogonalize(matrix, epsilon=0, workspace=None):
     """In-place Gram-Schmidt of a contiguous [rows, r] device matrix (powerSGD_hook.py:12-44)."""
     _lib.require_device_f32(matrix, "matrix")
     rows, r = matrix.shape
-    rc = _lib.load().conef_gram_schmidt_f32(matrix.data_ptr(), rows, r, float(epsilon), _lib.stream_ptr(matrix))
+    lib = _lib.load()
+    need = lib.conef_psgd_workspace_bytes(rows, 1, r)
+    if workspace is None or workspace.numel() < need:
+        workspace = _workspace(matrix.device, _lib.stream_ptr(matrix), need)
+    rc = lib.conef_gram_schmidt_f32(matrix.data_ptr(), rows, r, float(epsilon), workspace.data_ptr(),
+                                    workspace.numel(), _lib.stream_ptr(matrix))
     _lib.check(rc, "conef_gram_schmidt_f32")
+    return workspace
+
+
+_WORKSPACES = {}
+
+
+def _workspace(device, stream, nbytes):
+    """Device scratch for sums that cross workgroups: one buffer per (device, stream), grown on
+    demand.  Kernels that use it are ordered by that stream."""
+    key = (device, stream)
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+        _WORKSPACES[key] = ws
+    return ws
 
 
 def topk_sparsify(err, topk_ratio, workspace=None):
@@ -114,6 +134,9 @@ def run_round(state, bucket, error_mode):
         q_idx += m * rank
 
     eps = float(state.orthogonalization_epsilon)
+    ws_bytes = max([lib.conef_psgd_workspace_bytes(n, m, rank) for _, n, m, rank in work] or [256])
+    ws = _workspace(device, stream, ws_bytes)
+    ws_ptr, ws_len = ws.data_ptr(), ws.numel()
     if need_randomize_qs:
         # same seeded CPU draws as the reference so every replica starts from the same Q (:479-494)
         with torch.random.fork_rng(devices=[]):
@@ -122,7 +145,7 @@ def run_round(state, bucket, error_mode):
         for q, hq in zip(qs, host_q):
             q.copy_(hq)
     for q in qs:
-        rc = lib.conef_gram_schmidt_f32(q.data_ptr(), q.shape[0], q.shape[1], eps, stream)
+        rc = lib.conef_gram_schmidt_f32(q.data_ptr(), q.shape[0], q.shape[1], eps, ws_ptr, ws_len, stream)
         _lib.check(rc, "conef_gram_schmidt_f32")
 
     alpha = 1 - state.beta if error_mode == "conef" else 0.0
@@ -139,8 +162,14 @@ def run_round(state, bucket, error_mode):
             if cnt not in errs:
                 errs[cnt] = DenseCS(n, m, state.sketch_size, device=device)
             cs = errs[cnt]
-            rc = lib.conef_psgd_mq_conef_f32(matrix.data_ptr(), cs.cs.data_ptr(), q.data_ptr(), p.data_ptr(), n, m,
-                                             rank, cs.range, float(alpha), cs.a, cs.b, stream)
+            plan = cs.plan()
+            if plan is not None:
+                rc = lib.conef_psgd_mq_conef_planned_f32(matrix.data_ptr(), cs.cs.data_ptr(), q.data_ptr(),
+                                                         p.data_ptr(), plan.host_ptr, plan.device.data_ptr(), n, m,
+                                                         rank, cs.range, float(alpha), cs.a, cs.b, stream)
+            else:
+                rc = lib.conef_psgd_mq_conef_f32(matrix.data_ptr(), cs.cs.data_ptr(), q.data_ptr(), p.data_ptr(), n,
+                                                 m, rank, cs.range, float(alpha), cs.a, cs.b, stream)
         elif error_mode == "topk":
             if cnt not in errs:
                 errs[cnt] = torch.zeros_like(matrix)
@@ -161,9 +190,10 @@ def run_round(state, bucket, error_mode):
 
     # pass 2: orthogonalise P, Q = M^T P
     for (matrix, n, m, rank), p, q in zip(work, ps, qs):
-        _lib.check(lib.conef_gram_schmidt_f32(p.data_ptr(), n, rank, eps, stream), "conef_gram_schmidt_f32")
-        _lib.check(lib.conef_psgd_mtp_f32(matrix.data_ptr(), p.data_ptr(), q.data_ptr(), n, m, rank, stream),
-                   "conef_psgd_mtp_f32")
+        _lib.check(lib.conef_gram_schmidt_f32(p.data_ptr(), n, rank, eps, ws_ptr, ws_len, stream),
+                   "conef_gram_schmidt_f32")
+        _lib.check(lib.conef_psgd_mtp_f32(matrix.data_ptr(), p.data_ptr(), q.data_ptr(), n, m, rank, ws_ptr, ws_len,
+                                          stream), "conef_psgd_mtp_f32")
 
     # pass 3: M = P Q^T with the residual fused
     topk_ws = None
@@ -175,11 +205,18 @@ def run_round(state, bucket, error_mode):
                                            stream)
         elif error_mode == "conef":
             cs = errs[cnt]
-            out = cs.next_buffer()
-            rc = lib.conef_psgd_pqt_conef_f32(matrix.data_ptr(), p.data_ptr(), q.data_ptr(), cs.cs.data_ptr(),
-                                              out.data_ptr(), n, m, rank, cs.range, float(state.beta), cs.a, cs.b,
-                                              stream)
-            cs.commit(out)
+            plan = cs.plan()
+            if plan is not None and plan.in_place:
+                rc = lib.conef_psgd_pqt_conef_planned_f32(matrix.data_ptr(), p.data_ptr(), q.data_ptr(),
+                                                          cs.cs.data_ptr(), cs.cs.data_ptr(), plan.host_ptr,
+                                                          plan.device.data_ptr(), n, m, rank, cs.range,
+                                                          float(state.beta), cs.a, cs.b, stream)
+            else:
+                out = cs.next_buffer()
+                rc = lib.conef_psgd_pqt_conef_f32(matrix.data_ptr(), p.data_ptr(), q.data_ptr(), cs.cs.data_ptr(),
+                                                  out.data_ptr(), n, m, rank, cs.range, float(state.beta), cs.a,
+                                                  cs.b, stream)
+                cs.commit(out)
         elif error_mode == "topk":
             rc = lib.conef_psgd_pqt_ef_f32(matrix.data_ptr(), errs[cnt].data_ptr(), p.data_ptr(), q.data_ptr(), n, m,
                                            rank, stream)

@@ -4,9 +4,11 @@ Same constructor, attributes (N, D, blk_size, range, cs, a, b) and methods as th
 Differences a maintainer should know about:
   * the kernels are precompiled gfx950 code reached through libconef_hip.so, not CuPy/NVRTC;
   * alpha, beta, a, b travel by value, so ``a``/``b`` are Python ints, not 1-element device tensors;
-  * when a sketch row does not fit LDS (W above a few thousand) and the tensor has at most 8 rows,
-    updates run on a precomputed plan (two streaming passes, no atomics, deterministic); with more
-    rows ``update`` writes into a second buffer and ``self.cs`` is rebound to it;
+  * updates run on a plan built once per sketch (no atomics, deterministic, the accumulation order
+    of the reference's serial definition): per-bucket column lists when a row fits LDS, two binned
+    streaming passes for a flat bucket viewed as at most 8 long rows.  The binned fused step writes
+    into a second buffer and ``self.cs`` is rebound to it; shapes neither kind covers (long rows
+    and more than 8 of them) fall back to float atomics;
   * ``state_dict``/``load_state_dict`` round-trip (the reference's __setstate__ loses a, b).
 """
 import os
@@ -71,14 +73,14 @@ class DenseCS:
             raise ValueError("%s is on %s, the sketch on %s" % (name, t.device, self.cs.device))
 
     def plan(self):
-        """Accumulation plan for long rows (built on first use), or None when a row fits LDS or the
-        tensor has more than 8 rows.  CONEF_PLAN_CHUNK / CONEF_PLAN_BIN override the tile sizes and
+        """Accumulation plan (built on first use), or None when no kind of plan covers the shape.
+        CONEF_PLAN_CHUNK / CONEF_PLAN_BIN ask for a binned plan with those tile sizes and
         CONEF_PLAN=0 disables the planned path (the kernels then accumulate with float atomics)."""
-        if self._plan is None and not self._inplace and os.environ.get("CONEF_PLAN", "1") != "0":
-            if SketchPlan.applicable(self.N, self.D, self.range):
-                self._plan = SketchPlan(self.N, self.D, self.range, self.a, self.b, self.cs.device,
-                                        int(os.environ.get("CONEF_PLAN_CHUNK", "0")),
-                                        int(os.environ.get("CONEF_PLAN_BIN", "0")))
+        if self._plan is None and os.environ.get("CONEF_PLAN", "1") != "0":
+            chunk = int(os.environ.get("CONEF_PLAN_CHUNK", "0"))
+            tbin = int(os.environ.get("CONEF_PLAN_BIN", "0"))
+            if SketchPlan.applicable(self.N, self.D, self.range, chunk, tbin):
+                self._plan = SketchPlan(self.N, self.D, self.range, self.a, self.b, self.cs.device, chunk, tbin)
         if self._plan is not None and self._plan.key != (self.N, self.D, self.range, self.a, self.b):
             self._plan = None
             return self.plan()
@@ -123,7 +125,8 @@ class DenseCS:
         stream = _lib.stream_ptr(x)
         plan = self.plan()
         if plan is not None:
-            out = self.spare_buffer()      # the planned step reads the old sketch while it writes the new one
+            # the binned step reads the old sketch while it writes the new one
+            out = self.cs if plan.in_place else self.spare_buffer()
             rc = self._lib.conef_randblock_conef_step_planned_f32(
                 x.data_ptr(), self.cs.data_ptr(), out.data_ptr(), payload.data_ptr(), plan.host_ptr,
                 plan.device.data_ptr(), plan.workspace.data_ptr(), self.N, self.D, self.range, start, block,

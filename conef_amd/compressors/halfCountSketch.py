@@ -2,12 +2,15 @@
 
 The reference casts the whole sketch to fp32 before every kernel and back to fp16 after it.  Here
 the kernels read fp16 cells, compute in fp32 and round once on the way out, which gives the same
-values without the two extra passes; only when a sketch row does not fit LDS does ``update`` go
-through an explicit fp32 staging copy.
+values without the two extra passes.  ``update`` runs on a row-list plan (no atomics) when a row
+fits LDS; longer rows go through an explicit fp32 staging copy.
 """
+import os
+
 import torch
 
 from .. import _lib
+from .._plan import SketchPlan
 from .CountSketch import HASH_A, HASH_B
 
 
@@ -24,6 +27,15 @@ class DenseCS:
         self.b = HASH_B
         self._lib = _lib.load()
         self._inplace = bool(self._lib.conef_cs_update_inplace_ok(self.N, self.D, self.range))
+        self._plan = None
+
+    def plan(self):
+        """Row-list plan (built on first use) or None; CONEF_PLAN=0 disables it."""
+        if self._plan is None and os.environ.get("CONEF_PLAN", "1") != "0":
+            if SketchPlan.applicable(self.N, self.D, self.range):
+                plan = SketchPlan(self.N, self.D, self.range, self.a, self.b, self.cs.device)
+                self._plan = plan if plan.kind == SketchPlan.ROWLIST else False
+        return self._plan or None
 
     def state_dict(self):
         return {"N": self.N, "D": self.D, "blk_size": self.blk_size, "range": self.range,
@@ -43,6 +55,13 @@ class DenseCS:
     def update(self, vec, beta):
         self._check(vec, "vec")
         s = _lib.stream_ptr(vec)
+        plan = self.plan()
+        if plan is not None:
+            rc = self._lib.conef_cs_update_planned_f16(vec.data_ptr(), self.cs.data_ptr(), self.cs.data_ptr(),
+                                                       plan.host_ptr, plan.device.data_ptr(), self.N, self.D,
+                                                       self.range, float(beta), self.a, self.b, s)
+            _lib.check(rc, "conef_cs_update_planned_f16")
+            return
         if self._inplace:
             rc = self._lib.conef_cs_update_f16(vec.data_ptr(), self.cs.data_ptr(), self.cs.data_ptr(), self.N,
                                                self.D, self.range, float(beta), self.a, self.b, s)

@@ -26,22 +26,15 @@
 
 #include "conef_device.h"
 #include "conef_sketch_core.h"
-
-#ifdef CONEF_PHASE_CLOCKS
-// debugging aid (not compiled into the library): per-wave timestamps of kernel phases
-__device__ unsigned long long conef_clk[2][1024][16][8];
-#define CONEF_CLK(i) CONEF_CLKK(1, i)
-#define CONEF_CLKK(kk, i)                                                                                         \
-    do {                                                                                                          \
-        if ((threadIdx.x & 63) == 0 && blockIdx.x < 1024) conef_clk[kk][blockIdx.x][threadIdx.x >> 6][i] = wall_clock64(); \
-    } while (0)
-#else
-#define CONEF_CLK(i)
-#define CONEF_CLKK(kk, i)
-#endif
+#include "conef_rowlist.h"
 
 constexpr uint32_t kConefPlanMagic = 0x50464E43u;   // "CNFP"
 constexpr int kConefPlanMaxRows = 8;
+// Two kinds of plan share the header.  Row lists (conef_rowlist.h): a row fits LDS, any number of
+// rows, tables csr / ent (column | sign << 15) / pk only, no staging buffer.  Binned (this file):
+// long rows, at most 8 of them.
+constexpr int64_t kConefPlanBinned = 0;
+constexpr int64_t kConefPlanRowlist = 1;
 
 struct ConefPlanHeader {
     uint32_t magic;
@@ -60,17 +53,39 @@ struct ConefPlanHeader {
     int64_t off_ent;           // uint16[d]: (slot inside bin image) | (sign bit << 15), buckets ascending, columns ascending
     int64_t off_pk;            // uint32[d]: bucket | (sign bit << 31) of every column, for the column-order work
     int64_t total_bytes;
-    int64_t workspace_bytes;   // staging buffer: n * d floats, rounded up
-    int64_t reserved[3];
+    int64_t workspace_bytes;   // staging buffer: n * d floats, rounded up (binned plans only)
+    int64_t kind;              // kConefPlanBinned or kConefPlanRowlist
+    int64_t reserved[2];
 };
 
 inline int64_t conef_align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
-// Shape decisions that do not depend on the hash values.
+// Shape decisions that do not depend on the hash values.  Tile hints ask for a binned plan.
 inline bool conef_plan_shape(int64_t n, int64_t d, int32_t w, int32_t hint_chunk, int32_t hint_bin,
                              ConefPlanHeader* h)
 {
-    if (n < 1 || n > kConefPlanMaxRows || d < 1 || d > 0x7fffffffLL || w < 1 || w > (1 << 30)) return false;
+    if (n < 1 || d < 1 || d > 0x7fffffffLL || w < 1 || w > (1 << 30)) return false;
+    ConefRowlistShape rl;
+    if (hint_chunk <= 0 && hint_bin <= 0 && conef_rowlist_shape(n, d, w, true, &rl)) {
+        memset(h, 0, sizeof(*h));
+        h->magic = kConefPlanMagic;
+        h->version = 1;
+        h->kind = kConefPlanRowlist;
+        h->n = n;
+        h->d = d;
+        h->w = w;
+        int64_t off = conef_align256(sizeof(ConefPlanHeader));
+        h->off_csr = off;
+        off += conef_align256(4 * ((int64_t)w + 1));
+        h->off_ent = off;
+        off += conef_align256(2 * d);
+        h->off_pk = off;
+        off += conef_align256(4 * d);
+        h->total_bytes = off;
+        h->workspace_bytes = 0;
+        return true;
+    }
+    if (n > kConefPlanMaxRows) return false;
     memset(h, 0, sizeof(*h));
     int64_t c = hint_chunk > 0 ? hint_chunk : (100 * 1024) / (4 * n);   // a 100 KB chunk image: one workgroup per CU
     if (c > 16384) c = 16384;
@@ -90,6 +105,7 @@ inline bool conef_plan_shape(int64_t n, int64_t d, int32_t w, int32_t hint_chunk
     if (t > 768) t = 768;      // leaves room in a 1024-thread workgroup for the waves that do column work
     h->magic = kConefPlanMagic;
     h->version = 1;
+    h->kind = kConefPlanBinned;
     h->n = n;
     h->d = d;
     h->w = w;
@@ -121,6 +137,25 @@ inline bool conef_plan_fill(void* buf, const ConefPlanHeader& shape, int32_t a, 
     h.a = a;
     h.b = b;
     const int64_t d = h.d;
+    if (h.kind == kConefPlanRowlist) {
+        char* rbase = (char*)buf;
+        uint32_t* rcsr = (uint32_t*)(rbase + h.off_csr);
+        uint16_t* rent = (uint16_t*)(rbase + h.off_ent);
+        uint32_t* rpk = (uint32_t*)(rbase + h.off_pk);
+        ConefMod rmod = conef_make_mod(h.w);
+        std::vector<uint32_t> count((size_t)h.w + 1, 0);
+        for (int64_t i = 0; i < d; ++i) {
+            rpk[i] = conef_bucket_sign((int32_t)i, rmod, a, b, a + 2, b + 3);
+            count[(rpk[i] & 0x7fffffffu) + 1]++;
+        }
+        rcsr[0] = 0;
+        for (int32_t j = 0; j < h.w; ++j) rcsr[j + 1] = rcsr[j] + count[(size_t)j + 1];
+        std::vector<uint32_t> cur(rcsr, rcsr + h.w);
+        for (int64_t i = 0; i < d; ++i)       // ascending columns inside every bucket
+            rent[cur[rpk[i] & 0x7fffffffu]++] = (uint16_t)((uint32_t)i | ((rpk[i] >> 31) << 15));
+        memcpy(rbase, &h, sizeof(h));
+        return true;
+    }
     const int32_t w = h.w, C = h.chunk_cols, T = h.bin_buckets, nbins = h.nbins, nchunks = h.nchunks;
     char* base = (char*)buf;
     uint16_t* pos = (uint16_t*)(base + h.off_pos);
@@ -189,14 +224,16 @@ struct ConefPlanView {
     int32_t flags;   // bit 0: XCD-major work mapping, bit 1: streaming (nontemporal) stores
 };
 
-inline int32_t conef_plan_flags()
+// XCD-major work mapping and streaming stores for the zero fill: both measured faster on the
+// 25 MB bucket; streaming stores for the staging image (bit 2) measured slower.
+inline int32_t conef_plan_flags() { return 3; }
+
+inline ConefRowlistView conef_rowlist_view(const ConefPlanHeader* host, const void* dev)
 {
-    static int32_t flags = -1;
-    if (flags < 0) {
-        const char* e = getenv("CONEF_PLAN_FLAGS");
-        flags = e ? atoi(e) : 3;
-    }
-    return flags;
+    const char* b = (const char*)dev;
+    ConefRowlistView v = {(const uint32_t*)(b + host->off_csr), (const uint16_t*)(b + host->off_ent),
+                          (const uint32_t*)(b + host->off_pk)};
+    return v;
 }
 
 inline ConefPlanView conef_plan_view(const ConefPlanHeader* host, const void* dev)
@@ -293,7 +330,6 @@ __global__ void __launch_bounds__(1024)
 conef_binned_stage_kernel(Stage stage, ConefPlanView plan, float* __restrict__ staging, int64_t d, int nblocks_padded)
 {
     extern __shared__ float conef_img[];   // [chunk_cols][NROWS]
-    CONEF_CLKK(0, 0);
     const int chunk = conef_xcd_major(blockIdx.x, nblocks_padded, plan.flags);
     if (chunk >= plan.nchunks) return;
     const int64_t c_begin = (int64_t)chunk * plan.chunk_cols;
@@ -323,9 +359,7 @@ conef_binned_stage_kernel(Stage stage, ConefPlanView plan, float* __restrict__ s
             }
         }
     }
-    CONEF_CLKK(0, 1);
     __syncthreads();
-    CONEF_CLKK(0, 2);
     float* out = staging + c_begin * NROWS;        // 16-byte aligned: c_begin is a multiple of 4
     const int total = cols * NROWS;
     const int total4 = total >> 2;
@@ -334,7 +368,6 @@ conef_binned_stage_kernel(Stage stage, ConefPlanView plan, float* __restrict__ s
         conef_store4(out + 4 * e, v.x, v.y, v.z, v.w, (plan.flags & 4) != 0);
     }
     for (int e = (total4 << 2) + threadIdx.x; e < total; e += blockDim.x) out[e] = conef_img[e];
-    CONEF_CLKK(0, 3);
 }
 
 // Column-order work of the fused RandomBlock step that pass B carries (x == null: none).
@@ -369,7 +402,6 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
                                int glog, int col_threads, ConefBlockWork bw)
 {
     extern __shared__ float conef_img[];
-    CONEF_CLK(0);
     const int gthreads = blockDim.x - col_threads;      // threads that work on the bin
     if ((int)threadIdx.x >= gthreads) {
         // ---- column-order work of the fused step.  These waves owe the bin's threads nothing:
@@ -417,7 +449,6 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
                 }
             }
         }
-        CONEF_CLK(1);
         const bool vec_ok = (reinterpret_cast<uintptr_t>(bw.x) & 15u) == 0;
         const int64_t nquads = (bw.numel + 3) >> 2;
         for (int64_t q = me; q < nquads; q += nworkers) {
@@ -431,7 +462,6 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
                     if (!any_sel || conef_payload_pos(f + k, bw.blk) < 0) bw.x[f + k] = 0.f;
             }
         }
-        CONEF_CLK(2);
         return;
     }
 
@@ -487,10 +517,8 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
 #pragma unroll
         for (int r = 0; r < NROWS; ++r) v[u][r] = srcp[u][k * NROWS + r];
     }
-    CONEF_CLK(1);
     if (has_bin)
         for (uint32_t t = threadIdx.x; t < e_last - e_first; t += gthreads) ent_l[t] = plan.ent[e_first + t];
-    CONEF_CLK(2);
 
     // records into the image; segments longer than a lane group, and chunks beyond the first
     // four per group, take the slow lane-strided loop
@@ -516,9 +544,7 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
             }
         }
     }
-    CONEF_CLK(3);
     __syncthreads();
-    CONEF_CLK(4);
 
     if (!active) return;
     // per row: the decay c*aux (double) and the query term for sign +1 do not change along the
@@ -550,13 +576,11 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
             }
         }
     }
-    CONEF_CLK(5);
 #pragma unroll
     for (int k = 0; k < NROWS; ++k) {
         int r = sub + k * nsub;
         if (r < NROWS) cs_out[(int64_t)r * w + j] = acc[k];
     }
-    CONEF_CLK(6);
 }
 
 // ---------------------------------------------------------------- launcher ----
@@ -581,8 +605,7 @@ int conef_launch_binned_rows(Stage stage, const ConefPlanHeader* hp, const void*
     int threads_a = (hp->chunk_cols / 4 + 63) & ~63;
     if (threads_a > 1024) threads_a = 1024;
     int tpad = (hp->bin_buckets + 63) & ~63;
-    static int col_env = getenv("CONEF_COL_THREADS") ? atoi(getenv("CONEF_COL_THREADS")) : 256;
-    int col_threads = bw.x ? col_env : 0;               // waves of pass B that do the fused step's column work
+    int col_threads = bw.x ? 256 : 0;                   // waves of pass B that do the fused step's column work
     if (tpad + col_threads > 1024) col_threads = 1024 - tpad;
     if (bw.x && col_threads < 64) return CONEF_ERR_INVALID;
     int threads_b = (1024 - col_threads) / tpad * tpad + col_threads;
@@ -641,6 +664,7 @@ int conef_launch_binned(Stage stage, const ConefPlanHeader* hp, const void* plan
 // validates a host-side plan header against the call's shape
 inline bool conef_plan_matches(const ConefPlanHeader* hp, int64_t n, int64_t d, int32_t w, int32_t a, int32_t b)
 {
-    return hp && hp->magic == kConefPlanMagic && hp->version == 1 && hp->n == n && hp->d == d && hp->w == w &&
+    return hp && hp->magic == kConefPlanMagic && hp->version == 1 &&
+           (hp->kind == kConefPlanBinned || hp->kind == kConefPlanRowlist) && hp->n == n && hp->d == d && hp->w == w &&
            hp->a == a && hp->b == b;
 }

@@ -1,5 +1,5 @@
-// Entry points of the planned (atomic-free, deterministic) sketch accumulation for long rows;
-// the scheme is described at the top of conef_plan.h.
+// Entry points of the planned (atomic-free, deterministic) sketch accumulation: row lists when a
+// row fits LDS (conef_rowlist.h), two binned passes for a few long rows (conef_plan.h).
 #include "conef_plan.h"
 
 namespace {
@@ -8,14 +8,14 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 extern "C" {
 
-// Bytes of a plan for an [n,d] tensor sketched at width w; 0 when the planned path does not apply
-// (more than 8 rows), -1 on invalid arguments.  chunk_cols / bin_buckets = 0 pick defaults.
+// Bytes of a plan for an [n,d] tensor sketched at width w; 0 when no planned path applies (rows
+// too long for LDS and more than 8 of them), -1 on invalid arguments.  chunk_cols / bin_buckets:
+// 0 picks the kind and its defaults, a positive value asks for a binned plan with that tiling.
 int64_t conef_plan_bytes(int64_t n, int64_t d, int32_t w, int32_t chunk_cols, int32_t bin_buckets)
 {
     if (n < 1 || d < 1 || w < 1 || w > (1 << 30) || d > 0x7fffffffLL) return -1;
-    if (n > kConefPlanMaxRows) return 0;
     ConefPlanHeader h;
-    if (!conef_plan_shape(n, d, w, chunk_cols, bin_buckets, &h)) return -1;
+    if (!conef_plan_shape(n, d, w, chunk_cols, bin_buckets, &h)) return n > kConefPlanMaxRows ? 0 : -1;
     return h.total_bytes;
 }
 
@@ -29,7 +29,7 @@ int conef_plan_build_host(void* plan_host, int64_t plan_bytes, int64_t n, int64_
     if (plan_bytes < h.total_bytes) return CONEF_ERR_INVALID;
     if (!conef_plan_fill(plan_host, h, a, b)) return CONEF_ERR_INVALID;
     const ConefPlanHeader* built = (const ConefPlanHeader*)plan_host;
-    if (conef_binned_lds_b(built, (int)n) > 160 * 1024) return CONEF_ERR_INVALID;
+    if (built->kind == kConefPlanBinned && conef_binned_lds_b(built, (int)n) > 160 * 1024) return CONEF_ERR_INVALID;
     return CONEF_OK;
 }
 
@@ -45,12 +45,41 @@ int conef_cs_update_planned_f32(const float* vec, const float* cs_in, float* cs_
                                 int32_t a, int32_t b, void* stream)
 {
     const ConefPlanHeader* hp = (const ConefPlanHeader*)plan_host;
-    if (!conef_plan_matches(hp, n, d, w, a, b) || !plan_dev || !workspace || !vec || !cs_in || !cs_out)
-        return CONEF_ERR_INVALID;
+    if (!conef_plan_matches(hp, n, d, w, a, b) || !plan_dev || !vec || !cs_in || !cs_out) return CONEF_ERR_INVALID;
+    if (hp->kind == kConefPlanRowlist) {
+        ConefListVec front = {vec, aligned16(vec) && d % 4 == 0};
+        return conef_launch_rowlist(front, conef_rowlist_view(hp, plan_dev), cs_in, cs_out, n, d, w, beta,
+                                    (hipStream_t)stream);
+    }
+    if (!workspace) return CONEF_ERR_INVALID;
     ConefStageVec stage = {vec, d};
     ConefBlockWork none = {};
     return conef_launch_binned(stage, hp, plan_dev, (float*)workspace, cs_in, cs_out, 0.f, beta, aligned16(vec), none,
                                (hipStream_t)stream);
+}
+
+// fp16-storage sketch on a row-list plan (cells read as fp16, arithmetic as in the f32 update,
+// one rounding to nearest-even when a cell is written); binned plans are f32 only.
+int conef_cs_update_planned_f16(const float* vec, const void* cs_in_half, void* cs_out_half, const void* plan_host,
+                                const void* plan_dev, int64_t n, int64_t d, int32_t w, float beta, int32_t a,
+                                int32_t b, void* stream)
+{
+    const ConefPlanHeader* hp = (const ConefPlanHeader*)plan_host;
+    if (!conef_plan_matches(hp, n, d, w, a, b) || !plan_dev || !vec || !cs_in_half || !cs_out_half)
+        return CONEF_ERR_INVALID;
+    if (hp->kind != kConefPlanRowlist) return CONEF_ERR_INVALID;
+    ConefListVec front = {vec, aligned16(vec) && d % 4 == 0};
+    return conef_launch_rowlist(front, conef_rowlist_view(hp, plan_dev), (const __half*)cs_in_half,
+                                (__half*)cs_out_half, n, d, w, beta, (hipStream_t)stream);
+}
+
+// 0 = binned (needs the workspace, fused step needs cs_out != cs_in), 1 = row lists (no
+// workspace, in place allowed), -1 = not a plan.
+int conef_plan_kind(const void* plan_host)
+{
+    const ConefPlanHeader* h = (const ConefPlanHeader*)plan_host;
+    if (!h || h->magic != kConefPlanMagic) return -1;
+    return (int)h->kind;
 }
 
 int conef_randblock_conef_step_planned_f32(float* x, const float* cs_in, float* cs_out, float* payload,
@@ -59,12 +88,18 @@ int conef_randblock_conef_step_planned_f32(float* x, const float* cs_in, float* 
                                            float beta, int32_t a, int32_t b, void* stream)
 {
     const ConefPlanHeader* hp = (const ConefPlanHeader*)plan_host;
-    if (!conef_plan_matches(hp, n, m, w, a, b) || !plan_dev || !workspace || !x || !cs_in || !cs_out || !payload)
+    if (!conef_plan_matches(hp, n, m, w, a, b) || !plan_dev || !x || !cs_in || !cs_out || !payload)
         return CONEF_ERR_INVALID;
     int64_t numel = n * m;
     if (!(start >= 0 && start < numel && block >= 1 && block <= numel)) return CONEF_ERR_INVALID;
-    if (cs_in == cs_out) return CONEF_ERR_INVALID;   // the block is finished while buckets are being rewritten
     ConefBlock blk = conef_make_block(numel, start, block);
+    if (hp->kind == kConefPlanRowlist) {
+        ConefListRandBlock front = {x, payload, blk, alpha, aligned16(x) && m % 4 == 0};
+        return conef_launch_rowlist(front, conef_rowlist_view(hp, plan_dev), cs_in, cs_out, n, m, w, beta,
+                                    (hipStream_t)stream);
+    }
+    if (!workspace) return CONEF_ERR_INVALID;
+    if (cs_in == cs_out) return CONEF_ERR_INVALID;   // the block is finished while buckets are being rewritten
     ConefSeeds hs = {a, b, a + 2, b + 3};
     ConefStageRandBlock stage = {x, m, blk};
     ConefBlockWork bw = {x, payload, numel, m, block, blk, conef_make_mod(w), hs, alpha};

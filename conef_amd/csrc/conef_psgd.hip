@@ -6,10 +6,13 @@
 //
 // At the ranks gradient compression uses (1..8) these products move 4 bytes of M per 2r flops, far
 // below the fp32 ridge of the machine, so they are written as streaming kernels: M is read exactly
-// once per product, the rank dimension lives in registers, and the error-feedback add (before the
-// first product) and the residual (after the last) are fused into the passes that touch M anyway.
+// once per product with 16-byte accesses, the rank dimension lives in registers, and the
+// error-feedback add (before the first product) and the residual (after the last) are fused into
+// the passes that touch M anyway.  Sums that cross workgroups meet through a caller-provided
+// workspace in a fixed order: no atomics, results do not change from run to run.
 #include "conef_device.h"
 #include "conef_sketch_core.h"
+#include "conef_plan.h"
 
 namespace {
 
@@ -17,44 +20,107 @@ constexpr int kMaxRank = 32;
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+__device__ __forceinline__ void ld4(const float* p, float* v)
+{
+    float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void st4(float* p, const float* v)
+{
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+// All kernels come in a FAST form (r equals the compile-time rank bound RP, m % 4 == 0, every
+// pointer 16-byte aligned: 16-byte accesses, Q rows of a column quad are one contiguous run) and a
+// general form (any r <= RP, any alignment, 4-byte accesses).
+
 // ---------------------------------------------------------------- P = X Q ----
 // MODE 0: X = M as stored.  MODE 1: X = M + E (dense error), written back into M.
-// MODE 2: X = M + alpha * unsketch(cs), written back into M (DenseCS.query fused).
-// A workgroup owns RB consecutive rows and all columns; a thread owns columns tid, tid+256, ...
+// MODE 2: X = M + alpha * unsketch(cs), written back into M (DenseCS.query fused); the sketch rows
+// of the workgroup's matrix rows are parked in LDS first.
+// A workgroup owns RB consecutive rows and all columns; a thread owns column quads tid, tid+256, ...
 // and keeps RB x RP partial sums, reduced over the workgroup at the end in a fixed order.
-template <int RB, int RP, int MODE>
+template <int RB, int RP, int MODE, bool FAST>
 __global__ void __launch_bounds__(256)
 psgd_mq_kernel(float* __restrict__ x, const float* __restrict__ err, const float* __restrict__ cs,
-               const float* __restrict__ q, float* __restrict__ p, int64_t n, int64_t m, int r, ConefMod mod,
-               float alpha, ConefSeeds hs)
+               const uint32_t* __restrict__ pktab, const float* __restrict__ q, float* __restrict__ p, int64_t n,
+               int m, int r, ConefMod mod, float alpha, ConefSeeds hs)
 {
-    __shared__ float red[4][RB * RP];
+    extern __shared__ float mq_lds[];
+    float* red = mq_lds;                    // [4][RB*RP]
+    float* cells = mq_lds + 4 * RB * RP;    // [RB][w], MODE 2 only
     const int64_t row0 = (int64_t)blockIdx.x * RB;
+    const int w = (int)mod.w;
+    int64_t rowc[RB];                       // rows past the end are clamped for loads, their stores are skipped
+#pragma unroll
+    for (int a = 0; a < RB; ++a) rowc[a] = row0 + a < n ? row0 + a : n - 1;
+    if (MODE == 2) {
+#pragma unroll
+        for (int a = 0; a < RB; ++a)
+            for (int j = threadIdx.x; j < w; j += 256) cells[a * w + j] = cs[rowc[a] * w + j];
+        __syncthreads();
+    }
     float acc[RB][RP];
 #pragma unroll
     for (int a = 0; a < RB; ++a)
 #pragma unroll
         for (int c = 0; c < RP; ++c) acc[a][c] = 0.f;
 
-    for (int64_t k = threadIdx.x; k < m; k += 256) {
-        float qk[RP];
+    if (FAST) {
+        const int m4 = m >> 2;
+        for (int j = threadIdx.x; j < m4; j += 256) {
+            float xv[RB][4];
 #pragma unroll
-        for (int c = 0; c < RP; ++c) qk[c] = c < r ? q[k * r + c] : 0.f;
-        uint32_t pk = 0;
-        if (MODE == 2) pk = conef_bucket_sign((int32_t)k, mod, hs.a, hs.b, hs.sa, hs.sb);
+            for (int a = 0; a < RB; ++a) ld4(x + rowc[a] * m + 4 * j, xv[a]);
+            float qf[4 * RP];               // Q rows 4j..4j+3: 4*RP consecutive floats
 #pragma unroll
-        for (int a = 0; a < RB; ++a) {
-            int64_t row = row0 + a;
-            if (row < n) {
-                float v = x[row * m + k];
-                if (MODE == 1) {
-                    v = __fadd_rn(v, err[row * m + k]);
-                    x[row * m + k] = v;
-                } else if (MODE == 2) {
-                    float cell = cs[row * (int64_t)mod.w + (pk & 0x7fffffffu)];
-                    v = __fadd_rn(v, conef_query_term(cell, pk, alpha));
-                    x[row * m + k] = v;
+            for (int t = 0; t < RP; ++t) ld4(q + (int64_t)j * 4 * RP + 4 * t, qf + 4 * t);
+            if (MODE == 1) {
+#pragma unroll
+                for (int a = 0; a < RB; ++a) {
+                    float ev[4];
+                    ld4(err + rowc[a] * m + 4 * j, ev);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) xv[a][k] = __fadd_rn(xv[a][k], ev[k]);
+                    if (row0 + a < n) st4(x + rowc[a] * m + 4 * j, xv[a]);
                 }
+            } else if (MODE == 2) {
+                uint32_t pk[4];
+                if (pktab) {
+                    uint4 t = reinterpret_cast<const uint4*>(pktab)[j];
+                    pk[0] = t.x; pk[1] = t.y; pk[2] = t.z; pk[3] = t.w;
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) pk[k] = conef_bucket_sign(4 * j + k, mod, hs.a, hs.b, hs.sa, hs.sb);
+                }
+#pragma unroll
+                for (int a = 0; a < RB; ++a) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        xv[a][k] = __fadd_rn(xv[a][k], conef_query_term(cells[a * w + (pk[k] & 0x7fffffffu)], pk[k], alpha));
+                    if (row0 + a < n) st4(x + rowc[a] * m + 4 * j, xv[a]);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+#pragma unroll
+                for (int a = 0; a < RB; ++a)
+#pragma unroll
+                    for (int c = 0; c < RP; ++c) acc[a][c] = fmaf(xv[a][k], qf[k * RP + c], acc[a][c]);
+        }
+    } else {
+        for (int k = threadIdx.x; k < m; k += 256) {
+            float qk[RP];
+#pragma unroll
+            for (int c = 0; c < RP; ++c) qk[c] = c < r ? q[(int64_t)k * r + c] : 0.f;
+            uint32_t pk = 0;
+            if (MODE == 2) pk = pktab ? pktab[k] : conef_bucket_sign(k, mod, hs.a, hs.b, hs.sa, hs.sb);
+#pragma unroll
+            for (int a = 0; a < RB; ++a) {
+                float v = x[rowc[a] * m + k];
+                if (MODE == 1) v = __fadd_rn(v, err[rowc[a] * m + k]);
+                if (MODE == 2) v = __fadd_rn(v, conef_query_term(cells[a * w + (pk & 0x7fffffffu)], pk, alpha));
+                if (MODE != 0 && row0 + a < n) x[rowc[a] * m + k] = v;
 #pragma unroll
                 for (int c = 0; c < RP; ++c) acc[a][c] = fmaf(v, qk[c], acc[a][c]);
             }
@@ -66,81 +132,247 @@ psgd_mq_kernel(float* __restrict__ x, const float* __restrict__ err, const float
 #pragma unroll
         for (int c = 0; c < RP; ++c) {
             float s = conef_wave_sum(acc[a][c]);
-            if (lane == 0) red[wave][a * RP + c] = s;
+            if (lane == 0) red[wave * RB * RP + a * RP + c] = s;
         }
     __syncthreads();
     if (threadIdx.x < RB * RP) {
         int a = threadIdx.x / RP, c = threadIdx.x % RP;
-        int64_t row = row0 + a;
-        if (row < n && c < r)
-            p[row * r + c] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+        int t = threadIdx.x;
+        if (row0 + a < n && c < r)
+            p[(row0 + a) * r + c] = (red[t] + red[RB * RP + t]) + (red[2 * RB * RP + t] + red[3 * RB * RP + t]);
     }
 }
 
 // -------------------------------------------------------------- Q = X^T P ----
-// A thread owns one column of X; the workgroup walks a slab of rows.  With one slab the result is
-// stored, with several the slabs meet through float atomics on a zeroed Q.
-template <int RP>
-__global__ void __launch_bounds__(256)
-psgd_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, float* q, int64_t n, int64_t m, int r,
-                int64_t rows_per_slab, int use_atomics)
+// A workgroup of 8 waves owns 256 columns and a slab of rows.  A lane owns a column quad, wave v
+// takes rows v, v+8, ... of the slab (one contiguous kilobyte per row), the 8 waves meet in LDS.
+// With one slab the result is stored, with several each slab writes a partial [m,r] and a second
+// small kernel adds the partials in slab order: deterministic, no atomics.
+constexpr int kMtpWaves = 8;
+constexpr int kMtpThreads = 64 * kMtpWaves;
+
+template <int RP, bool FAST>
+__global__ void __launch_bounds__(kMtpThreads)
+psgd_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, float* __restrict__ out, int64_t n, int m,
+                int r, int rows_per_slab)
 {
-    int64_t k = blockIdx.x * (int64_t)256 + threadIdx.x;
-    if (k >= m) return;
-    int64_t i0 = (int64_t)blockIdx.y * rows_per_slab;
-    int64_t i1 = i0 + rows_per_slab < n ? i0 + rows_per_slab : n;
-    float acc[RP];
+    constexpr int CH = RP < 4 ? RP : 4;            // ranks reduced per LDS round
+    __shared__ float red[kMtpWaves][CH][256];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int c0 = blockIdx.x * 256 + lane * 4;    // first column of my quad
+    const int64_t i0 = (int64_t)blockIdx.y * rows_per_slab;
+    const int64_t i1 = i0 + rows_per_slab < n ? i0 + rows_per_slab : n;
+    float acc[4][RP];
 #pragma unroll
-    for (int c = 0; c < RP; ++c) acc[c] = 0.f;
-    for (int64_t i = i0; i < i1; ++i) {
-        float v = x[i * m + k];
-        const float* pi = p + i * r;
+    for (int k = 0; k < 4; ++k)
 #pragma unroll
-        for (int c = 0; c < RP; ++c)
-            if (c < r) acc[c] = fmaf(v, pi[c], acc[c]);
-    }
+        for (int c = 0; c < RP; ++c) acc[k][c] = 0.f;
+    if (FAST) {
+        const int cc = c0 < m ? c0 : m - 4;         // clamped: lanes past the edge load a valid quad, results unused
+        for (int64_t i = i0 + wave; i < i1; i += kMtpWaves) {
+            float xv[4];
+            ld4(x + i * m + cc, xv);
+            const float* pi = p + i * RP;
 #pragma unroll
-    for (int c = 0; c < RP; ++c)
-        if (c < r) {
-            if (use_atomics) unsafeAtomicAdd(q + k * r + c, acc[c]);
-            else q[k * r + c] = acc[c];
+            for (int c = 0; c < RP; ++c) {
+                float pc = pi[c];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) acc[k][c] = fmaf(xv[k], pc, acc[k][c]);
+            }
         }
+    } else {
+        for (int64_t i = i0 + wave; i < i1; i += kMtpWaves) {
+            float xv[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) xv[k] = x[i * m + (c0 + k < m ? c0 + k : m - 1)];
+            const float* pi = p + i * r;
+#pragma unroll
+            for (int c = 0; c < RP; ++c) {
+                float pc = c < r ? pi[c] : 0.f;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) acc[k][c] = fmaf(xv[k], pc, acc[k][c]);
+            }
+        }
+    }
+    float* dst = out + (int64_t)blockIdx.y * m * r;   // partial of this slab (or Q itself with one slab)
+#pragma unroll
+    for (int cb = 0; cb < RP; cb += CH) {
+        if (cb) __syncthreads();
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) red[wave][c][lane * 4 + k] = acc[k][cb + c];
+        __syncthreads();
+        if (threadIdx.x < 256) {
+            const int col = blockIdx.x * 256 + threadIdx.x;
+            float s[CH];
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                float t = 0.f;
+#pragma unroll
+                for (int v = 0; v < kMtpWaves; ++v) t += red[v][c][threadIdx.x];
+                s[c] = t;
+            }
+            if (col < m) {
+                if (FAST && CH == 4) {
+                    st4(dst + (int64_t)col * RP + cb, s);
+                } else {
+#pragma unroll
+                    for (int c = 0; c < CH; ++c)
+                        if (cb + c < r) dst[(int64_t)col * r + cb + c] = s[c];
+                }
+            }
+        }
+    }
 }
 
-__global__ void zero_kernel(float* x, int64_t count)
+// out[i] = sum over slabs of partial[s][i], slabs in ascending order
+__global__ void __launch_bounds__(256)
+psgd_sum_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, int64_t count, int slabs)
 {
-    int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
-    int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (; i < count; i += stride) x[i] = 0.f;
+    int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
+    if (i >= count) return;
+    float s = partial[i];
+    for (int k = 1; k < slabs; ++k) s += partial[(int64_t)k * count + i];
+    out[i] = s;
 }
 
 // ------------------------------------------------------------ M = P Q^T ----
 // MODE 0: write M.  MODE 1: also write the dense residual E = X - M (X = what M held on entry).
-template <int RP, int MODE>
+// A thread owns a column quad (its 4 x r slice of Q stays in registers), the workgroup walks a slab
+// of rows; the row of P is uniform over the workgroup.
+template <int RP, int MODE, bool FAST>
 __global__ void __launch_bounds__(256)
 psgd_pqt_kernel(float* __restrict__ x, float* __restrict__ err, const float* __restrict__ p,
-                const float* __restrict__ q, int64_t n, int64_t m, int r, int64_t rows_per_slab)
+                const float* __restrict__ q, int64_t n, int m, int r, int rows_per_slab)
 {
-    int64_t k = blockIdx.x * (int64_t)256 + threadIdx.x;
-    if (k >= m) return;
-    float qk[RP];
+    const int c0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (c0 >= m) return;
+    const int64_t i0 = (int64_t)blockIdx.y * rows_per_slab;
+    const int64_t i1 = i0 + rows_per_slab < n ? i0 + rows_per_slab : n;
+    float qf[4][RP];
+    if (FAST) {
+        float flat[4 * RP];
 #pragma unroll
-    for (int c = 0; c < RP; ++c) qk[c] = c < r ? q[k * r + c] : 0.f;
-    int64_t i0 = (int64_t)blockIdx.y * rows_per_slab;
-    int64_t i1 = i0 + rows_per_slab < n ? i0 + rows_per_slab : n;
-    for (int64_t i = i0; i < i1; ++i) {
-        const float* pi = p + i * r;
-        float mh = 0.f;
+        for (int t = 0; t < RP; ++t) ld4(q + (int64_t)c0 * RP + 4 * t, flat + 4 * t);
 #pragma unroll
-        for (int c = 0; c < RP; ++c)
-            if (c < r) mh = fmaf(pi[c], qk[c], mh);
-        if (MODE == 1) err[i * m + k] = __fsub_rn(x[i * m + k], mh);
-        x[i * m + k] = mh;
+        for (int k = 0; k < 4; ++k)
+#pragma unroll
+            for (int c = 0; c < RP; ++c) qf[k][c] = flat[k * RP + c];
+        for (int64_t i = i0; i < i1; ++i) {
+            const float* pi = p + i * RP;
+            float mh[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < RP; ++c) {
+                float pc = pi[c];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) mh[k] = fmaf(pc, qf[k][c], mh[k]);
+            }
+            float* px = x + i * m + c0;
+            if (MODE == 1) {
+                float xv[4], ev[4];
+                ld4(px, xv);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) ev[k] = __fsub_rn(xv[k], mh[k]);
+                st4(err + i * m + c0, ev);
+            }
+            st4(px, mh);
+        }
+    } else {
+        const int valid = m - c0 < 4 ? m - c0 : 4;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+#pragma unroll
+            for (int c = 0; c < RP; ++c) qf[k][c] = (k < valid && c < r) ? q[(int64_t)(c0 + k) * r + c] : 0.f;
+        for (int64_t i = i0; i < i1; ++i) {
+            const float* pi = p + i * r;
+            float mh[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < RP; ++c) {
+                float pc = c < r ? pi[c] : 0.f;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) mh[k] = fmaf(pc, qf[k][c], mh[k]);
+            }
+            for (int k = 0; k < valid; ++k) {
+                int64_t f = i * m + c0 + k;
+                if (MODE == 1) err[f] = __fsub_rn(x[f], mh[k]);
+                x[f] = mh[k];
+            }
+        }
     }
 }
 
-// Front for the sketch back end: the value to sketch is the residual X - P Q^T, and M is
+// Front of the row-list sketch kernel: the value to sketch is the residual X - P Q^T, and M is
 // overwritten with P Q^T on the way (powerSGD_hook.py:551,563-564).
+template <int RP, bool FAST>
+struct ListPsgdResidual {
+    float* x;
+    const float* p;
+    const float* q;
+    int r;
+    static constexpr bool kNeedsCells = false;
+    __device__ __forceinline__ void stage(int64_t row0, int rows, int d, int, float* vals, const float*,
+                                          const uint32_t*) const
+    {
+        float* base = x + row0 * d;
+        if (FAST) {
+            const int d4 = d >> 2, total4 = rows * d4;
+            int row = threadIdx.x / d4, c4 = threadIdx.x - row * d4;
+            const int srow = kConefRowlistThreads / d4, sc = kConefRowlistThreads - srow * d4;
+            for (int t = threadIdx.x; t < total4; t += kConefRowlistThreads) {
+                float xv[4], flat[4 * RP], pr[RP];
+                ld4(base + 4 * t, xv);
+#pragma unroll
+                for (int u = 0; u < RP; ++u) ld4(q + (int64_t)c4 * 4 * RP + 4 * u, flat + 4 * u);
+                const float* pi = p + (row0 + row) * RP;
+                if (RP >= 4) {
+#pragma unroll
+                    for (int u = 0; u < RP / 4; ++u) ld4(pi + 4 * u, pr + 4 * u);
+                } else {
+#pragma unroll
+                    for (int c = 0; c < RP; ++c) pr[c] = pi[c];
+                }
+                float mh[4] = {0.f, 0.f, 0.f, 0.f}, v[4];
+#pragma unroll
+                for (int c = 0; c < RP; ++c)
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) mh[k] = fmaf(pr[c], flat[k * RP + c], mh[k]);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[k] = __fsub_rn(xv[k], mh[k]);
+                st4(base + 4 * t, mh);
+                st4(vals + 4 * t, v);
+                row += srow;
+                c4 += sc;
+                if (c4 >= d4) {
+                    c4 -= d4;
+                    ++row;
+                }
+            }
+        } else {
+            const int total = rows * d;
+            int row = threadIdx.x / d, col = threadIdx.x - row * d;
+            const int srow = kConefRowlistThreads / d, sc = kConefRowlistThreads - srow * d;
+            for (int e = threadIdx.x; e < total; e += kConefRowlistThreads) {
+                const float* pi = p + (row0 + row) * r;
+                const float* qk = q + (int64_t)col * r;
+                float mh = 0.f;
+#pragma unroll
+                for (int c = 0; c < RP; ++c)
+                    if (c < r) mh = fmaf(pi[c], qk[c], mh);
+                vals[e] = __fsub_rn(base[e], mh);
+                base[e] = mh;
+                row += srow;
+                col += sc;
+                if (col >= d) {
+                    col -= d;
+                    ++row;
+                }
+            }
+        }
+    }
+};
+
+// Same residual as a front of the atomics-based sketch kernels (no plan given).
 struct FrontPsgdResidual {
     float* x;
     const float* p;
@@ -172,24 +404,38 @@ struct FrontPsgdResidual {
 };
 
 // ------------------------------------------------------------ Gram-Schmidt ----
-// In place on a row-major [rows, r] matrix; one workgroup per matrix.  Column by column:
-// col /= ||col|| (+eps when eps != 0), then every later column loses its projection on col
-// (powerSGD_hook.py:21-43).  Each thread keeps to its own rows, so the only exchange per column
-// is one workgroup reduction of (||col||^2, col . later columns); the projection coefficients of
-// the normalised column are those dot products divided by the norm.
+// In place on a row-major [rows, r] matrix.  Column by column: col /= ||col|| (+eps when eps != 0),
+// then every later column loses its projection on col (powerSGD_hook.py:21-43).  Each thread keeps
+// to its own rows, so the only exchange per column is one reduction of (||col||^2, col . later
+// columns); the projection coefficients of the normalised column are those dot products divided
+// by the norm.
+//
+// Small matrices: one workgroup, the matrix lives in LDS (row stride r+1: no bank conflicts) for
+// the whole factorisation.
+constexpr size_t kGsLdsLimit = 144 * 1024;
+
 template <int RP>
 __global__ void __launch_bounds__(1024)
-gram_schmidt_kernel(float* __restrict__ a, int64_t rows, int r, float eps)
+gram_schmidt_lds_kernel(float* __restrict__ a, int rows, int r, float eps)
 {
-    __shared__ float red[16][RP];
-    __shared__ float tot[RP];
+    extern __shared__ float gs_lds[];
+    float* red = gs_lds;                 // [16][RP]
+    float* tot = red + 16 * RP;          // [RP]
+    float* al = tot + RP;                // [rows][r+1]
+    const int ld = r + 1;
+    const int nthreads = blockDim.x, nwaves = nthreads >> 6;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int e = threadIdx.x; e < rows * r; e += nthreads) {
+        int k = e / r;
+        al[k * ld + (e - k * r)] = a[e];
+    }
+    __syncthreads();
     for (int i = 0; i < r; ++i) {
         float acc[RP];
 #pragma unroll
         for (int c = 0; c < RP; ++c) acc[c] = 0.f;
-        for (int64_t k = threadIdx.x; k < rows; k += 1024) {
-            const float* row = a + k * r;
+        for (int k = threadIdx.x; k < rows; k += nthreads) {
+            const float* row = al + k * ld;
             float ci = row[i];
 #pragma unroll
             for (int c = 0; c < RP; ++c)
@@ -197,14 +443,15 @@ gram_schmidt_kernel(float* __restrict__ a, int64_t rows, int r, float eps)
         }
 #pragma unroll
         for (int c = 0; c < RP; ++c) {
-            float s = conef_wave_sum(acc[c]);
-            if (lane == 0) red[wave][c] = s;
+            if (i + c < r) {
+                float s = conef_wave_sum(acc[c]);
+                if (lane == 0) red[wave * RP + c] = s;
+            }
         }
         __syncthreads();
         if (threadIdx.x < RP) {
             float s = 0.f;
-#pragma unroll
-            for (int wv = 0; wv < 16; ++wv) s += red[wv][threadIdx.x];
+            for (int wv = 0; wv < nwaves; ++wv) s += red[wv * RP + threadIdx.x];
             tot[threadIdx.x] = s;
         }
         __syncthreads();
@@ -213,49 +460,171 @@ gram_schmidt_kernel(float* __restrict__ a, int64_t rows, int r, float eps)
         float coef[RP];
 #pragma unroll
         for (int c = 1; c < RP; ++c) coef[c] = (i + c < r) ? tot[c] / den : 0.f;
-        for (int64_t k = threadIdx.x; k < rows; k += 1024) {
-            float* row = a + k * r;
+        for (int k = threadIdx.x; k < rows; k += nthreads) {
+            float* row = al + k * ld;
             float ci = row[i] / den;
             row[i] = ci;
 #pragma unroll
             for (int c = 1; c < RP; ++c)
                 if (i + c < r) row[i + c] = __fsub_rn(row[i + c], __fmul_rn(coef[c], ci));
         }
-        __syncthreads();   // red/tot are reused by the next column
+        // the next column's sums read only the thread's own rows; red/tot are rewritten after the
+        // next pair of barriers has been passed by everyone who read them
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < rows * r; e += nthreads) {
+        int k = e / r;
+        a[e] = al[k * ld + (e - k * r)];
     }
 }
 
+// Large matrices: r+1 launches over all CUs.  Launch i first finishes column i-1 on its own rows
+// (normalise it, take its projection off the later columns) from the sums launch i-1 left, then
+// sums column i against the later columns over its rows and leaves one partial per workgroup.
+// Every workgroup adds the partials in the same order, so all of them see the same sums.
+template <int RP>
+__global__ void __launch_bounds__(256)
+gram_schmidt_step_kernel(float* __restrict__ a, int64_t rows, int r, float eps, int i, const float* __restrict__ sums_in,
+                         float* __restrict__ sums_out, int rows_per_wg)
+{
+    __shared__ float red[4][RP];
+    __shared__ float tot[RP];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    float coef[RP];
+    float den = 1.f;
+    if (i > 0) {
+        if (threadIdx.x < RP) {
+            float s = 0.f;
+            for (int g = 0; g < (int)gridDim.x; ++g) s += sums_in[g * RP + threadIdx.x];
+            tot[threadIdx.x] = s;
+        }
+        __syncthreads();
+        float nrm = sqrtf(tot[0]);
+        den = eps == 0.f ? nrm : nrm + eps;
+#pragma unroll
+        for (int c = 1; c < RP; ++c) coef[c] = (i - 1 + c < r) ? tot[c] / den : 0.f;
+    }
+    float acc[RP];
+#pragma unroll
+    for (int c = 0; c < RP; ++c) acc[c] = 0.f;
+    const int64_t k0 = (int64_t)blockIdx.x * rows_per_wg;
+    const int64_t k1 = k0 + rows_per_wg < rows ? k0 + rows_per_wg : rows;
+    for (int64_t k = k0 + threadIdx.x; k < k1; k += 256) {
+        float* row = a + k * r;
+        float cur[RP];                  // columns i.. of this row after column i-1 has been dealt with
+#pragma unroll
+        for (int c = 0; c < RP; ++c) cur[c] = 0.f;
+        if (i > 0) {
+            float ci = row[i - 1] / den;
+            row[i - 1] = ci;
+#pragma unroll
+            for (int c = 1; c < RP; ++c)
+                if (i - 1 + c < r) {
+                    float v = __fsub_rn(row[i - 1 + c], __fmul_rn(coef[c], ci));
+                    row[i - 1 + c] = v;
+                    cur[c - 1] = v;
+                }
+        } else {
+#pragma unroll
+            for (int c = 0; c < RP; ++c)
+                if (c < r) cur[c] = row[c];
+        }
+        if (i < r) {
+#pragma unroll
+            for (int c = 0; c < RP; ++c)
+                if (i + c < r) acc[c] = fmaf(cur[0], cur[c], acc[c]);
+        }
+    }
+    if (i >= r) return;
+#pragma unroll
+    for (int c = 0; c < RP; ++c) {
+        float s = conef_wave_sum(acc[c]);
+        if (lane == 0) red[wave][c] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x < RP)
+        sums_out[blockIdx.x * RP + threadIdx.x] =
+            (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+}
+
+constexpr int kGsMaxWorkgroups = 256;
+
 // ---------------------------------------------------------------- dispatch ----
+inline int rank_bound(int r) { return r <= 1 ? 1 : r <= 2 ? 2 : r <= 4 ? 4 : r <= 8 ? 8 : r <= 16 ? 16 : 32; }
+
+#define CONEF_RANK_SWITCH(r, CALL)      \
+    switch (rank_bound(r)) {            \
+        case 1: CALL(1); break;         \
+        case 2: CALL(2); break;         \
+        case 4: CALL(4); break;         \
+        case 8: CALL(8); break;         \
+        case 16: CALL(16); break;       \
+        default: CALL(32); break;       \
+    }
+
 template <int MODE>
-int launch_mq(float* x, const float* err, const float* cs, const float* q, float* p, int64_t n, int64_t m, int r,
-              int32_t w, float alpha, ConefSeeds hs, hipStream_t s)
+int launch_mq(float* x, const float* err, const float* cs, const uint32_t* pktab, const float* q, float* p, int64_t n,
+              int64_t m, int r, int32_t w, float alpha, ConefSeeds hs, hipStream_t s)
 {
     ConefMod mod = conef_make_mod(w > 0 ? w : 1);
-#define CONEF_MQ(RB, RP)                                                                                          \
-    hipLaunchKernelGGL((psgd_mq_kernel<RB, RP, MODE>), dim3((unsigned)((n + RB - 1) / RB)), dim3(256), 0, s, x, err, \
-                       cs, q, p, n, m, r, mod, alpha, hs)
-    if (r <= 1) CONEF_MQ(8, 1);
-    else if (r <= 2) CONEF_MQ(8, 2);
-    else if (r <= 4) CONEF_MQ(8, 4);
-    else if (r <= 8) CONEF_MQ(4, 8);
-    else if (r <= 16) CONEF_MQ(2, 16);
-    else CONEF_MQ(1, 32);
+    const bool fast = r == rank_bound(r) && m % 4 == 0 && aligned16(x) && aligned16(q) && (MODE != 1 || aligned16(err)) &&
+                      (!pktab || aligned16(pktab));
+    // rows per workgroup: 4 amortises the Q traffic, but small matrices need the workgroups
+    const int rp = rank_bound(r);
+    int rb = rp >= 32 ? 2 : 4;
+    if (n / rb < 512) rb = rp >= 32 ? 2 : 1;
+    size_t lds = (size_t)4 * rb * rp * 4 + (MODE == 2 ? (size_t)rb * w * 4 : 0);
+    if (lds > 64 * 1024) return CONEF_ERR_INVALID;   // sketch rows wider than 16K cells per matrix row group
+    dim3 grid((unsigned)((n + rb - 1) / rb));
+#define CONEF_MQ_GO(RB, RP, F)                                                                                    \
+    hipLaunchKernelGGL((psgd_mq_kernel<RB, RP, MODE, F>), grid, dim3(256), lds, s, x, err, cs, pktab, q, p, n, (int)m, \
+                       r, mod, alpha, hs)
+#define CONEF_MQ(RP)                                     \
+    do {                                                 \
+        if (RP >= 32) {                                  \
+            if (fast) CONEF_MQ_GO(2, RP, true);          \
+            else CONEF_MQ_GO(2, RP, false);              \
+        } else if (rb == 4) {                            \
+            if (fast) CONEF_MQ_GO(4, RP, true);          \
+            else CONEF_MQ_GO(4, RP, false);              \
+        } else {                                         \
+            if (fast) CONEF_MQ_GO(1, RP, true);          \
+            else CONEF_MQ_GO(1, RP, false);              \
+        }                                                \
+    } while (0)
+    CONEF_RANK_SWITCH(r, CONEF_MQ)
 #undef CONEF_MQ
+#undef CONEF_MQ_GO
     return (int)hipGetLastError();
 }
 
-inline int64_t slab_rows(int64_t n, int64_t col_tiles)
+struct MtpShape {
+    int col_tiles, slabs, rows_per_slab;
+};
+
+// enough slabs for about a thousand workgroups, each wave at least two rows
+inline MtpShape mtp_shape(int64_t n, int64_t m)
 {
-    int64_t slabs = (1024 + col_tiles - 1) / col_tiles;
-    if (slabs > (n + 7) / 8) slabs = (n + 7) / 8;
-    if (slabs < 1) slabs = 1;
-    if (slabs > 65535) slabs = 65535;
-    return (n + slabs - 1) / slabs;
+    MtpShape g;
+    g.col_tiles = (int)((m + 255) / 256);
+    int64_t slabs = (1024 + g.col_tiles - 1) / g.col_tiles;
+    int64_t rps = (n + slabs - 1) / slabs;
+    rps = (rps + 2 * kMtpWaves - 1) / (2 * kMtpWaves) * (2 * kMtpWaves);
+    g.rows_per_slab = (int)rps;
+    g.slabs = (int)((n + rps - 1) / rps);
+    return g;
+}
+
+inline int64_t gs_sums_floats(int64_t rows, int r) { return 2 * (int64_t)kGsMaxWorkgroups * rank_bound(r); }
+
+inline bool gs_fits_lds(int64_t rows, int r)
+{
+    return (size_t)(rows * (r + 1) + 17 * rank_bound(r)) * 4 <= kGsLdsLimit;
 }
 
 inline bool psgd_args_ok(int64_t n, int64_t m, int32_t r)
 {
-    return n >= 1 && m >= 1 && r >= 1 && r <= kMaxRank && n * m > 0;
+    return n >= 1 && m >= 1 && r >= 1 && r <= kMaxRank && m <= 0x7fffffffLL && n <= 0x7fffffffLL;
 }
 
 }  // namespace
@@ -266,7 +635,7 @@ int conef_psgd_mq_f32(float* x, const float* q, float* p, int64_t n, int64_t m, 
 {
     if (!psgd_args_ok(n, m, r) || !x || !q || !p) return CONEF_ERR_INVALID;
     ConefSeeds hs = {0, 0, 0, 0};
-    return launch_mq<0>(x, nullptr, nullptr, q, p, n, m, r, 1, 0.f, hs, (hipStream_t)stream);
+    return launch_mq<0>(x, nullptr, nullptr, nullptr, q, p, n, m, r, 1, 0.f, hs, (hipStream_t)stream);
 }
 
 int conef_psgd_mq_ef_f32(float* x, const float* err, const float* q, float* p, int64_t n, int64_t m, int32_t r,
@@ -274,62 +643,101 @@ int conef_psgd_mq_ef_f32(float* x, const float* err, const float* q, float* p, i
 {
     if (!psgd_args_ok(n, m, r) || !x || !err || !q || !p) return CONEF_ERR_INVALID;
     ConefSeeds hs = {0, 0, 0, 0};
-    return launch_mq<1>(x, err, nullptr, q, p, n, m, r, 1, 0.f, hs, (hipStream_t)stream);
+    return launch_mq<1>(x, err, nullptr, nullptr, q, p, n, m, r, 1, 0.f, hs, (hipStream_t)stream);
 }
 
 int conef_psgd_mq_conef_f32(float* x, const float* cs, const float* q, float* p, int64_t n, int64_t m, int32_t r,
                             int32_t w, float alpha, int32_t a, int32_t b, void* stream)
 {
-    if (!psgd_args_ok(n, m, r) || !x || !cs || !q || !p || w < 1 || w > (1 << 30) || m > 0x7fffffffLL)
-        return CONEF_ERR_INVALID;
+    if (!psgd_args_ok(n, m, r) || !x || !cs || !q || !p || w < 1 || w > (1 << 30)) return CONEF_ERR_INVALID;
     ConefSeeds hs = {a, b, a + 2, b + 3};
-    return launch_mq<2>(x, nullptr, cs, q, p, n, m, r, w, alpha, hs, (hipStream_t)stream);
+    return launch_mq<2>(x, nullptr, cs, nullptr, q, p, n, m, r, w, alpha, hs, (hipStream_t)stream);
 }
 
-int conef_psgd_mtp_f32(const float* x, const float* p, float* q, int64_t n, int64_t m, int32_t r, void* stream)
+// The same with the (bucket, sign) of every column read from a plan's table instead of hashed.
+int conef_psgd_mq_conef_planned_f32(float* x, const float* cs, const float* q, float* p, const void* plan_host,
+                                    const void* plan_dev, int64_t n, int64_t m, int32_t r, int32_t w, float alpha,
+                                    int32_t a, int32_t b, void* stream)
+{
+    const ConefPlanHeader* hp = (const ConefPlanHeader*)plan_host;
+    if (!psgd_args_ok(n, m, r) || !x || !cs || !q || !p || !plan_dev || !conef_plan_matches(hp, n, m, w, a, b))
+        return CONEF_ERR_INVALID;
+    ConefSeeds hs = {a, b, a + 2, b + 3};
+    const uint32_t* pk = (const uint32_t*)((const char*)plan_dev + hp->off_pk);
+    return launch_mq<2>(x, nullptr, cs, pk, q, p, n, m, r, w, alpha, hs, (hipStream_t)stream);
+}
+
+// Bytes of device workspace conef_psgd_mtp_f32 and conef_gram_schmidt_f32 may need for an [n,m]
+// matrix at rank r (partial sums that meet across workgroups).
+int64_t conef_psgd_workspace_bytes(int64_t n, int64_t m, int32_t r)
+{
+    if (!psgd_args_ok(n, m, r)) return -1;
+    MtpShape g = mtp_shape(n, m);
+    int64_t mtp = g.slabs > 1 ? (int64_t)g.slabs * m * r : 0;
+    int64_t rows = n > m ? n : m;
+    int64_t gs = gs_sums_floats(rows, r);
+    return conef_align256(4 * (mtp > gs ? mtp : gs));
+}
+
+int conef_psgd_mtp_f32(const float* x, const float* p, float* q, int64_t n, int64_t m, int32_t r, void* workspace,
+                       int64_t workspace_bytes, void* stream)
 {
     if (!psgd_args_ok(n, m, r) || !x || !q || !p) return CONEF_ERR_INVALID;
     hipStream_t s = (hipStream_t)stream;
-    int64_t col_tiles = (m + 255) / 256;
-    int64_t rps = slab_rows(n, col_tiles);
-    int64_t slabs = (n + rps - 1) / rps;
-    int atom = slabs > 1;
-    if (atom) {
-        int64_t cnt = m * r;
-        int64_t g = (cnt + 255) / 256;
-        if (g > 4096) g = 4096;
-        hipLaunchKernelGGL(zero_kernel, dim3((unsigned)g), dim3(256), 0, s, q, cnt);
+    MtpShape g = mtp_shape(n, m);
+    float* out = q;
+    if (g.slabs > 1) {
+        if (!workspace || workspace_bytes < (int64_t)g.slabs * m * r * 4) return CONEF_ERR_INVALID;
+        out = (float*)workspace;
     }
-    dim3 grid((unsigned)col_tiles, (unsigned)slabs);
-#define CONEF_MTP(RP) hipLaunchKernelGGL(psgd_mtp_kernel<RP>, grid, dim3(256), 0, s, x, p, q, n, m, r, rps, atom)
-    if (r <= 1) CONEF_MTP(1);
-    else if (r <= 2) CONEF_MTP(2);
-    else if (r <= 4) CONEF_MTP(4);
-    else if (r <= 8) CONEF_MTP(8);
-    else if (r <= 16) CONEF_MTP(16);
-    else CONEF_MTP(32);
+    const bool fast = r == rank_bound(r) && m % 4 == 0 && aligned16(x) && aligned16(p) && aligned16(out);
+    dim3 grid((unsigned)g.col_tiles, (unsigned)g.slabs);
+#define CONEF_MTP(RP)                                                                                            \
+    do {                                                                                                         \
+        if (fast) hipLaunchKernelGGL((psgd_mtp_kernel<RP, true>), grid, dim3(kMtpThreads), 0, s, x, p, out, n, (int)m, r, \
+                                     g.rows_per_slab);                                                           \
+        else hipLaunchKernelGGL((psgd_mtp_kernel<RP, false>), grid, dim3(kMtpThreads), 0, s, x, p, out, n, (int)m, r,     \
+                                g.rows_per_slab);                                                                \
+    } while (0)
+    CONEF_RANK_SWITCH(r, CONEF_MTP)
 #undef CONEF_MTP
+    if (g.slabs > 1) {
+        int64_t count = m * r;
+        hipLaunchKernelGGL(psgd_sum_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s, out, q,
+                           count, g.slabs);
+    }
     return (int)hipGetLastError();
 }
 
 static int launch_pqt(float* x, float* err, const float* p, const float* q, int64_t n, int64_t m, int32_t r,
                       hipStream_t s)
 {
-    int64_t col_tiles = (m + 255) / 256;
-    int64_t rps = slab_rows(n, col_tiles);
-    dim3 grid((unsigned)col_tiles, (unsigned)((n + rps - 1) / rps));
-#define CONEF_PQT(RP)                                                                                        \
-    do {                                                                                                     \
-        if (err) hipLaunchKernelGGL((psgd_pqt_kernel<RP, 1>), grid, dim3(256), 0, s, x, err, p, q, n, m, r, rps); \
-        else hipLaunchKernelGGL((psgd_pqt_kernel<RP, 0>), grid, dim3(256), 0, s, x, err, p, q, n, m, r, rps);     \
+    const bool fast = r == rank_bound(r) && m % 4 == 0 && aligned16(x) && aligned16(q) && (!err || aligned16(err));
+    int64_t col_tiles = (m + 1023) / 1024;
+    int64_t slabs = (1024 + col_tiles - 1) / col_tiles;       // about a thousand workgroups ...
+    int64_t rps = (n + slabs - 1) / slabs;
+    if (rps < 4) rps = 4;                                     // ... of at least four rows
+    slabs = (n + rps - 1) / rps;
+    if (slabs > 65535) {
+        rps = (n + 65534) / 65535;
+        slabs = (n + rps - 1) / rps;
+    }
+    dim3 grid((unsigned)col_tiles, (unsigned)slabs);
+#define CONEF_PQT_GO(RP, MODE, F) \
+    hipLaunchKernelGGL((psgd_pqt_kernel<RP, MODE, F>), grid, dim3(256), 0, s, x, err, p, q, n, (int)m, r, (int)rps)
+#define CONEF_PQT(RP)                                 \
+    do {                                              \
+        if (err) {                                    \
+            if (fast) CONEF_PQT_GO(RP, 1, true);      \
+            else CONEF_PQT_GO(RP, 1, false);          \
+        } else {                                      \
+            if (fast) CONEF_PQT_GO(RP, 0, true);      \
+            else CONEF_PQT_GO(RP, 0, false);          \
+        }                                             \
     } while (0)
-    if (r <= 1) CONEF_PQT(1);
-    else if (r <= 2) CONEF_PQT(2);
-    else if (r <= 4) CONEF_PQT(4);
-    else if (r <= 8) CONEF_PQT(8);
-    else if (r <= 16) CONEF_PQT(16);
-    else CONEF_PQT(32);
+    CONEF_RANK_SWITCH(r, CONEF_PQT)
 #undef CONEF_PQT
+#undef CONEF_PQT_GO
     return (int)hipGetLastError();
 }
 
@@ -349,26 +757,78 @@ int conef_psgd_pqt_ef_f32(float* x, float* err, const float* p, const float* q, 
 int conef_psgd_pqt_conef_f32(float* x, const float* p, const float* q, const float* cs_in, float* cs_out, int64_t n,
                              int64_t m, int32_t r, int32_t w, float beta, int32_t a, int32_t b, void* stream)
 {
-    if (!psgd_args_ok(n, m, r) || !x || !q || !p || !cs_in || !cs_out || w < 1 || w > (1 << 30) ||
-        m > 0x7fffffffLL)
+    if (!psgd_args_ok(n, m, r) || !x || !q || !p || !cs_in || !cs_out || w < 1 || w > (1 << 30))
         return CONEF_ERR_INVALID;
     ConefSeeds hs = {a, b, a + 2, b + 3};
     FrontPsgdResidual front = {x, p, q, m, r};
     return conef_launch_sketch_step<float>(front, cs_in, cs_out, n, m, w, beta, hs, (hipStream_t)stream, false);
 }
 
-int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* stream)
+// The same on a row-list plan: no atomics, bit-exact accumulation order, cs_out may be cs_in.
+int conef_psgd_pqt_conef_planned_f32(float* x, const float* p, const float* q, const float* cs_in, float* cs_out,
+                                     const void* plan_host, const void* plan_dev, int64_t n, int64_t m, int32_t r,
+                                     int32_t w, float beta, int32_t a, int32_t b, void* stream)
 {
-    if (rows < 1 || r < 1 || r > kMaxRank || !a) return CONEF_ERR_INVALID;
+    const ConefPlanHeader* hp = (const ConefPlanHeader*)plan_host;
+    if (!psgd_args_ok(n, m, r) || !x || !q || !p || !cs_in || !cs_out || !plan_dev ||
+        !conef_plan_matches(hp, n, m, w, a, b) || hp->kind != kConefPlanRowlist)
+        return CONEF_ERR_INVALID;
+    const bool fast = r == rank_bound(r) && m % 4 == 0 && aligned16(x) && aligned16(q) && aligned16(p);
+    ConefRowlistView view = conef_rowlist_view(hp, plan_dev);
     hipStream_t s = (hipStream_t)stream;
-#define CONEF_GS(RP) hipLaunchKernelGGL(gram_schmidt_kernel<RP>, dim3(1), dim3(1024), 0, s, a, rows, r, eps)
-    if (r <= 1) CONEF_GS(1);
-    else if (r <= 2) CONEF_GS(2);
-    else if (r <= 4) CONEF_GS(4);
-    else if (r <= 8) CONEF_GS(8);
-    else if (r <= 16) CONEF_GS(16);
-    else CONEF_GS(32);
+    int rc = CONEF_ERR_INVALID;
+#define CONEF_RES(RP)                                                                          \
+    do {                                                                                       \
+        if (fast) {                                                                            \
+            ListPsgdResidual<RP, true> front = {x, p, q, r};                                   \
+            rc = conef_launch_rowlist(front, view, cs_in, cs_out, n, m, w, beta, s);           \
+        } else {                                                                               \
+            ListPsgdResidual<RP, false> front = {x, p, q, r};                                  \
+            rc = conef_launch_rowlist(front, view, cs_in, cs_out, n, m, w, beta, s);           \
+        }                                                                                      \
+    } while (0)
+    CONEF_RANK_SWITCH(r, CONEF_RES)
+#undef CONEF_RES
+    return rc;
+}
+
+int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* workspace, int64_t workspace_bytes,
+                           void* stream)
+{
+    if (rows < 1 || rows > 0x7fffffffLL || r < 1 || r > kMaxRank || !a) return CONEF_ERR_INVALID;
+    hipStream_t s = (hipStream_t)stream;
+    const int rp = rank_bound(r);
+    if (gs_fits_lds(rows, r)) {
+        size_t lds = (size_t)(rows * (r + 1) + 17 * rp) * 4;
+        int threads = (int)((rows + 63) / 64 * 64);
+        if (threads > 1024) threads = 1024;
+#define CONEF_GS(RP)                                                                                              \
+    do {                                                                                                          \
+        auto k = gram_schmidt_lds_kernel<RP>;                                                                     \
+        if (lds > 48 * 1024) {                                                                                    \
+            hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+            if (e != hipSuccess) return (int)e;                                                                   \
+        }                                                                                                         \
+        hipLaunchKernelGGL(k, dim3(1), dim3(threads), lds, s, a, (int)rows, r, eps);                              \
+    } while (0)
+        CONEF_RANK_SWITCH(r, CONEF_GS)
 #undef CONEF_GS
+        return (int)hipGetLastError();
+    }
+    if (!workspace || workspace_bytes < gs_sums_floats(rows, r) * 4) return CONEF_ERR_INVALID;
+    int64_t wgs = (rows + 255) / 256;
+    if (wgs > kGsMaxWorkgroups) wgs = kGsMaxWorkgroups;
+    int rows_per_wg = (int)((rows + wgs - 1) / wgs);
+    wgs = (rows + rows_per_wg - 1) / rows_per_wg;
+    float* sums = (float*)workspace;
+    for (int i = 0; i <= r; ++i) {
+        const float* in = sums + ((i + 1) & 1) * (int64_t)kGsMaxWorkgroups * rp;
+        float* out = sums + (i & 1) * (int64_t)kGsMaxWorkgroups * rp;
+#define CONEF_GSS(RP) \
+    hipLaunchKernelGGL(gram_schmidt_step_kernel<RP>, dim3((unsigned)wgs), dim3(256), 0, s, a, rows, r, eps, i, in, out, rows_per_wg)
+        CONEF_RANK_SWITCH(r, CONEF_GSS)
+#undef CONEF_GSS
+    }
     return (int)hipGetLastError();
 }
 

@@ -1,0 +1,232 @@
+// Row-list sketch accumulation: the count-sketch update without atomics for rows that fit LDS.
+//
+// The bucket and sign of a column depend on the column alone, so every row of an [n,d] tensor
+// scatters the same way.  A plan built once per sketch lists, per bucket, the columns that fall
+// into it (ascending).  A workgroup then takes a tile of `rb` consecutive rows:
+//
+//   stage   the values to be sketched are produced in column order with 16-byte accesses and
+//           parked in LDS; whatever the fused step has to do in column order (payload, writing
+//           the decompressed gradient, the low-rank product) happens here;
+//   gather  one thread per (row, bucket) walks the bucket's list, picks its values out of LDS
+//           and adds the terms in ascending column order; the new cell leaves with a coalesced
+//           store.
+//
+// No atomics, one read of the tensor, deterministic, and the order of the adds is the CPU
+// oracle's, so the sketch comes out bit for bit.  cs_out may be cs_in: a tile reads its rows'
+// old cells before it writes them and no other tile touches those rows.
+#pragma once
+#include "conef_device.h"
+#include "conef_sketch_core.h"
+
+constexpr int kConefRowlistThreads = 256;
+constexpr int64_t kConefRowlistMaxCols = 24576;       // 4 B value + 2 B list entry per column in LDS
+constexpr size_t kConefRowlistLdsLimit = 152 * 1024;
+
+struct ConefRowlistView {
+    const uint32_t* csr;   // [w+1] first list entry of bucket j
+    const uint16_t* ent;   // [d] column | sign bit << 15, buckets ascending, columns ascending
+    const uint32_t* pk;    // [d] bucket | sign bit << 31 of every column
+};
+
+struct ConefRowlistShape {
+    int rb;          // rows per tile
+    size_t lds;      // bytes of dynamic LDS
+    int64_t tiles;
+};
+
+inline size_t conef_rowlist_lds(int rb, int64_t d, int32_t w, bool cells)
+{
+    size_t vals = (((size_t)rb * d + 3) & ~(size_t)3) * 4;
+    size_t ent = (((size_t)d + 7) & ~(size_t)7) * 2;
+    return vals + ent + (cells ? (size_t)rb * w * 4 : 0);
+}
+
+// Rows per tile: about 32 KB of values (several tiles per CU), but no more than leaves a
+// thousand tiles for the 256 CUs.
+inline bool conef_rowlist_shape(int64_t n, int64_t d, int32_t w, bool cells, ConefRowlistShape* s)
+{
+    if (d < 1 || d > kConefRowlistMaxCols || n < 1 || w < 1) return false;
+    int64_t rb = 8192 / d;
+    if (rb > n / 1024) rb = n / 1024;
+    if (rb > 16) rb = 16;
+    if (rb < 1) rb = 1;
+    while (rb > 1 && conef_rowlist_lds((int)rb, d, w, cells) > 64 * 1024) --rb;
+    size_t lds = conef_rowlist_lds((int)rb, d, w, cells);
+    if (lds > kConefRowlistLdsLimit) return false;
+    s->rb = (int)rb;
+    s->lds = lds;
+    s->tiles = (n + rb - 1) / rb;
+    return s->tiles <= 0x7fffffff;
+}
+
+// ------------------------------------------------------------------ fronts ----
+// A front fills vals[row_in_tile * d + col] for the tile's rows.  `cells` (only when
+// kNeedsCells) holds the tile's old sketch rows, [rows][w].
+
+// DenseCS.update: the value is the dense tensor itself.
+struct ConefListVec {
+    const float* vec;
+    bool vec_ok;           // 16-byte accesses allowed: base aligned and d % 4 == 0
+    static constexpr bool kNeedsCells = false;
+    __device__ __forceinline__ void stage(int64_t row0, int rows, int d, int, float* vals, const float*,
+                                          const uint32_t*) const
+    {
+        const float* base = vec + row0 * d;
+        const int total = rows * d;
+        if (vec_ok) {
+            for (int q = threadIdx.x; q < (total >> 2); q += kConefRowlistThreads)
+                reinterpret_cast<float4*>(vals)[q] = reinterpret_cast<const float4*>(base)[q];
+        } else {
+            for (int e = threadIdx.x; e < total; e += kConefRowlistThreads) vals[e] = base[e];
+        }
+    }
+};
+
+// RandomBlock + ConEF (reference: communication/RandomBlock_hook.py:190,216-243,272-280 at world
+// size 1): xq = x + alpha * unsketch(old cells); inside the wrap-around block xq goes to the
+// payload and stays in x and a zero is sketched, outside x becomes zero and xq is sketched.
+struct ConefListRandBlock {
+    float* x;
+    float* payload;
+    ConefBlock blk;
+    float alpha;
+    bool vec_ok;
+    static constexpr bool kNeedsCells = true;
+
+    __device__ __forceinline__ float finish(int64_t f, float g, float cell, uint32_t pk, float* out) const
+    {
+        float xq = __fadd_rn(g, conef_query_term(cell, pk, alpha));
+        int64_t pos = conef_payload_pos(f, blk);
+        if (pos >= 0) {
+            payload[pos] = xq;
+            *out = xq;
+            return 0.f;
+        }
+        *out = 0.f;
+        return xq;
+    }
+
+    __device__ __forceinline__ void stage(int64_t row0, int rows, int d, int w, float* vals, const float* cells,
+                                          const uint32_t* pk) const
+    {
+        const int64_t f0 = row0 * d;
+        float* base = x + f0;
+        if (vec_ok) {
+            const int d4 = d >> 2, total4 = rows * d4;
+            int row = threadIdx.x / d4, c4 = threadIdx.x - row * d4;
+            const int srow = kConefRowlistThreads / d4, sc = kConefRowlistThreads - srow * d4;
+            for (int q = threadIdx.x; q < total4; q += kConefRowlistThreads) {
+                float4 g = reinterpret_cast<const float4*>(base)[q];
+                uint4 p = reinterpret_cast<const uint4*>(pk)[c4];
+                const float* cr = cells + row * w;
+                float c0 = cr[p.x & 0x7fffffffu], c1 = cr[p.y & 0x7fffffffu];
+                float c2 = cr[p.z & 0x7fffffffu], c3 = cr[p.w & 0x7fffffffu];
+                int64_t f = f0 + ((int64_t)q << 2);
+                float4 o, v;
+                if ((f < blk.end && f + 4 > blk.start) || f < blk.rest) {
+                    v.x = finish(f, g.x, c0, p.x, &o.x);
+                    v.y = finish(f + 1, g.y, c1, p.y, &o.y);
+                    v.z = finish(f + 2, g.z, c2, p.z, &o.z);
+                    v.w = finish(f + 3, g.w, c3, p.w, &o.w);
+                } else {      // the block is one wrap-around range: most quads are entirely outside it
+                    o = make_float4(0.f, 0.f, 0.f, 0.f);
+                    v.x = __fadd_rn(g.x, conef_query_term(c0, p.x, alpha));
+                    v.y = __fadd_rn(g.y, conef_query_term(c1, p.y, alpha));
+                    v.z = __fadd_rn(g.z, conef_query_term(c2, p.z, alpha));
+                    v.w = __fadd_rn(g.w, conef_query_term(c3, p.w, alpha));
+                }
+                reinterpret_cast<float4*>(base)[q] = o;
+                reinterpret_cast<float4*>(vals)[q] = v;
+                row += srow;
+                c4 += sc;
+                if (c4 >= d4) {
+                    c4 -= d4;
+                    ++row;
+                }
+            }
+        } else {
+            const int total = rows * d;
+            int row = threadIdx.x / d, col = threadIdx.x - row * d;
+            const int srow = kConefRowlistThreads / d, sc = kConefRowlistThreads - srow * d;
+            for (int e = threadIdx.x; e < total; e += kConefRowlistThreads) {
+                uint32_t p = pk[col];
+                float o;
+                vals[e] = finish(f0 + e, base[e], cells[row * w + (p & 0x7fffffffu)], p, &o);
+                base[e] = o;
+                row += srow;
+                col += sc;
+                if (col >= d) {
+                    col -= d;
+                    ++row;
+                }
+            }
+        }
+    }
+};
+
+// ------------------------------------------------------------------ kernel ----
+template <typename CsT, typename Front>
+__global__ void __launch_bounds__(kConefRowlistThreads)
+conef_rowlist_kernel(Front front, ConefRowlistView plan, const CsT* cs_in, CsT* cs_out, int64_t n, int d, int w,
+                     int rb, double one_minus_beta)
+{
+    extern __shared__ float conef_rl[];
+    float* vals = conef_rl;
+    uint16_t* ent_l = reinterpret_cast<uint16_t*>(vals + ((rb * d + 3) & ~3));
+    float* cells = reinterpret_cast<float*>(ent_l + ((d + 7) & ~7));
+    const int64_t row0 = (int64_t)blockIdx.x * rb;
+    const int rows = n - row0 < rb ? (int)(n - row0) : rb;
+
+    // the bucket lists, two entries per load (the table is padded to a multiple of 256 bytes)
+    for (int i = threadIdx.x; i < ((d + 1) >> 1); i += kConefRowlistThreads)
+        reinterpret_cast<uint32_t*>(ent_l)[i] = reinterpret_cast<const uint32_t*>(plan.ent)[i];
+    if (Front::kNeedsCells) {
+        const CsT* src = cs_in + row0 * w;
+        for (int i = threadIdx.x; i < rows * w; i += kConefRowlistThreads) cells[i] = conef_ld(src + i);
+        __syncthreads();
+    }
+    front.stage(row0, rows, d, w, vals, cells, plan.pk);
+    __syncthreads();
+
+    const int total = rows * w;
+    int row = threadIdx.x / w, j = threadIdx.x - row * w;
+    const int srow = kConefRowlistThreads / w, sj = kConefRowlistThreads - srow * w;
+    for (int p = threadIdx.x; p < total; p += kConefRowlistThreads) {
+        const uint32_t e0 = plan.csr[j], e1 = plan.csr[j + 1];
+        const int64_t cell = (row0 + row) * w + j;
+        const float aux = Front::kNeedsCells ? cells[row * w + j] : conef_ld(cs_in + cell);
+        const double decay = __dmul_rn(one_minus_beta, (double)aux);
+        const float* vr = vals + row * d;
+        float acc = aux;
+        for (uint32_t e = e0; e < e1; ++e) {
+            uint32_t en = ent_l[e];
+            uint32_t flip = ((~en) & 0x8000u) << 16;      // sign bit clear (-1): flip the float's sign
+            double sv = (double)__uint_as_float(__float_as_uint(vr[en & 0x7fffu]) ^ flip);
+            acc = __fadd_rn(acc, (float)__dsub_rn(sv, decay));
+        }
+        conef_st(cs_out + cell, acc);
+        row += srow;
+        j += sj;
+        if (j >= w) {
+            j -= w;
+            ++row;
+        }
+    }
+}
+
+template <typename CsT, typename Front>
+int conef_launch_rowlist(Front front, ConefRowlistView plan, const CsT* cs_in, CsT* cs_out, int64_t n, int64_t d,
+                         int32_t w, float beta, hipStream_t s)
+{
+    ConefRowlistShape shape;
+    if (!conef_rowlist_shape(n, d, w, Front::kNeedsCells, &shape)) return CONEF_ERR_INVALID;
+    auto k = conef_rowlist_kernel<CsT, Front>;
+    if (shape.lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shape.lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    const double omb = 1. - (double)beta;   // (1. - beta) with beta an fp32 value, CountSketch.py:38,63
+    hipLaunchKernelGGL(k, dim3((unsigned)shape.tiles), dim3(kConefRowlistThreads), shape.lds, s, front, plan, cs_in,
+                       cs_out, n, (int)d, (int)w, shape.rb, omb);
+    return (int)hipGetLastError();
+}

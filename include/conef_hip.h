@@ -95,28 +95,38 @@ int conef_cs3_query_f32(float* x, const float* cs0, const float* cs1, const floa
 int conef_cs3_update_f32(const float* vec, const float* in0, const float* in1, const float* in2, float* out0,
                          float* out1, float* out2, int64_t n, int64_t d, int32_t w, float beta, void* stream);
 
-/* ------------------------------------------- planned accumulation for long rows -------- */
-/* When a sketch row does not fit LDS (W above a few thousand) the update has no locality and
- * float atomics on global memory are far too slow.  The hash is a fixed function of (column, w,
- * a, b), so a plan built once per sketch turns the update into two streaming passes through a
- * staging buffer, without atomics, adding each bucket's terms in ascending column order (the
- * CPU restatement's order, so results match it bit for bit).  Applies to tensors of <= 8 rows.
- * No counterpart in the reference, whose kernel cannot launch at all for such widths (it asks
- * for 8*W bytes of shared memory, CountSketch.py:158). */
+/* ------------------------------------------------ planned accumulation (no atomics) ---- */
+/* The hash is a fixed function of (column, w, a, b), so where every column of an [n,d] tensor
+ * goes is known before the first step.  A plan built once per sketch turns the update into
+ * streaming passes without atomics that add every bucket's terms in ascending column order -
+ * deterministic, and bit for bit the order of the reference's serial definition.  Two kinds:
+ *   row lists  a row fits LDS (d <= 24576), any number of rows: one pass, per-bucket column
+ *              lists, no workspace, cs_out may be cs_in;
+ *   binned     rows too long for LDS, n <= 8 (a flat bucket viewed as a few long rows): two
+ *              passes through a staging workspace of n*d floats.
+ * No counterpart in the reference (its update is one atomicAdd per element, CountSketch.py:63). */
 
-/* Size in bytes of the plan for an [n,d] tensor at width w; 0 = not applicable (n > 8),
- * -1 = invalid.  chunk_cols / bin_buckets tune the tile sizes, 0 = default.  Host function. */
+/* Bytes of a plan; 0 when neither kind applies (long rows and n > 8), -1 on invalid arguments.
+ * chunk_cols / bin_buckets: 0 picks kind and tiling, a positive value asks for a binned plan with
+ * that tiling (columns per staging workgroup, buckets per accumulating workgroup). */
 int64_t conef_plan_bytes(int64_t n, int64_t d, int32_t w, int32_t chunk_cols, int32_t bin_buckets);
 /* Builds the plan into HOST memory (plan_bytes >= conef_plan_bytes(...)).  The caller copies the
  * same bytes to the device and hands both copies to the *_planned entry points; the host copy
  * is only read for the launch geometry.  Host function, O(d). */
 int conef_plan_build_host(void* plan_host, int64_t plan_bytes, int64_t n, int64_t d, int32_t w, int32_t a,
                           int32_t b, int32_t chunk_cols, int32_t bin_buckets);
-/* Bytes of device staging memory the planned entry points need (n*d floats, rounded up). */
+/* Bytes of device staging memory the planned entry points need (binned: n*d floats, rounded up;
+ * row lists: 0, the workspace argument may then be null). */
 int64_t conef_plan_workspace_bytes(const void* plan_host);
+/* 0 = binned, 1 = row lists, -1 = not a plan. */
+int conef_plan_kind(const void* plan_host);
 
 /* conef_cs_update_f32 on a plan.  cs_out may be the same buffer as cs_in.  Calls that share a
- * workspace must be ordered on one stream. */
+ * workspace must be ordered on one stream.  The f16 form (fp16-storage sketch, replaces
+ * halfCountSketch.py:151-172) takes row-list plans only. */
+int conef_cs_update_planned_f16(const float* vec, const void* cs_in_half, void* cs_out_half, const void* plan_host,
+                                const void* plan_dev, int64_t n, int64_t d, int32_t w, float beta, int32_t a,
+                                int32_t b, void* stream);
 int conef_cs_update_planned_f32(const float* vec, const float* cs_in, float* cs_out, const void* plan_host,
                                 const void* plan_dev, void* workspace, int64_t n, int64_t d, int32_t w, float beta,
                                 int32_t a, int32_t b, void* stream);
@@ -135,8 +145,9 @@ int conef_randblock_conef_step_f32(float* x, const float* cs_in, float* cs_out, 
                                    int64_t m, int32_t w, int64_t start, int64_t block, float alpha, float beta,
                                    int32_t a, int32_t b, void* stream);
 
-/* conef_randblock_conef_step_f32 on a plan (see above).  cs_out must NOT be cs_in here (-1): the
- * selected block is finished from the old sketch while the new one is being written. */
+/* conef_randblock_conef_step_f32 on a plan (see above).  With a binned plan cs_out must NOT be
+ * cs_in (-1): the selected block is finished from the old sketch while the new one is being
+ * written.  With a row-list plan it may. */
 int conef_randblock_conef_step_planned_f32(float* x, const float* cs_in, float* cs_out, float* payload,
                                            const void* plan_host, const void* plan_dev, void* workspace, int64_t n,
                                            int64_t m, int32_t w, int64_t start, int64_t block, float alpha,
@@ -167,7 +178,13 @@ int conef_randblock_scatter_f32(float* x, const float* payload, int64_t numel, i
 /* In-place Gram-Schmidt of a row-major [rows, r] matrix: column by column, col /= ||col|| (+ eps
  * if eps != 0), then every later column loses its projection on col.
  * Replaces: _orthogonalize, powerSGD_hook.py:12-44 (about 4r torch kernels per matrix). */
-int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* stream);
+int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* workspace, int64_t workspace_bytes,
+                           void* stream);
+
+/* Bytes of device workspace conef_gram_schmidt_f32 (matrices too large for LDS) and
+ * conef_psgd_mtp_f32 (sums across row slabs) may need for an [n,m] matrix at rank r.  The sums
+ * meet in a fixed order: no atomics, results do not change from run to run. */
+int64_t conef_psgd_workspace_bytes(int64_t n, int64_t m, int32_t r);
 
 /* P = M Q.  Replaces: torch.matmul(tensor, q, out=p), powerSGD_hook.py:498. */
 int conef_psgd_mq_f32(float* x, const float* q, float* p, int64_t n, int64_t m, int32_t r, void* stream);
@@ -178,9 +195,14 @@ int conef_psgd_mq_ef_f32(float* x, const float* err, const float* q, float* p, i
 /* M += alpha*unsketch(cs) (kept in M), then P = M Q.  Replaces: DenseCS.query :409 + :498. */
 int conef_psgd_mq_conef_f32(float* x, const float* cs, const float* q, float* p, int64_t n, int64_t m,
                             int32_t r, int32_t w, float alpha, int32_t a, int32_t b, void* stream);
+/* The same with bucket and sign of every column read from a plan's table instead of hashed. */
+int conef_psgd_mq_conef_planned_f32(float* x, const float* cs, const float* q, float* p, const void* plan_host,
+                                    const void* plan_dev, int64_t n, int64_t m, int32_t r, int32_t w, float alpha,
+                                    int32_t a, int32_t b, void* stream);
 
 /* Q = M^T P.  Replaces: torch.matmul(tensor.t(), p, out=q), powerSGD_hook.py:532. */
-int conef_psgd_mtp_f32(const float* x, const float* p, float* q, int64_t n, int64_t m, int32_t r, void* stream);
+int conef_psgd_mtp_f32(const float* x, const float* p, float* q, int64_t n, int64_t m, int32_t r, void* workspace,
+                       int64_t workspace_bytes, void* stream);
 
 /* M = P Q^T.  Replaces: torch.matmul(p, q.t(), out=tensor), powerSGD_hook.py:551. */
 int conef_psgd_pqt_f32(float* x, const float* p, const float* q, int64_t n, int64_t m, int32_t r, void* stream);
@@ -193,6 +215,10 @@ int conef_psgd_pqt_ef_f32(float* x, float* err, const float* p, const float* q, 
 int conef_psgd_pqt_conef_f32(float* x, const float* p, const float* q, const float* cs_in, float* cs_out,
                              int64_t n, int64_t m, int32_t r, int32_t w, float beta, int32_t a, int32_t b,
                              void* stream);
+/* The same on a row-list plan: no atomics, the oracle's accumulation order, cs_out may be cs_in. */
+int conef_psgd_pqt_conef_planned_f32(float* x, const float* p, const float* q, const float* cs_in, float* cs_out,
+                                     const void* plan_host, const void* plan_dev, int64_t n, int64_t m, int32_t r,
+                                     int32_t w, float beta, int32_t a, int32_t b, void* stream);
 
 /* Dense error feedback on a stretch of the bucket that is not compressed: x += err; err = 0
  * (the copy-minus-result of powerSGD_hook.py:558 is exactly zero there). */

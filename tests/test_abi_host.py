@@ -57,7 +57,11 @@ def test_argument_validation_without_gpu(lib):
     assert lib.conef_randblock_ef_step_f32(1, 1, 1, 10, 10, 1, 0) == -1         # start == numel
     assert lib.conef_randblock_ef_step_f32(1, 1, 1, 10, 0, 11, 0) == -1         # block > numel
     assert lib.conef_randblock_unbiased_step_f32(1, 1, 10, 0, 1, 0.0, 0) == -1  # prob must be > 0
-    assert lib.conef_gram_schmidt_f32(1, 10, 33, 0.0, 0) == -1                  # rank above 32
+    assert lib.conef_gram_schmidt_f32(1, 10, 33, 0.0, 0, 0, 0) == -1            # rank above 32
+    assert lib.conef_gram_schmidt_f32(1, 100_000, 8, 0.0, 0, 0, 0) == -1        # too large for LDS: needs the workspace
+    assert lib.conef_psgd_mtp_f32(1, 1, 1, 640, 5760, 4, 0, 0, 0) == -1         # several row slabs: needs the workspace
+    assert lib.conef_psgd_workspace_bytes(640, 5760, 4) >= 4 * 5760 * 4
+    assert lib.conef_psgd_workspace_bytes(0, 5, 1) == -1
     assert lib.conef_psgd_mq_f32(1, 1, 1, 4, 4, 0, 0) == -1
     assert lib.conef_topk_sparsify_f32(1, 100, 10, 0, 0, 0) == -1               # no workspace
     assert lib.conef_topk_sparsify_f32(1, 100, 100, 0, 0, 0) == 0               # k >= numel: nothing to do

@@ -138,8 +138,10 @@ def test_unbiased_randomblock_bit_exact(oracle, shapes, ratio):
 
 def test_gram_schmidt_parity(oracle):
     from conef_amd.powerSGD_hook import _orthogonalize
-    for rows, r, eps in [(27, 1, 0.0), (576, 2, 0.0), (5760, 4, 0.0), (1024, 8, 0.0), (4096, 32, 0.0),
-                         (300, 3, 1e-8), (33278, 4, 0.0), (2000, 13, 0.0)]:
+    # one workgroup with the matrix in LDS up to about 36K padded elements, r+1 launches above
+    for rows, r, eps in [(27, 1, 0.0), (576, 2, 0.0), (5760, 4, 0.0), (1024, 8, 0.0), (4096, 8, 0.0), (4096, 32, 0.0),
+                         (300, 3, 1e-8), (33278, 4, 0.0), (2000, 13, 0.0), (30522, 8, 0.0), (70001, 3, 1e-8),
+                         (64, 32, 0.0), (1, 1, 0.0)]:
         g = torch.Generator().manual_seed(rows + r)
         a = torch.randn(rows, r, generator=g)
         want = a.numpy().copy()
@@ -155,21 +157,79 @@ def test_products_parity(oracle):
     from conef_amd import _lib
     lib = _lib.load()
     rng = np.random.RandomState(0)
-    for n, m, r in [(16, 27, 2), (64, 576, 2), (640, 5760, 4), (13, 29, 3), (1024, 1024, 8), (300, 4096, 32),
-                    (1000, 77, 1), (9, 4100, 16)]:
+    # (n, m, r, offset): shapes on the 16-byte path and off it (odd m, rank not a power of two,
+    # matrix starting `offset` floats into an allocation), row counts that leave ragged tiles
+    for n, m, r, off in [(16, 27, 2, 0), (64, 576, 2, 0), (640, 5760, 4, 0), (13, 29, 3, 0), (1024, 1024, 8, 0),
+                         (300, 4096, 32, 0), (1000, 77, 1, 0), (9, 4100, 16, 0), (2049, 1024, 8, 0),
+                         (4099, 260, 4, 0), (640, 5760, 4, 3), (37, 4096, 8, 2), (5000, 64, 1, 0),
+                         (30522, 128, 8, 0), (515, 1028, 5, 0)]:
         M = rng.randn(n, m).astype(np.float32)
         Q = rng.randn(m, r).astype(np.float32)
         P = rng.randn(n, r).astype(np.float32)
-        Md, Qd, Pd = (torch.from_numpy(t).cuda() for t in (M, Q, P))
+        Qd, Pd = (torch.from_numpy(t).cuda() for t in (Q, P))
+        Md = torch.zeros(n * m + off, device="cuda")[off:].view(n, m)
+        Md.copy_(torch.from_numpy(M))
+        ws = torch.empty(lib.conef_psgd_workspace_bytes(n, m, r), dtype=torch.uint8, device="cuda")
+        what = str((n, m, r, off))
         out = torch.empty(n, r, device="cuda")
         assert lib.conef_psgd_mq_f32(Md.data_ptr(), Qd.data_ptr(), out.data_ptr(), n, m, r, 0) == 0
-        assert_close(out, oracle.mq(M, Q), what="MQ %s" % ((n, m, r),))
+        assert_close(out, oracle.mq(M, Q), what="MQ " + what)
         outq = torch.empty(m, r, device="cuda")
-        assert lib.conef_psgd_mtp_f32(Md.data_ptr(), Pd.data_ptr(), outq.data_ptr(), n, m, r, 0) == 0
-        assert_close(outq, oracle.mtp(M, P), what="MtP %s" % ((n, m, r),))
-        outm = torch.empty(n, m, device="cuda")
+        assert lib.conef_psgd_mtp_f32(Md.data_ptr(), Pd.data_ptr(), outq.data_ptr(), n, m, r, ws.data_ptr(),
+                                      ws.numel(), 0) == 0
+        assert_close(outq, oracle.mtp(M, P), what="MtP " + what)
+        # dense error feedback fused into the products
+        E = rng.randn(n, m).astype(np.float32)
+        Ed = torch.from_numpy(E).cuda()
+        assert lib.conef_psgd_mq_ef_f32(Md.data_ptr(), Ed.data_ptr(), Qd.data_ptr(), out.data_ptr(), n, m, r, 0) == 0
+        ME = M + E
+        np.testing.assert_array_equal(to_np(Md), ME)
+        assert_close(out, oracle.mq(ME, Q), what="MQ+EF " + what)
+        want = oracle.pqt(P, Q)
+        assert lib.conef_psgd_pqt_ef_f32(Md.data_ptr(), Ed.data_ptr(), Pd.data_ptr(), Qd.data_ptr(), n, m, r, 0) == 0
+        assert_close(Md, want, what="PQt " + what)
+        np.testing.assert_array_equal(to_np(Ed), ME - to_np(Md))
+        outm = torch.zeros(n * m + off, device="cuda")[off:].view(n, m)
         assert lib.conef_psgd_pqt_f32(outm.data_ptr(), Pd.data_ptr(), Qd.data_ptr(), n, m, r, 0) == 0
-        assert_close(outm, oracle.pqt(P, Q), what="PQt %s" % ((n, m, r),))
+        np.testing.assert_array_equal(to_np(outm), to_np(Md))
+
+
+def test_products_with_sketch_on_a_plan(oracle):
+    """P = (M + alpha unsketch) Q and the residual sketch after M = P Q^T, on row-list plans: the
+    sketch must come out bit for bit (same terms, same order as the serial definition)."""
+    from conef_amd import _lib
+    from conef_amd.compressors.CountSketch import DenseCS
+    lib = _lib.load()
+    rng = np.random.RandomState(1)
+    for n, m, r, ss in [(64, 576, 2, 0.5), (640, 5760, 4, 0.2), (1024, 1024, 8, 0.1), (37, 4097, 3, 0.3),
+                        (4100, 260, 8, 0.25), (5, 20000, 4, 0.01)]:
+        M = rng.randn(n, m).astype(np.float32)
+        Q = rng.randn(m, r).astype(np.float32)
+        P = rng.randn(n, r).astype(np.float32)
+        cs = DenseCS(n, m, ss)
+        ocs = oracle.DenseCS(n, m, ss)
+        ocs.cs[:] = rng.randn(n, cs.range).astype(np.float32)
+        cs.cs.copy_(torch.from_numpy(ocs.cs))
+        plan = cs.plan()
+        assert plan is not None and plan.in_place
+        Md, Qd, Pd = (torch.from_numpy(t).cuda() for t in (M, Q, P))
+        out = torch.empty(n, r, device="cuda")
+        rc = lib.conef_psgd_mq_conef_planned_f32(Md.data_ptr(), cs.cs.data_ptr(), Qd.data_ptr(), out.data_ptr(),
+                                                 plan.host_ptr, plan.device.data_ptr(), n, m, r, cs.range, 0.1,
+                                                 cs.a, cs.b, 0)
+        assert rc == 0
+        MQ = M.copy()
+        ocs.query(MQ, 0.1)
+        np.testing.assert_array_equal(to_np(Md), MQ)
+        assert_close(out, oracle.mq(MQ, Q), what="MQ+ConEF %s" % ((n, m, r),))
+        rc = lib.conef_psgd_pqt_conef_planned_f32(Md.data_ptr(), Pd.data_ptr(), Qd.data_ptr(), cs.cs.data_ptr(),
+                                                  cs.cs.data_ptr(), plan.host_ptr, plan.device.data_ptr(), n, m, r,
+                                                  cs.range, 0.9, cs.a, cs.b, 0)
+        assert rc == 0
+        low = to_np(Md)
+        assert_close(low, oracle.pqt(P, Q), what="PQt %s" % ((n, m, r),))
+        ocs.update(MQ - low, 0.9)         # the residual against the low-rank product the GPU wrote
+        np.testing.assert_array_equal(to_np(cs.cs), ocs.cs)
 
 
 def psgd_check_factory(st, ost, mode):

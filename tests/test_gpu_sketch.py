@@ -1,7 +1,7 @@
 """GPU parity of the count-sketch kernels against the CPU oracle, through the C-ABI library
 (ctypes) and the product classes that wrap it.  Buckets, signs and query results must be bit
-exact; update results are compared at 1e-5 relative because the reference accumulates with float
-atomics in no fixed order."""
+exact.  Updates on a plan add in the oracle's order and must be bit exact too; updates without a
+plan (float atomics in no fixed order, as in the reference) are compared at 1e-5 relative."""
 import ctypes
 
 import numpy as np
@@ -180,16 +180,18 @@ def test_rejects_host_tensors():
 
 # ---- long rows: the planned (atomic-free) path is deterministic and follows the oracle's order ----
 
-PLANNED_SHAPES = [(5, 40_003, 0.1), (5, 100_000, 0.1), (2, 65_537, 0.5), (3, 8191, 1.0), (1, 300_001, 0.05),
-                  (8, 20_000, 0.9)]
+PLANNED_SHAPES = [  # (n, d, sketch_size, kind): 0 = binned long rows, 1 = row lists
+    (5, 40_003, 0.1, 0), (5, 100_000, 0.1, 0), (2, 65_537, 0.5, 0), (1, 300_001, 0.05, 0), (8, 30_000, 0.9, 0),
+    (8, 20_000, 0.9, 0), (3, 8191, 1.0, 1), (8, 20_000, 0.3, 1), (1, 1, 0.5, 1), (3, 17, 0.3, 1), (64, 576, 0.2, 1), (40, 5760, 0.2, 1),
+    (2100, 650, 0.1, 1), (4099, 1024, 0.1, 1), (7, 24_576, 0.05, 1), (33, 1023, 2.0, 1), (20_000, 66, 0.1, 1)]
 
 
-@pytest.mark.parametrize("n,d,ss", PLANNED_SHAPES)
-def test_planned_update_bit_exact(oracle, n, d, ss):
+@pytest.mark.parametrize("n,d,ss,kind", PLANNED_SHAPES)
+def test_planned_update_bit_exact(oracle, n, d, ss, kind):
     from conef_amd.compressors.CountSketch import DenseCS
     rng = np.random.RandomState(d)
     cs = DenseCS(n, d, ss)
-    assert cs.plan() is not None
+    assert cs.plan() is not None and cs.plan().kind == kind
     o = oracle.DenseCS(n, d, ss)
     for step in range(3):
         v = (rng.randn(n, d) * 1e-3).astype(np.float32)
@@ -213,6 +215,36 @@ def test_planned_update_any_tiling(oracle, monkeypatch, chunk, tbin):
         cs.update(dev(v), 0.9)
         o.update(v, 0.9)
     np.testing.assert_array_equal(to_np(cs.cs), o.cs)
+
+
+@pytest.mark.parametrize("n,d,ss", [(3, 17, 0.3), (64, 576, 0.2), (2100, 650, 0.1), (40, 5760, 0.2)])
+def test_unplanned_row_kernels_still_match(oracle, monkeypatch, n, d, ss):
+    """The entry points that take no plan (one wavefront per row, LDS atomics) stay in the library."""
+    from conef_amd.compressors.CountSketch import DenseCS
+    monkeypatch.setenv("CONEF_PLAN", "0")
+    cs = DenseCS(n, d, ss)
+    assert cs.plan() is None
+    o = oracle.DenseCS(n, d, ss)
+    rng = np.random.RandomState(n)
+    for _ in range(2):
+        v = (rng.randn(n, d) * 1e-3).astype(np.float32)
+        cs.update(dev(v), 0.9)
+        o.update(v, 0.9)
+        assert_close(cs.cs, o.cs, what="row kernel without a plan")
+
+
+@pytest.mark.parametrize("n,d,ss", [(3, 17, 0.3), (64, 576, 0.2), (2100, 650, 0.1)])
+def test_half_sketch_on_a_plan_bit_exact(oracle, n, d, ss):
+    from conef_amd.compressors.halfCountSketch import DenseCS as HalfCS
+    cs = HalfCS(n, d, ss)
+    assert cs.plan() is not None
+    o = oracle.HalfDenseCS(n, d, ss)
+    rng = np.random.RandomState(d)
+    for _ in range(3):
+        v = (rng.randn(n, d) * 1e-2).astype(np.float32)
+        cs.update(dev(v), 0.9)
+        o.update(v, 0.9)
+        np.testing.assert_array_equal(to_np(cs.cs), o.cs)
 
 
 def test_atomic_fallback_still_matches(oracle, monkeypatch):

@@ -1,4 +1,5 @@
-"""CPU-only check of the accumulation plan the long-row sketch kernels run on.
+"""CPU-only check of the accumulation plans the sketch kernels run on (binned plans for long
+rows first, row-list plans at the end).
 
 The two GPU passes are replayed here in numpy, reading only the plan's tables: pass A permutes
 each chunk's records into its image, pass B collects a bin's segments and adds every bucket's
@@ -67,7 +68,7 @@ def replay(h, vec, cs, beta, oracle):
 
 
 @pytest.mark.parametrize("n,d,w,chunk,tbin", [(5, 9000, 900, 1024, 64), (1, 5000, 5000, 2048, 128),
-                                              (8, 3001, 77, 1024, 64), (3, 12345, 4000, 0, 0)])
+                                              (8, 3001, 77, 1024, 64), (3, 30011, 4000, 0, 0)])
 def test_plan_replay_matches_oracle_bit_for_bit(oracle, n, d, w, chunk, tbin):
     rng = np.random.RandomState(d)
     h = build_plan(n, d, w, chunk, tbin)
@@ -95,10 +96,53 @@ def test_plan_tables_are_consistent(oracle):
     np.testing.assert_array_equal(h["ent"] >> 15, (sign[order] > 0).astype(np.uint16))
 
 
+def build_rowlist(n, d, w):
+    from conef_amd import _lib
+    lib = _lib.load()
+    nb = lib.conef_plan_bytes(n, d, w, 0, 0)
+    assert nb > 0
+    buf = np.zeros(nb, np.uint8)
+    assert lib.conef_plan_build_host(buf.ctypes.data, nb, n, d, w, A, B, 0, 0) == 0
+    assert lib.conef_plan_kind(buf.ctypes.data) == 1
+    assert lib.conef_plan_workspace_bytes(buf.ctypes.data) == 0
+    i64 = buf[:128].view(np.int64)
+    csr = buf[int(i64[9]):int(i64[9]) + 4 * (w + 1)].view(np.uint32)
+    ent = buf[int(i64[10]):int(i64[10]) + 2 * d].view(np.uint16)
+    pk = buf[int(i64[11]):int(i64[11]) + 4 * d].view(np.uint32)
+    return csr, ent, pk
+
+
+@pytest.mark.parametrize("n,d,w", [(3, 17, 5), (40, 5760, 1152), (7, 24576, 100), (100, 650, 65), (2, 100, 300)])
+def test_rowlist_plan_replay_matches_oracle_bit_for_bit(oracle, n, d, w):
+    """Walking the per-bucket column lists the way the kernel does reproduces the oracle's update."""
+    csr, ent, pk = build_rowlist(n, d, w)
+    bucket, sign = oracle.hash_table(d, w)
+    np.testing.assert_array_equal(pk & 0x7fffffff, bucket.astype(np.uint32))
+    np.testing.assert_array_equal(pk >> 31, (sign > 0).astype(np.uint32))
+    assert csr[0] == 0 and csr[-1] == d
+    rng = np.random.RandomState(d)
+    vec = rng.randn(n, d).astype(np.float32)
+    cs0 = rng.randn(n, w).astype(np.float32)
+    omb = 1.0 - float(np.float32(0.9))
+    got = cs0.copy()
+    for j in range(w):
+        cols = ent[csr[j]:csr[j + 1]].astype(np.int64)
+        assert (np.diff(cols & 0x7fff) > 0).all()                       # ascending columns
+        for en in cols:
+            s = 1.0 if en >> 15 else -1.0
+            term = (s * vec[:, en & 0x7fff].astype(np.float64) - omb * cs0[:, j].astype(np.float64)).astype(np.float32)
+            got[:, j] = got[:, j] + term
+    want = cs0.copy()
+    oracle.cs_update(vec, want, 0.9)
+    np.testing.assert_array_equal(got, want)
+
+
 def test_plan_argument_checks():
     from conef_amd import _lib
     lib = _lib.load()
-    assert lib.conef_plan_bytes(9, 1000, 100, 0, 0) == 0          # more than 8 rows: not applicable
+    assert lib.conef_plan_bytes(9, 100_000, 100, 0, 0) == 0       # long rows and more than 8 of them: no plan
+    assert lib.conef_plan_bytes(9, 1000, 100, 0, 0) > 0           # short rows: row lists, any number of rows
+    assert lib.conef_plan_bytes(9, 1000, 100, 1024, 64) == 0      # a binned plan was asked for
     assert lib.conef_plan_bytes(0, 1000, 100, 0, 0) == -1
     buf = np.zeros(64, np.uint8)
     assert lib.conef_plan_build_host(buf.ctypes.data, 64, 5, 1000, 100, A, B, 0, 0) == -1   # buffer too small
