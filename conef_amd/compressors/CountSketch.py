@@ -80,7 +80,12 @@ class DenseCS:
             chunk = int(os.environ.get("CONEF_PLAN_CHUNK", "0"))
             tbin = int(os.environ.get("CONEF_PLAN_BIN", "0"))
             if SketchPlan.applicable(self.N, self.D, self.range, chunk, tbin):
-                self._plan = SketchPlan(self.N, self.D, self.range, self.a, self.b, self.cs.device, chunk, tbin)
+                try:
+                    self._plan = SketchPlan(self.N, self.D, self.range, self.a, self.b, self.cs.device, chunk, tbin)
+                except ValueError:       # e.g. one bucket collects more columns than a bin image can hold
+                    self._plan = False
+        if self._plan is False:
+            return None
         if self._plan is not None and self._plan.key != (self.N, self.D, self.range, self.a, self.b):
             self._plan = None
             return self.plan()

@@ -108,9 +108,22 @@ __device__ __forceinline__ int64_t conef_payload_pos(int64_t flat, ConefBlock b)
 }
 
 // ------------------------------------------------------------ wave helpers ----
+// Butterfly sum over the 64 lanes; every lane ends with the total.  The four steps inside a row
+// of 16 lanes are DPP operands of the adds (vector ALU), only the last two cross rows and go
+// through the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float conef_dpp(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+
 __device__ __forceinline__ float conef_wave_sum(float v)
 {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    v += conef_dpp<0xB1>(v);    // quad_perm [1,0,3,2]: lane ^ 1
+    v += conef_dpp<0x4E>(v);    // quad_perm [2,3,0,1]: lane ^ 2
+    v += conef_dpp<0x141>(v);   // row_half_mirror: the other quad of the 8
+    v += conef_dpp<0x140>(v);   // row_mirror: the other half of the 16
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
     return v;
 }

@@ -99,9 +99,9 @@ inline bool conef_plan_shape(int64_t n, int64_t d, int32_t w, int32_t hint_chunk
         // buckets = records * w / d
         double records = 52.0 * 1024 / (4.0 * n);
         t = (int64_t)(records * (double)w / (double)d);
-        t = t / 64 * 64;
+        if (t >= 64) t = t / 64 * 64;      // narrow sketches: fewer buckets than lanes per bin rather than an image that overflows LDS
     }
-    if (t < 64) t = 64;
+    if (t < 1) t = 1;
     if (t > 768) t = 768;      // leaves room in a 1024-thread workgroup for the waves that do column work
     h->magic = kConefPlanMagic;
     h->version = 1;

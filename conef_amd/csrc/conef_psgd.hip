@@ -68,45 +68,62 @@ psgd_mq_kernel(float* __restrict__ x, const float* __restrict__ err, const float
 
     if (FAST) {
         const int m4 = m >> 2;
-        for (int j = threadIdx.x; j < m4; j += 256) {
-            float xv[RB][4];
+        constexpr int U = (RB * RP <= 16) ? 4 : 2;      // column quads in flight per thread
+        for (int j0 = threadIdx.x; j0 < m4; j0 += U * 256) {
+            float xv[U][RB][4];
+            float qf[U][4 * RP];                        // Q rows 4j..4j+3: 4*RP consecutive floats
+            float ev[U][RB][4];
+            uint32_t pk[U][4];
 #pragma unroll
-            for (int a = 0; a < RB; ++a) ld4(x + rowc[a] * m + 4 * j, xv[a]);
-            float qf[4 * RP];               // Q rows 4j..4j+3: 4*RP consecutive floats
+            for (int u = 0; u < U; ++u) {               // past the last quad: a valid address, result unused
+                const int j = j0 + u * 256 < m4 ? j0 + u * 256 : m4 - 1;
 #pragma unroll
-            for (int t = 0; t < RP; ++t) ld4(q + (int64_t)j * 4 * RP + 4 * t, qf + 4 * t);
-            if (MODE == 1) {
+                for (int a = 0; a < RB; ++a) ld4(x + rowc[a] * m + 4 * j, xv[u][a]);
 #pragma unroll
-                for (int a = 0; a < RB; ++a) {
-                    float ev[4];
-                    ld4(err + rowc[a] * m + 4 * j, ev);
+                for (int t = 0; t < RP; ++t) ld4(q + (int64_t)j * 4 * RP + 4 * t, qf[u] + 4 * t);
+                if (MODE == 1) {
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) xv[a][k] = __fadd_rn(xv[a][k], ev[k]);
-                    if (row0 + a < n) st4(x + rowc[a] * m + 4 * j, xv[a]);
+                    for (int a = 0; a < RB; ++a) ld4(err + rowc[a] * m + 4 * j, ev[u][a]);
                 }
-            } else if (MODE == 2) {
-                uint32_t pk[4];
-                if (pktab) {
-                    uint4 t = reinterpret_cast<const uint4*>(pktab)[j];
-                    pk[0] = t.x; pk[1] = t.y; pk[2] = t.z; pk[3] = t.w;
-                } else {
+                if (MODE == 2) {
+                    if (pktab) {
+                        uint4 t = reinterpret_cast<const uint4*>(pktab)[j];
+                        pk[u][0] = t.x; pk[u][1] = t.y; pk[u][2] = t.z; pk[u][3] = t.w;
+                    } else {
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) pk[k] = conef_bucket_sign(4 * j + k, mod, hs.a, hs.b, hs.sa, hs.sb);
-                }
-#pragma unroll
-                for (int a = 0; a < RB; ++a) {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k)
-                        xv[a][k] = __fadd_rn(xv[a][k], conef_query_term(cells[a * w + (pk[k] & 0x7fffffffu)], pk[k], alpha));
-                    if (row0 + a < n) st4(x + rowc[a] * m + 4 * j, xv[a]);
+                        for (int k = 0; k < 4; ++k)
+                            pk[u][k] = conef_bucket_sign(4 * j + k, mod, hs.a, hs.b, hs.sa, hs.sb);
+                    }
                 }
             }
 #pragma unroll
-            for (int k = 0; k < 4; ++k)
+            for (int u = 0; u < U; ++u) {
+                const int j = j0 + u * 256;
+                if (j >= m4) break;
+                if (MODE == 1) {
 #pragma unroll
-                for (int a = 0; a < RB; ++a)
+                    for (int a = 0; a < RB; ++a) {
 #pragma unroll
-                    for (int c = 0; c < RP; ++c) acc[a][c] = fmaf(xv[a][k], qf[k * RP + c], acc[a][c]);
+                        for (int k = 0; k < 4; ++k) xv[u][a][k] = __fadd_rn(xv[u][a][k], ev[u][a][k]);
+                        if (row0 + a < n) st4(x + rowc[a] * m + 4 * j, xv[u][a]);
+                    }
+                } else if (MODE == 2) {
+#pragma unroll
+                    for (int a = 0; a < RB; ++a) {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                            xv[u][a][k] = __fadd_rn(xv[u][a][k], conef_query_term(cells[a * w + (pk[u][k] & 0x7fffffffu)],
+                                                                                   pk[u][k], alpha));
+                        if (row0 + a < n) st4(x + rowc[a] * m + 4 * j, xv[u][a]);
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+#pragma unroll
+                    for (int a = 0; a < RB; ++a)
+#pragma unroll
+                        for (int c = 0; c < RP; ++c) acc[a][c] = fmaf(xv[u][a][k], qf[u][k * RP + c], acc[a][c]);
+            }
         }
     } else {
         for (int k = threadIdx.x; k < m; k += 256) {
@@ -169,7 +186,23 @@ psgd_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, float*
         for (int c = 0; c < RP; ++c) acc[k][c] = 0.f;
     if (FAST) {
         const int cc = c0 < m ? c0 : m - 4;         // clamped: lanes past the edge load a valid quad, results unused
-        for (int64_t i = i0 + wave; i < i1; i += kMtpWaves) {
+        int64_t i = i0 + wave;
+        for (; i + 3 * kMtpWaves < i1; i += 4 * kMtpWaves) {      // four rows in flight
+            float xv[4][4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) ld4(x + (i + u * kMtpWaves) * m + cc, xv[u]);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const float* pi = p + (i + u * kMtpWaves) * RP;
+#pragma unroll
+                for (int c = 0; c < RP; ++c) {
+                    float pc = pi[c];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) acc[k][c] = fmaf(xv[u][k], pc, acc[k][c]);
+                }
+            }
+        }
+        for (; i < i1; i += kMtpWaves) {
             float xv[4];
             ld4(x + i * m + cc, xv);
             const float* pi = p + i * RP;
@@ -259,24 +292,32 @@ psgd_pqt_kernel(float* __restrict__ x, float* __restrict__ err, const float* __r
         for (int k = 0; k < 4; ++k)
 #pragma unroll
             for (int c = 0; c < RP; ++c) qf[k][c] = flat[k * RP + c];
-        for (int64_t i = i0; i < i1; ++i) {
-            const float* pi = p + i * RP;
-            float mh[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int c = 0; c < RP; ++c) {
-                float pc = pi[c];
-#pragma unroll
-                for (int k = 0; k < 4; ++k) mh[k] = fmaf(pc, qf[k][c], mh[k]);
-            }
-            float* px = x + i * m + c0;
+        for (int64_t ib = i0; ib < i1; ib += 4) {          // four rows in flight
+            float xv[4][4];
             if (MODE == 1) {
-                float xv[4], ev[4];
-                ld4(px, xv);
 #pragma unroll
-                for (int k = 0; k < 4; ++k) ev[k] = __fsub_rn(xv[k], mh[k]);
-                st4(err + i * m + c0, ev);
+                for (int u = 0; u < 4; ++u) ld4(x + (ib + u < i1 ? ib + u : i1 - 1) * m + c0, xv[u]);
             }
-            st4(px, mh);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int64_t i = ib + u;
+                if (i >= i1) break;
+                const float* pi = p + i * RP;
+                float mh[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < RP; ++c) {
+                    float pc = pi[c];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) mh[k] = fmaf(pc, qf[k][c], mh[k]);
+                }
+                if (MODE == 1) {
+                    float ev[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) ev[k] = __fsub_rn(xv[u][k], mh[k]);
+                    st4(err + i * m + c0, ev);
+                }
+                st4(x + i * m + c0, mh);
+            }
         }
     } else {
         const int valid = m - c0 < 4 ? m - c0 : 4;
@@ -319,33 +360,45 @@ struct ListPsgdResidual {
             const int d4 = d >> 2, total4 = rows * d4;
             int row = threadIdx.x / d4, c4 = threadIdx.x - row * d4;
             const int srow = kConefRowlistThreads / d4, sc = kConefRowlistThreads - srow * d4;
-            for (int t = threadIdx.x; t < total4; t += kConefRowlistThreads) {
-                float xv[4], flat[4 * RP], pr[RP];
-                ld4(base + 4 * t, xv);
+            constexpr int U = RP <= 8 ? 4 : 2;         // quads in flight per thread
+            for (int t0 = threadIdx.x; t0 < total4; t0 += U * kConefRowlistThreads) {
+                float xv[U][4], flat[U][4 * RP], pr[U][RP];
 #pragma unroll
-                for (int u = 0; u < RP; ++u) ld4(q + (int64_t)c4 * 4 * RP + 4 * u, flat + 4 * u);
-                const float* pi = p + (row0 + row) * RP;
-                if (RP >= 4) {
+                for (int u = 0; u < U; ++u) {           // past the end: a valid address, result unused
+                    const bool in = t0 + u * kConefRowlistThreads < total4;
+                    const int t = in ? t0 + u * kConefRowlistThreads : total4 - 1;
+                    const int cq = in ? c4 : 0, rq = in ? row : 0;
+                    ld4(base + 4 * t, xv[u]);
 #pragma unroll
-                    for (int u = 0; u < RP / 4; ++u) ld4(pi + 4 * u, pr + 4 * u);
-                } else {
+                    for (int v = 0; v < RP; ++v) ld4(q + (int64_t)cq * 4 * RP + 4 * v, flat[u] + 4 * v);
+                    const float* pi = p + (row0 + rq) * RP;
+                    if (RP >= 4) {
 #pragma unroll
-                    for (int c = 0; c < RP; ++c) pr[c] = pi[c];
+                        for (int v = 0; v < RP / 4; ++v) ld4(pi + 4 * v, pr[u] + 4 * v);
+                    } else {
+#pragma unroll
+                        for (int c = 0; c < RP; ++c) pr[u][c] = pi[c];
+                    }
+                    row += srow;
+                    c4 += sc;
+                    if (c4 >= d4) {
+                        c4 -= d4;
+                        ++row;
+                    }
                 }
-                float mh[4] = {0.f, 0.f, 0.f, 0.f}, v[4];
 #pragma unroll
-                for (int c = 0; c < RP; ++c)
+                for (int u = 0; u < U; ++u) {
+                    const int t = t0 + u * kConefRowlistThreads;
+                    if (t >= total4) break;
+                    float mh[4] = {0.f, 0.f, 0.f, 0.f}, v[4];
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) mh[k] = fmaf(pr[c], flat[k * RP + c], mh[k]);
+                    for (int c = 0; c < RP; ++c)
 #pragma unroll
-                for (int k = 0; k < 4; ++k) v[k] = __fsub_rn(xv[k], mh[k]);
-                st4(base + 4 * t, mh);
-                st4(vals + 4 * t, v);
-                row += srow;
-                c4 += sc;
-                if (c4 >= d4) {
-                    c4 -= d4;
-                    ++row;
+                        for (int k = 0; k < 4; ++k) mh[k] = fmaf(pr[u][c], flat[u][k * RP + c], mh[k]);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) v[k] = __fsub_rn(xv[u][k], mh[k]);
+                    st4(base + 4 * t, mh);
+                    st4(vals + 4 * t, v);
                 }
             }
         } else {
@@ -572,7 +625,7 @@ int launch_mq(float* x, const float* err, const float* cs, const uint32_t* pktab
     // rows per workgroup: 4 amortises the Q traffic, but small matrices need the workgroups
     const int rp = rank_bound(r);
     int rb = rp >= 32 ? 2 : 4;
-    if (n / rb < 512) rb = rp >= 32 ? 2 : 1;
+    if (n / rb < 256) rb = rp >= 32 ? 2 : 1;
     size_t lds = (size_t)4 * rb * rp * 4 + (MODE == 2 ? (size_t)rb * w * 4 : 0);
     if (lds > 64 * 1024) return CONEF_ERR_INVALID;   // sketch rows wider than 16K cells per matrix row group
     dim3 grid((unsigned)((n + rb - 1) / rb));
@@ -602,14 +655,14 @@ struct MtpShape {
     int col_tiles, slabs, rows_per_slab;
 };
 
-// enough slabs for about a thousand workgroups, each wave at least two rows
+// enough slabs for about 256 workgroups of 8 waves, each wave at least eight rows
 inline MtpShape mtp_shape(int64_t n, int64_t m)
 {
     MtpShape g;
     g.col_tiles = (int)((m + 255) / 256);
-    int64_t slabs = (1024 + g.col_tiles - 1) / g.col_tiles;
+    int64_t slabs = (256 + g.col_tiles - 1) / g.col_tiles;
     int64_t rps = (n + slabs - 1) / slabs;
-    rps = (rps + 2 * kMtpWaves - 1) / (2 * kMtpWaves) * (2 * kMtpWaves);
+    rps = (rps + 8 * kMtpWaves - 1) / (8 * kMtpWaves) * (8 * kMtpWaves);
     g.rows_per_slab = (int)rps;
     g.slabs = (int)((n + rps - 1) / rps);
     return g;

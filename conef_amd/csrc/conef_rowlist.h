@@ -4,6 +4,7 @@
 // scatters the same way.  A plan built once per sketch lists, per bucket, the columns that fall
 // into it (ascending).  A workgroup then takes a tile of `rb` consecutive rows:
 //
+//   (the bucket lists and their offsets are copied into LDS first: d + w small integers)
 //   stage   the values to be sketched are produced in column order with 16-byte accesses and
 //           parked in LDS; whatever the fused step has to do in column order (payload, writing
 //           the decompressed gradient, the low-rank product) happens here;
@@ -20,7 +21,7 @@
 
 constexpr int kConefRowlistThreads = 256;
 constexpr int64_t kConefRowlistMaxCols = 24576;       // 4 B value + 2 B list entry per column in LDS
-constexpr size_t kConefRowlistLdsLimit = 152 * 1024;
+constexpr size_t kConefRowlistLdsLimit = 160 * 1024;   // LDS of a gfx950 CU
 
 struct ConefRowlistView {
     const uint32_t* csr;   // [w+1] first list entry of bucket j
@@ -38,7 +39,8 @@ inline size_t conef_rowlist_lds(int rb, int64_t d, int32_t w, bool cells)
 {
     size_t vals = (((size_t)rb * d + 3) & ~(size_t)3) * 4;
     size_t ent = (((size_t)d + 7) & ~(size_t)7) * 2;
-    return vals + ent + (cells ? (size_t)rb * w * 4 : 0);
+    size_t csr = (((size_t)w + 1 + 3) & ~(size_t)3) * 4;
+    return vals + ent + csr + (cells ? (size_t)rb * w * 4 : 0);
 }
 
 // Rows per tile: about 32 KB of values (several tiles per CU), but no more than leaves a
@@ -74,10 +76,35 @@ struct ConefListVec {
         const float* base = vec + row0 * d;
         const int total = rows * d;
         if (vec_ok) {
-            for (int q = threadIdx.x; q < (total >> 2); q += kConefRowlistThreads)
-                reinterpret_cast<float4*>(vals)[q] = reinterpret_cast<const float4*>(base)[q];
+            // eight loads in flight per thread; indices past the end are clamped, not branched around
+            const int total4 = total >> 2;
+            for (int q0 = threadIdx.x; q0 < total4; q0 += 8 * kConefRowlistThreads) {
+                float4 t[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    int q = q0 + u * kConefRowlistThreads;
+                    t[u] = reinterpret_cast<const float4*>(base)[q < total4 ? q : total4 - 1];
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    int q = q0 + u * kConefRowlistThreads;
+                    if (q < total4) reinterpret_cast<float4*>(vals)[q] = t[u];
+                }
+            }
         } else {
-            for (int e = threadIdx.x; e < total; e += kConefRowlistThreads) vals[e] = base[e];
+            for (int e0 = threadIdx.x; e0 < total; e0 += 8 * kConefRowlistThreads) {
+                float t[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    int e = e0 + u * kConefRowlistThreads;
+                    t[u] = base[e < total ? e : total - 1];
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    int e = e0 + u * kConefRowlistThreads;
+                    if (e < total) vals[e] = t[u];
+                }
+            }
         }
     }
 };
@@ -115,33 +142,47 @@ struct ConefListRandBlock {
             const int d4 = d >> 2, total4 = rows * d4;
             int row = threadIdx.x / d4, c4 = threadIdx.x - row * d4;
             const int srow = kConefRowlistThreads / d4, sc = kConefRowlistThreads - srow * d4;
-            for (int q = threadIdx.x; q < total4; q += kConefRowlistThreads) {
-                float4 g = reinterpret_cast<const float4*>(base)[q];
-                uint4 p = reinterpret_cast<const uint4*>(pk)[c4];
-                const float* cr = cells + row * w;
-                float c0 = cr[p.x & 0x7fffffffu], c1 = cr[p.y & 0x7fffffffu];
-                float c2 = cr[p.z & 0x7fffffffu], c3 = cr[p.w & 0x7fffffffu];
-                int64_t f = f0 + ((int64_t)q << 2);
-                float4 o, v;
-                if ((f < blk.end && f + 4 > blk.start) || f < blk.rest) {
-                    v.x = finish(f, g.x, c0, p.x, &o.x);
-                    v.y = finish(f + 1, g.y, c1, p.y, &o.y);
-                    v.z = finish(f + 2, g.z, c2, p.z, &o.z);
-                    v.w = finish(f + 3, g.w, c3, p.w, &o.w);
-                } else {      // the block is one wrap-around range: most quads are entirely outside it
-                    o = make_float4(0.f, 0.f, 0.f, 0.f);
-                    v.x = __fadd_rn(g.x, conef_query_term(c0, p.x, alpha));
-                    v.y = __fadd_rn(g.y, conef_query_term(c1, p.y, alpha));
-                    v.z = __fadd_rn(g.z, conef_query_term(c2, p.z, alpha));
-                    v.w = __fadd_rn(g.w, conef_query_term(c3, p.w, alpha));
+            for (int q0 = threadIdx.x; q0 < total4; q0 += 4 * kConefRowlistThreads) {
+                float4 g[4];
+                uint4 p[4];
+                int rw[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {      // four quads in flight; past the end: a valid address, result unused
+                    int q = q0 + u * kConefRowlistThreads;
+                    bool in = q < total4;
+                    g[u] = reinterpret_cast<const float4*>(base)[in ? q : total4 - 1];
+                    p[u] = reinterpret_cast<const uint4*>(pk)[in ? c4 : 0];
+                    rw[u] = in ? row : 0;
+                    row += srow;
+                    c4 += sc;
+                    if (c4 >= d4) {
+                        c4 -= d4;
+                        ++row;
+                    }
                 }
-                reinterpret_cast<float4*>(base)[q] = o;
-                reinterpret_cast<float4*>(vals)[q] = v;
-                row += srow;
-                c4 += sc;
-                if (c4 >= d4) {
-                    c4 -= d4;
-                    ++row;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    int q = q0 + u * kConefRowlistThreads;
+                    if (q >= total4) break;
+                    const float* cr = cells + rw[u] * w;
+                    float c0 = cr[p[u].x & 0x7fffffffu], c1 = cr[p[u].y & 0x7fffffffu];
+                    float c2 = cr[p[u].z & 0x7fffffffu], c3 = cr[p[u].w & 0x7fffffffu];
+                    int64_t f = f0 + ((int64_t)q << 2);
+                    float4 o, v;
+                    if ((f < blk.end && f + 4 > blk.start) || f < blk.rest) {
+                        v.x = finish(f, g[u].x, c0, p[u].x, &o.x);
+                        v.y = finish(f + 1, g[u].y, c1, p[u].y, &o.y);
+                        v.z = finish(f + 2, g[u].z, c2, p[u].z, &o.z);
+                        v.w = finish(f + 3, g[u].w, c3, p[u].w, &o.w);
+                    } else {      // the block is one wrap-around range: most quads are entirely outside it
+                        o = make_float4(0.f, 0.f, 0.f, 0.f);
+                        v.x = __fadd_rn(g[u].x, conef_query_term(c0, p[u].x, alpha));
+                        v.y = __fadd_rn(g[u].y, conef_query_term(c1, p[u].y, alpha));
+                        v.z = __fadd_rn(g[u].z, conef_query_term(c2, p[u].z, alpha));
+                        v.w = __fadd_rn(g[u].w, conef_query_term(c3, p[u].w, alpha));
+                    }
+                    reinterpret_cast<float4*>(base)[q] = o;
+                    reinterpret_cast<float4*>(vals)[q] = v;
                 }
             }
         } else {
@@ -165,6 +206,24 @@ struct ConefListRandBlock {
 };
 
 // ------------------------------------------------------------------ kernel ----
+// count >= 1 words from global memory to LDS, eight loads in flight per thread
+__device__ __forceinline__ void conef_copy_words_to_lds(uint32_t* dst, const uint32_t* __restrict__ src, int count)
+{
+    for (int i0 = threadIdx.x; i0 < count; i0 += 8 * kConefRowlistThreads) {
+        uint32_t t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            int i = i0 + u * kConefRowlistThreads;
+            t[u] = src[i < count ? i : count - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            int i = i0 + u * kConefRowlistThreads;
+            if (i < count) dst[i] = t[u];
+        }
+    }
+}
+
 template <typename CsT, typename Front>
 __global__ void __launch_bounds__(kConefRowlistThreads)
 conef_rowlist_kernel(Front front, ConefRowlistView plan, const CsT* cs_in, CsT* cs_out, int64_t n, int d, int w,
@@ -173,16 +232,30 @@ conef_rowlist_kernel(Front front, ConefRowlistView plan, const CsT* cs_in, CsT* 
     extern __shared__ float conef_rl[];
     float* vals = conef_rl;
     uint16_t* ent_l = reinterpret_cast<uint16_t*>(vals + ((rb * d + 3) & ~3));
-    float* cells = reinterpret_cast<float*>(ent_l + ((d + 7) & ~7));
+    uint32_t* csr_l = reinterpret_cast<uint32_t*>(ent_l + ((d + 7) & ~7));
+    float* cells = reinterpret_cast<float*>(csr_l + ((w + 1 + 3) & ~3));
     const int64_t row0 = (int64_t)blockIdx.x * rb;
     const int rows = n - row0 < rb ? (int)(n - row0) : rb;
 
     // the bucket lists, two entries per load (the table is padded to a multiple of 256 bytes)
-    for (int i = threadIdx.x; i < ((d + 1) >> 1); i += kConefRowlistThreads)
-        reinterpret_cast<uint32_t*>(ent_l)[i] = reinterpret_cast<const uint32_t*>(plan.ent)[i];
+    conef_copy_words_to_lds(reinterpret_cast<uint32_t*>(ent_l), reinterpret_cast<const uint32_t*>(plan.ent), (d + 1) >> 1);
+    conef_copy_words_to_lds(csr_l, plan.csr, w + 1);
     if (Front::kNeedsCells) {
         const CsT* src = cs_in + row0 * w;
-        for (int i = threadIdx.x; i < rows * w; i += kConefRowlistThreads) cells[i] = conef_ld(src + i);
+        const int count = rows * w;
+        for (int i0 = threadIdx.x; i0 < count; i0 += 4 * kConefRowlistThreads) {
+            float t[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                int i = i0 + u * kConefRowlistThreads;
+                t[u] = conef_ld(src + (i < count ? i : count - 1));
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                int i = i0 + u * kConefRowlistThreads;
+                if (i < count) cells[i] = t[u];
+            }
+        }
         __syncthreads();
     }
     front.stage(row0, rows, d, w, vals, cells, plan.pk);
@@ -192,7 +265,7 @@ conef_rowlist_kernel(Front front, ConefRowlistView plan, const CsT* cs_in, CsT* 
     int row = threadIdx.x / w, j = threadIdx.x - row * w;
     const int srow = kConefRowlistThreads / w, sj = kConefRowlistThreads - srow * w;
     for (int p = threadIdx.x; p < total; p += kConefRowlistThreads) {
-        const uint32_t e0 = plan.csr[j], e1 = plan.csr[j + 1];
+        const uint32_t e0 = csr_l[j], e1 = csr_l[j + 1];
         const int64_t cell = (row0 + row) * w + j;
         const float aux = Front::kNeedsCells ? cells[row * w + j] : conef_ld(cs_in + cell);
         const double decay = __dmul_rn(one_minus_beta, (double)aux);

@@ -137,6 +137,20 @@ def test_rowlist_plan_replay_matches_oracle_bit_for_bit(oracle, n, d, w):
     np.testing.assert_array_equal(got, want)
 
 
+@pytest.mark.parametrize("n,d,w,kind", [(5, 1_300_000, 130_000, 0), (640, 5760, 1152, 1), (33278, 650, 65, 1),
+                                        (7, 24_576, 1228, 1), (8, 20_000, 1000, 1), (8, 20_000, 18_000, 0),
+                                        (8, 30_000, 27_000, 0), (1, 1, 1, 1), (3, 8191, 8191, 1), (20_000, 66, 6, 1),
+                                        (5, 24_577, 100, 0), (33, 1023, 2046, 1)])
+def test_which_kind_of_plan_a_shape_gets(n, d, w, kind):
+    from conef_amd import _lib
+    lib = _lib.load()
+    nb = lib.conef_plan_bytes(n, d, w, 0, 0)
+    assert nb > 0
+    buf = np.zeros(nb, np.uint8)
+    assert lib.conef_plan_build_host(buf.ctypes.data, nb, n, d, w, A, B, 0, 0) == 0
+    assert lib.conef_plan_kind(buf.ctypes.data) == kind
+
+
 def test_plan_argument_checks():
     from conef_amd import _lib
     lib = _lib.load()
