@@ -99,7 +99,7 @@ def _block_size(state, numel):
     return max(1, int(state.compression_ratio * numel))      # RandomBlock_hook.py:207,216
 
 
-def RandomBlock_hook(state: RandomBlockState, bucket) -> torch.futures.Future:
+def RandomBlock_hook(state: RandomBlockState, bucket) -> torch.futures.Future[torch.Tensor]:
     group, world_size = _bucket.group_and_size(state.process_group)
     input_tensor = _bucket.buffer(bucket)
 

@@ -56,7 +56,7 @@ class UnbiasedRandomBlockState(object):
             logging.info("Start to apply PowerSGD after {} iterations.".format(self.iter))
 
 
-def UnbiasedRandomBlock_hook(state: UnbiasedRandomBlockState, bucket) -> torch.futures.Future:
+def UnbiasedRandomBlock_hook(state: UnbiasedRandomBlockState, bucket) -> torch.futures.Future[torch.Tensor]:
     group, world_size = _bucket.group_and_size(state.process_group)
     input_tensor = _bucket.buffer(bucket)
 

@@ -51,6 +51,19 @@ def _workspace(device, stream, nbytes):
     return ws
 
 
+_SCRATCH = {}
+
+
+def _scratch_f32(device, stream, numel):
+    """fp32 scratch for a residual that only lives between two launches on ``stream``."""
+    key = (device, stream)
+    buf = _SCRATCH.get(key)
+    if buf is None or buf.numel() < numel:
+        buf = torch.empty(numel, dtype=torch.float32, device=device)
+        _SCRATCH[key] = buf
+    return buf
+
+
 def topk_sparsify(err, topk_ratio, workspace=None):
     """Keeps the max(1, int(0.5 * ratio * numel)) largest magnitudes of ``err`` in place
     (hPowerSGD_hook.py:90-97); ties on the threshold keep the lowest flat indices."""
@@ -69,7 +82,8 @@ def topk_sparsify(err, topk_ratio, workspace=None):
 
 def run_round(state, bucket, error_mode):
     """One hook call.  error_mode: None | 'ef' (dense, whole bucket) | 'conef' (count sketch per
-    matrix) | 'topk' (dense per matrix, magnitude-sparsified)."""
+    matrix) | 'conef_v2' (count sketch over the [m,n] re-view of each matrix's memory,
+    powerSGD_hook.py:918-920,1074-1076) | 'topk' (dense per matrix, magnitude-sparsified)."""
     group, world_size = _bucket.group_and_size(state.process_group)
     input_tensor = _bucket.buffer(bucket)
 
@@ -95,7 +109,7 @@ def run_round(state, bucket, error_mode):
             logging.info("A zero tensor of length {} that represents local error is created.".format(total_length))
             state.error_dict[bucket_index] = torch.zeros(total_length, device=device, dtype=dtype)
         dense_err = state.error_dict[bucket_index]
-    elif error_mode in ("conef", "topk"):
+    elif error_mode in ("conef", "conef_v2", "topk"):
         state.error_dict.setdefault(bucket_index, {})
 
     # Step I: which tensors are worth compressing (:394-418)
@@ -148,7 +162,10 @@ def run_round(state, bucket, error_mode):
         rc = lib.conef_gram_schmidt_f32(q.data_ptr(), q.shape[0], q.shape[1], eps, ws_ptr, ws_len, stream)
         _lib.check(rc, "conef_gram_schmidt_f32")
 
-    alpha = 1 - state.beta if error_mode == "conef" else 0.0
+    alpha = 1 - state.beta if error_mode in ("conef", "conef_v2") else 0.0
+    residual = None
+    if error_mode == "conef_v2" and work:
+        residual = _scratch_f32(device, stream, max(n * m for _, n, m, _ in work))
     errs = state.error_dict.get(bucket_index)
 
     # pass 1: error add fused into P = M Q
@@ -170,6 +187,13 @@ def run_round(state, bucket, error_mode):
             else:
                 rc = lib.conef_psgd_mq_conef_f32(matrix.data_ptr(), cs.cs.data_ptr(), q.data_ptr(), p.data_ptr(), n,
                                                  m, rank, cs.range, float(alpha), cs.a, cs.b, stream)
+        elif error_mode == "conef_v2":
+            # the sketch sees the same memory as m rows of n columns, so its rows are not the
+            # matrix rows: query as a pass of its own, then the plain product
+            if cnt not in errs:
+                errs[cnt] = DenseCS(m, n, state.sketch_size, device=device)
+            errs[cnt].query(matrix.view(m, n), alpha)
+            rc = lib.conef_psgd_mq_f32(matrix.data_ptr(), q.data_ptr(), p.data_ptr(), n, m, rank, stream)
         elif error_mode == "topk":
             if cnt not in errs:
                 errs[cnt] = torch.zeros_like(matrix)
@@ -217,6 +241,13 @@ def run_round(state, bucket, error_mode):
                                                   out.data_ptr(), n, m, rank, cs.range, float(state.beta), cs.a,
                                                   cs.b, stream)
                 cs.commit(out)
+        elif error_mode == "conef_v2":
+            res = residual[: n * m]
+            rc = lib.conef_psgd_pqt_ef_f32(matrix.data_ptr(), res.data_ptr(), p.data_ptr(), q.data_ptr(), n, m, rank,
+                                           stream)
+            _lib.check(rc, "conef_psgd_pqt_ef_f32")
+            errs[cnt].update(res.view(m, n), state.beta)
+            rc = 0
         elif error_mode == "topk":
             rc = lib.conef_psgd_pqt_ef_f32(matrix.data_ptr(), errs[cnt].data_ptr(), p.data_ptr(), q.data_ptr(), n, m,
                                            rank, stream)
@@ -231,5 +262,95 @@ def run_round(state, bucket, error_mode):
         state.p_memory_dict.clear()
         state.q_memory_dict.clear()
 
+    state.maybe_increase_iter(bucket)
+    return _bucket.completed_future(input_tensor)
+
+
+def run_batched_round(state, bucket):
+    """batched_powerSGD_hook (powerSGD_hook.py:583-787): the whole flat bucket, zero-padded to a
+    square [s,s] with s = ceil(sqrt(length)), is one matrix; dense error feedback over the padded
+    length; P and Q are [s, matrix_approximation_rank]."""
+    import math
+
+    group, world_size = _bucket.group_and_size(state.process_group)
+    input_tensor = _bucket.buffer(bucket)
+    if state.iter < state.start_powerSGD_iter:
+        state.maybe_increase_iter(bucket)
+        return _bucket.allreduce_fut(group, input_tensor, world_size)
+    if world_size != 1:
+        raise NotImplementedError(
+            "the MI355X PowerSGD hooks run the whole round on one GPU; with %d ranks the P and Q "
+            "all-reduces between the passes are not wired up" % world_size)
+    _lib.require_device_f32(input_tensor, "bucket buffer")
+    lib = _lib.load()
+    stream = _lib.stream_ptr(input_tensor)
+    device, dtype = input_tensor.device, input_tensor.dtype
+    bucket_index = _bucket.index(bucket)
+    total_length = input_tensor.shape[0]
+    side = math.isqrt(total_length)
+    if side * side < total_length:
+        side += 1
+    rank = state.matrix_approximation_rank
+    state.total_numel_before_compression += total_length
+    state.total_numel_after_compression += side * rank * 2
+    padded = side * side
+    if rank > side or rank > 32:
+        raise ValueError("matrix_approximation_rank %d does not fit a %d x %d matrix (at most 32)" % (rank, side, side))
+
+    # the bucket buffer cannot grow in place, so a padded bucket is worked on in a square buffer
+    if padded == total_length:
+        square = input_tensor
+    else:
+        square = state.batched_square_dict.get(bucket_index)
+        if square is None or square.numel() != padded:
+            square = torch.empty(padded, device=device, dtype=dtype)
+            state.batched_square_dict[bucket_index] = square
+        square[:total_length].copy_(input_tensor)
+        square[total_length:].zero_()
+
+    err = None
+    if state.use_error_feedback:
+        if bucket_index not in state.error_dict:
+            logging.info("A zero tensor of length {} that represents local error is created.".format(padded))
+            state.error_dict[bucket_index] = torch.zeros(padded, device=device, dtype=dtype)
+        err = state.error_dict[bucket_index]
+
+    if not state.warm_start or bucket_index not in state.p_memory_dict:
+        if state.warm_start:
+            logging.info("Initializing low-rank tensors P and Q, each of which has a shape of {} x {}.".format(
+                side, rank))
+        state.p_memory_dict[bucket_index] = torch.empty(side, rank, device=device, dtype=dtype)
+        with torch.random.fork_rng(devices=[]):
+            torch.manual_seed(state.rng.randint(1_000_000_000))
+            host_q = torch.randn(side, rank, device="cpu", dtype=dtype)
+        state.q_memory_dict[bucket_index] = host_q.to(device)
+    p, q = state.p_memory_dict[bucket_index], state.q_memory_dict[bucket_index]
+
+    eps = float(state.orthogonalization_epsilon)
+    ws = _workspace(device, stream, lib.conef_psgd_workspace_bytes(side, side, rank))
+    ws_ptr, ws_len = ws.data_ptr(), ws.numel()
+    _lib.check(lib.conef_gram_schmidt_f32(q.data_ptr(), side, rank, eps, ws_ptr, ws_len, stream),
+               "conef_gram_schmidt_f32")
+    if err is not None:
+        rc = lib.conef_psgd_mq_ef_f32(square.data_ptr(), err.data_ptr(), q.data_ptr(), p.data_ptr(), side, side, rank,
+                                      stream)
+    else:
+        rc = lib.conef_psgd_mq_f32(square.data_ptr(), q.data_ptr(), p.data_ptr(), side, side, rank, stream)
+    _lib.check(rc, "conef_psgd_mq")
+    _lib.check(lib.conef_gram_schmidt_f32(p.data_ptr(), side, rank, eps, ws_ptr, ws_len, stream),
+               "conef_gram_schmidt_f32")
+    _lib.check(lib.conef_psgd_mtp_f32(square.data_ptr(), p.data_ptr(), q.data_ptr(), side, side, rank, ws_ptr, ws_len,
+                                      stream), "conef_psgd_mtp_f32")
+    if err is not None:
+        rc = lib.conef_psgd_pqt_ef_f32(square.data_ptr(), err.data_ptr(), p.data_ptr(), q.data_ptr(), side, side, rank,
+                                       stream)
+    else:
+        rc = lib.conef_psgd_pqt_f32(square.data_ptr(), p.data_ptr(), q.data_ptr(), side, side, rank, stream)
+    _lib.check(rc, "conef_psgd_pqt")
+    if square is not input_tensor:
+        input_tensor.copy_(square[:total_length])
+    if not state.warm_start:
+        state.p_memory_dict.clear()
+        state.q_memory_dict.clear()
     state.maybe_increase_iter(bucket)
     return _bucket.completed_future(input_tensor)

@@ -105,7 +105,7 @@ class hPowerSGDState(object):
                     per_bucket.zero_()
 
 
-def hpowerSGD_hook(state: hPowerSGDState, bucket) -> torch.futures.Future:
+def hpowerSGD_hook(state: hPowerSGDState, bucket) -> torch.futures.Future[torch.Tensor]:
     if not state.use_error_feedback:
         mode = None
     else:

@@ -13,7 +13,7 @@ import torch
 
 from . import _bucket
 from ._psgd_engine import orthogonalize as _orthogonalize  # noqa: F401  (reference name, :12)
-from ._psgd_engine import run_round
+from ._psgd_engine import run_batched_round, run_round
 from ._psgd_engine import should_compress as _should_compress  # noqa: F401  (reference name, :46)
 
 
@@ -49,6 +49,7 @@ class PowerSGDState(object):
         "total_numel_after_compression",
         "compression_stats_logging_frequency",
         "next_stats_report",
+        "batched_square_dict",
     ]
 
     def __init__(
@@ -96,6 +97,7 @@ class PowerSGDState(object):
         self.use_error_compression = use_error_compression
         self.beta = beta
         self.sketch_size = sketch_size
+        self.batched_square_dict = {}    # batched_powerSGD_hook: the zero-padded square copy of a bucket
 
     def maybe_increase_iter(self, bucket):
         if _bucket.is_last(bucket):
@@ -123,5 +125,17 @@ def _error_mode(state):
     return "conef" if state.use_error_compression else "ef"
 
 
-def powerSGD_hook(state: PowerSGDState, bucket) -> torch.futures.Future:
+def powerSGD_hook(state: PowerSGDState, bucket) -> torch.futures.Future[torch.Tensor]:
     return run_round(state, bucket, _error_mode(state))
+
+
+def batched_powerSGD_hook(state: PowerSGDState, bucket) -> torch.futures.Future[torch.Tensor]:
+    """The whole bucket as one zero-padded square matrix, dense error feedback (reference :583-787)."""
+    return run_batched_round(state, bucket)
+
+
+def C2CS_hook_v2(state: PowerSGDState, bucket) -> torch.futures.Future[torch.Tensor]:
+    """powerSGD_hook whose count sketches are built over the [m,n] re-view of each [n,m] matrix's
+    memory: DenseCS(m, n, sketch_size) on matrix.view(m, n) (reference :791-1092)."""
+    mode = _error_mode(state)
+    return run_round(state, bucket, "conef_v2" if mode == "conef" else mode)

@@ -395,8 +395,10 @@ class UnbiasedRandomBlockOracle:
 class PowerSGDOracle:
     """powerSGD_hook.py:89-277 (state) and :280-580 (hook body) at world size 1.
     ``error_mode``: None (no EF), 'ef' (dense error over the whole bucket), 'conef' (count sketch
-    per compressed matrix), 'topk' (hPowerSGD_hook.py:393-400,549-554: dense per-matrix error,
-    sparsified by magnitude after each step)."""
+    per compressed matrix), 'conef_v2' (C2CS_hook_v2, :791-1092: the sketch is DenseCS(m, n) over
+    the [m,n] re-view of the matrix's memory, :918-920,1074-1076), 'topk'
+    (hPowerSGD_hook.py:393-400,549-554: dense per-matrix error, sparsified by magnitude after
+    each step)."""
 
     def __init__(self, matrix_approximation_rank=1, min_compression_rate=2, error_mode="ef", beta=0.9,
                  sketch_size=0.5, topk_ratio=0.4, warm_start=True, orthogonalization_epsilon=0,
@@ -421,7 +423,7 @@ class PowerSGDOracle:
             else:
                 self.error_dict[bucket_index] = np.zeros_like(flat)
             cp_flat = flat.copy()
-        elif self.error_mode in ("conef", "topk"):
+        elif self.error_mode in ("conef", "conef_v2", "topk"):
             self.error_dict.setdefault(bucket_index, {})
         mats, copies, ranks = [], [], []
         for t in split_bucket(flat, shapes):                          # :394-418
@@ -437,6 +439,11 @@ class PowerSGDOracle:
                     errs[cnt] = DenseCS(n, m, self.sketch_size)
                 errs[cnt].query(mat, 1 - self.beta)                   # :409
                 copies.append(mat.copy())                             # :410
+            elif self.error_mode == "conef_v2":
+                if cnt not in errs:
+                    errs[cnt] = DenseCS(m, n, self.sketch_size)       # :918
+                errs[cnt].query(mat.reshape(m, n), 1 - self.beta)     # :920 (a view of the same memory)
+                copies.append(mat.copy())
             elif self.error_mode == "topk":
                 if cnt not in errs:
                     errs[cnt] = np.zeros_like(mat)
@@ -475,6 +482,11 @@ class PowerSGDOracle:
             for cnt, (mat, cp) in enumerate(zip(mats, copies)):
                 cp -= mat                                             # :563
                 self.error_dict[bucket_index][cnt].update(cp, self.beta)   # :564
+        elif self.error_mode == "conef_v2":
+            for cnt, (mat, cp) in enumerate(zip(mats, copies)):
+                n, m = mat.shape
+                cp -= mat                                             # :1075
+                self.error_dict[bucket_index][cnt].update(cp.reshape(m, n), self.beta)   # :1076
         elif self.error_mode == "topk":
             for cnt, (mat, cp) in enumerate(zip(mats, copies)):
                 err = cp - mat                                        # hPowerSGD_hook.py:553
@@ -483,3 +495,55 @@ class PowerSGDOracle:
         if not self.warm_start:
             self.p_memory_dict.clear()
             self.q_memory_dict.clear()
+
+
+class BatchedPowerSGDOracle:
+    """batched_powerSGD_hook (powerSGD_hook.py:583-787) at world size 1: the flat bucket, padded
+    with zeros to a square of side ceil(sqrt(length)) (:657-663), is one matrix; dense error over
+    the padded length (:669-687); P, Q are [side, rank]; Q is orthogonalised on every call (:733)."""
+
+    def __init__(self, matrix_approximation_rank=1, use_error_feedback=True, warm_start=True,
+                 orthogonalization_epsilon=0, random_seed=0):
+        self.rank = matrix_approximation_rank
+        self.use_error_feedback, self.warm_start = use_error_feedback, warm_start
+        self.eps = orthogonalization_epsilon
+        self.rng = np.random.RandomState(random_seed)
+        self.error_dict, self.p_memory_dict, self.q_memory_dict = {}, {}, {}
+
+    def step(self, bucket_index, flat, shapes=None):
+        import math
+
+        import torch
+
+        total = flat.shape[0]
+        side = math.ceil(math.sqrt(total))
+        while side * side < total:          # guard against sqrt rounding on large lengths
+            side += 1
+        padded = np.zeros(side * side, dtype=np.float32)
+        padded[:total] = flat
+        cp = None
+        if self.use_error_feedback:
+            if bucket_index in self.error_dict:
+                padded += self.error_dict[bucket_index]
+            else:
+                self.error_dict[bucket_index] = np.zeros_like(padded)
+            cp = padded.copy()
+        mat = padded.reshape(side, side)
+        if not self.warm_start or bucket_index not in self.p_memory_dict:
+            self.p_memory_dict[bucket_index] = np.empty((side, self.rank), dtype=np.float32)
+            with torch.random.fork_rng(devices=[]):
+                torch.manual_seed(int(self.rng.randint(1_000_000_000)))
+                self.q_memory_dict[bucket_index] = torch.randn(side, self.rank, device="cpu",
+                                                               dtype=torch.float32).numpy().copy()
+        p, q = self.p_memory_dict[bucket_index], self.q_memory_dict[bucket_index]
+        gram_schmidt(q, self.eps)
+        p[...] = mq(mat, q)
+        gram_schmidt(p, self.eps)
+        q[...] = mtp(mat, p)
+        mat[...] = pqt(p, q)
+        if self.use_error_feedback:
+            self.error_dict[bucket_index] = cp - padded
+        if not self.warm_start:
+            self.p_memory_dict.clear()
+            self.q_memory_dict.clear()
+        flat[...] = padded[:total]

@@ -241,7 +241,7 @@ def psgd_check_factory(st, ost, mode):
             assert_close(q, oq, what="Q")
         if mode == "ef":
             assert_close(st.error_dict[0], ost.error_dict[0], what="dense error, step %d" % step)
-        elif mode == "conef":
+        elif mode in ("conef", "conef_v2"):
             for k in ost.error_dict[0]:
                 assert_close(st.error_dict[0][k].cs, ost.error_dict[0][k].cs, what="sketch %d step %d" % (k, step))
         elif mode == "topk":
@@ -282,6 +282,35 @@ def test_powersgd_hook_parity(oracle, shapes, rank, ss, mode):
     run_steps(powerSGD_hook, st, ost, shapes, 4, check=psgd_check_factory(st, ost, mode))
     rate, before, after = st.compression_stats()
     assert before == 4 * numel_of(shapes) and 0 < after < before and rate > 1
+
+
+@pytest.mark.parametrize("shapes,rank,ss", PSGD_CASES[:3])
+def test_c2cs_hook_v2_parity(oracle, shapes, rank, ss):
+    """The sketch lives on the [m,n] re-view of every compressed matrix's memory."""
+    from conef_amd.powerSGD_hook import C2CS_hook_v2, PowerSGDState
+    st = PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, use_error_compression=True,
+                       sketch_size=ss, beta=0.9)
+    ost = oracle.PowerSGDOracle(matrix_approximation_rank=rank, error_mode="conef_v2", sketch_size=ss, beta=0.9)
+    run_steps(C2CS_hook_v2, st, ost, shapes, 4, check=psgd_check_factory(st, ost, "conef_v2"))
+    for k, cs in st.error_dict[0].items():
+        assert (cs.N, cs.D) == (ost.error_dict[0][k].N, ost.error_dict[0][k].D)
+
+
+@pytest.mark.parametrize("total,rank,ef", [(64 * 64, 1, True), (5000, 2, True), (268_346, 1, True), (1000, 4, False),
+                                           (7, 1, True)])
+def test_batched_powersgd_hook_parity(oracle, total, rank, ef):
+    from conef_amd.powerSGD_hook import PowerSGDState, batched_powerSGD_hook
+    st = PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, use_error_feedback=ef)
+    ost = oracle.BatchedPowerSGDOracle(matrix_approximation_rank=rank, use_error_feedback=ef)
+
+    def check(step, gd, og):
+        assert_close(gd, og, what="batched: decompressed bucket, step %d" % step)
+        assert_close(st.p_memory_dict[0], ost.p_memory_dict[0], what="P")
+        assert_close(st.q_memory_dict[0], ost.q_memory_dict[0], what="Q")
+        if ef:
+            assert_close(st.error_dict[0], ost.error_dict[0], what="padded dense error, step %d" % step)
+
+    run_steps(batched_powerSGD_hook, st, ost, [(total,)], 4, check=check)
 
 
 def test_hpowersgd_topk_parity(oracle):
@@ -329,3 +358,37 @@ def test_powersgd_state_errors_and_warmup():
     powerSGD_hook(st, FakeGradBucket(g, [(64, 64)])).wait()
     assert st.iter == 4 and not torch.equal(g, ref)
     assert torch.linalg.matrix_rank(g.view(64, 64).cpu().double(), tol=1e-4) <= 2
+
+
+# ------------------------------------------------------- unbiased random matrix --
+
+def test_unbiased_mtrx_hook_parity(oracle):
+    """M <- (M Q) Q^T with Q drawn from the device generator under the seeds of RandomState(421)
+    (unbiasedMtrx_hook.py:41-45,231-232,292): the same draws, then the oracle's products."""
+    from conef_amd.unbiasedMtrx_hook import UnbiasedMtrx_hook, unbiasedMtrxState
+    shapes, rank = [(64, 576), (64,), (300, 40), (2, 1024)], 4
+    total = numel_of(shapes)
+    st = unbiasedMtrxState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2)
+    st.iter = 2
+    seeds = np.random.RandomState(421)
+    for step in range(3):
+        g = grads(total, 50 + step)
+        gd = g.cuda()
+        host_state = torch.get_rng_state()
+        out = UnbiasedMtrx_hook(st, FakeGradBucket(gd, shapes)).wait()
+        assert out.data_ptr() == gd.data_ptr()
+        assert torch.equal(torch.get_rng_state(), host_state)      # the host generator is put back
+        want = g.numpy().copy()
+        for t in oracle.split_bucket(want, shapes):
+            mat = t.reshape(t.shape[0], -1)
+            n, m = mat.shape
+            r = min(n, m, rank)
+            if not oracle.should_compress(n, m, r, 2):
+                continue
+            torch.manual_seed(int(seeds.randint(1_000_000_000)))
+            q = torch.randn(m, r, device="cuda").cpu().numpy()
+            mat[...] = oracle.pqt(oracle.mq(np.ascontiguousarray(mat), q), q)
+        assert_close(gd, want, what="unbiased matrix hook, step %d" % step)
+    assert st.p_memory_dict == {} and st.q_memory_dict == {} and st.iter == 5
+    rate, before, after = st.compression_stats()
+    assert before == 3 * total and after < before

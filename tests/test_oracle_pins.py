@@ -434,3 +434,72 @@ def test_powersgd_vs_installed_torch_hook(oracle, tmp_path):
         scale = np.abs(g).max()
         np.testing.assert_allclose(og, out.numpy(), rtol=0, atol=2e-5 * scale)
         np.testing.assert_allclose(ostate.error_dict[0], tstate.error_dict[0].numpy(), rtol=0, atol=2e-5 * scale)
+
+
+def test_batched_powersgd_vs_installed_torch_hook(oracle, tmp_path, monkeypatch):
+    """torch's batched_powerSGD_hook is the upstream of the reference's (powerSGD_hook.py:583-787);
+    at rank <= 2 it orthogonalises with the same Gram-Schmidt.  The installed hook hands its 2-D
+    P and Q to a routine that asserts a batch dimension, so for the duration of this test that
+    routine is given the batch dimension (the library's own code does the work)."""
+    import torch.distributed as dist
+    from torch.distributed.algorithms.ddp_comm_hooks import powerSGD_hook as T
+
+    if not dist.is_initialized():
+        dist.init_process_group("gloo", init_method=f"file://{tmp_path}/pg", rank=0, world_size=1)
+    library_orthogonalize = T._orthogonalize
+    monkeypatch.setattr(T, "_orthogonalize",
+                        lambda mat, epsilon=0: library_orthogonalize(mat.unsqueeze(0) if mat.dim() == 2 else mat, epsilon))
+
+    class Bucket:
+        def __init__(self, flat):
+            self._flat = flat
+
+        def buffer(self):
+            return self._flat
+
+        def index(self):
+            return 0
+
+        def is_last(self):
+            return True
+
+    for total, rank in [(5000, 1), (64 * 64, 2), (777, 2)]:
+        tstate = T.PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, random_seed=0)
+        tstate.iter = 5
+        ostate = oracle.BatchedPowerSGDOracle(matrix_approximation_rank=rank, random_seed=0)
+        rng = np.random.RandomState(34)
+        for step in range(3):
+            g = (rng.randn(total) * 1e-3).astype(np.float32)
+            tg = torch.tensor(g)          # owns its storage: the hook resizes the buffer in place
+            out = T.batched_powerSGD_hook(tstate, Bucket(tg)).wait()
+            og = g.copy()
+            ostate.step(0, og)
+            scale = np.abs(g).max()
+            assert out.shape[0] == total
+            np.testing.assert_allclose(og, out.numpy(), rtol=0, atol=2e-5 * scale)
+            np.testing.assert_allclose(ostate.error_dict[0], tstate.error_dict[0].numpy(), rtol=0, atol=2e-5 * scale)
+
+
+def test_c2cs_v2_sketch_is_over_the_reviewed_memory(oracle):
+    """C2CS_hook_v2 builds DenseCS(m, n) on matrix.view(m, n): with one [n,m] matrix and no
+    compression loss to speak of, the sketch after a step equals a hand-made update of the
+    residual re-viewed [m,n]; and for a square matrix v2 and the plain ConEF hook agree."""
+    rng = np.random.RandomState(5)
+    n, m, r = 12, 40, 2
+    g = (rng.randn(n * m) * 1e-3).astype(np.float32)
+    st = oracle.PowerSGDOracle(matrix_approximation_rank=r, error_mode="conef_v2", sketch_size=0.5, beta=0.9)
+    work = g.copy()
+    st.step(0, work, [(n, m)])
+    cs = st.error_dict[0][0]
+    assert (cs.N, cs.D, cs.range) == (m, n, max(int(n * 0.5), 1))
+    hand = oracle.DenseCS(m, n, 0.5)
+    hand.update((g - work).reshape(m, n), 0.9)       # first step: the queried sketch was zero
+    np.testing.assert_array_equal(cs.cs, hand.cs)
+    sq = (rng.randn(30 * 30) * 1e-3).astype(np.float32)
+    a = oracle.PowerSGDOracle(matrix_approximation_rank=r, error_mode="conef_v2", sketch_size=0.5)
+    b = oracle.PowerSGDOracle(matrix_approximation_rank=r, error_mode="conef", sketch_size=0.5)
+    for _ in range(3):
+        ga, gb = sq.copy(), sq.copy()
+        a.step(0, ga, [(30, 30)])
+        b.step(0, gb, [(30, 30)])
+        np.testing.assert_array_equal(ga, gb)
