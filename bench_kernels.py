@@ -174,19 +174,22 @@ def main():
         ws = torch.empty(lib.conef_psgd_workspace_bytes(n, m, r), dtype=torch.uint8, device=dev)
         plan = SketchPlan(n, m, w, A, B, dev)
         timeit("psgd_mq_f32 " + shape, 4 * n * m + 4 * (n + m) * r, make,
-               lambda s, n=n, m=m, r=r: ck(lib.conef_psgd_mq_f32(s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(), n, m,
-                                                                 r, stream), "mq"), flops=fl)
+               lambda s, n=n, m=m, r=r, ws=ws: ck(lib.conef_psgd_mq_f32(s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(),
+                                                                        n, m, r, ws.data_ptr(), ws.numel(), stream),
+                                                  "mq"), flops=fl)
         timeit("psgd_mq_ef_f32 " + shape, 12 * n * m + 4 * (n + m) * r, make,
-               lambda s, n=n, m=m, r=r: ck(lib.conef_psgd_mq_ef_f32(s[0].data_ptr(), s[3].data_ptr(), s[1].data_ptr(),
-                                                                    s[2].data_ptr(), n, m, r, stream), "mq ef"), flops=fl)
+               lambda s, n=n, m=m, r=r, ws=ws: ck(lib.conef_psgd_mq_ef_f32(s[0].data_ptr(), s[3].data_ptr(), s[1].data_ptr(),
+                                                                           s[2].data_ptr(), n, m, r, ws.data_ptr(),
+                                                                           ws.numel(), stream), "mq ef"), flops=fl)
         timeit("psgd_mq_conef_f32 %s W=%d" % (shape, w), 8 * n * m + 4 * n * w + 4 * (n + m) * r, make,
-               lambda s, n=n, m=m, r=r, w=w: ck(lib.conef_psgd_mq_conef_f32(s[0].data_ptr(), s[4].data_ptr(),
-                                                                            s[1].data_ptr(), s[2].data_ptr(), n, m, r, w,
-                                                                            0.1, A, B, stream), "mq conef"), flops=fl)
+               lambda s, n=n, m=m, r=r, w=w, ws=ws: ck(lib.conef_psgd_mq_conef_f32(
+                   s[0].data_ptr(), s[4].data_ptr(), s[1].data_ptr(), s[2].data_ptr(), n, m, r, w, 0.1, A, B,
+                   ws.data_ptr(), ws.numel(), stream), "mq conef"), flops=fl)
         timeit("psgd_mq_conef_planned_f32 %s W=%d" % (shape, w), 8 * n * m + 4 * n * w + 4 * (n + m) * r, make,
-               lambda s, n=n, m=m, r=r, w=w, plan=plan: ck(lib.conef_psgd_mq_conef_planned_f32(
+               lambda s, n=n, m=m, r=r, w=w, plan=plan, ws=ws: ck(lib.conef_psgd_mq_conef_planned_f32(
                    s[0].data_ptr(), s[4].data_ptr(), s[1].data_ptr(), s[2].data_ptr(), plan.host_ptr,
-                   plan.device.data_ptr(), n, m, r, w, 0.1, A, B, stream), "mq conef planned"), flops=fl)
+                   plan.device.data_ptr(), n, m, r, w, 0.1, A, B, ws.data_ptr(), ws.numel(), stream),
+                   "mq conef planned"), flops=fl)
         timeit("psgd_mtp_f32 " + shape, 4 * n * m + 4 * (n + m) * r, make,
                lambda s, n=n, m=m, r=r, ws=ws: ck(lib.conef_psgd_mtp_f32(s[0].data_ptr(), s[2].data_ptr(), s[1].data_ptr(),
                                                                          n, m, r, ws.data_ptr(), ws.numel(), stream),

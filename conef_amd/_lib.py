@@ -41,10 +41,11 @@ SIGNATURES = {
     "conef_randblock_unbiased_step_f32": [_P, _P, _I64, _I64, _I64, _F32, _P],
     "conef_randblock_gather_f32": [_P, _P, _I64, _I64, _I64, _F32, _P],
     "conef_randblock_scatter_f32": [_P, _P, _I64, _I64, _I64, _P],
-    "conef_psgd_mq_f32": [_P, _P, _P, _I64, _I64, _I32, _P],
-    "conef_psgd_mq_ef_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _P],
-    "conef_psgd_mq_conef_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P],
-    "conef_psgd_mq_conef_planned_f32": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P],
+    "conef_psgd_mq_f32": [_P, _P, _P, _I64, _I64, _I32, _P, _I64, _P],
+    "conef_psgd_mq_ef_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _P, _I64, _P],
+    "conef_psgd_mq_conef_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P, _I64, _P],
+    "conef_psgd_mq_conef_planned_f32": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P, _I64,
+                                        _P],
     "conef_psgd_workspace_bytes": [_I64, _I64, _I32],
     "conef_psgd_mtp_f32": [_P, _P, _P, _I64, _I64, _I32, _P, _I64, _P],
     "conef_psgd_pqt_f32": [_P, _P, _P, _I64, _I64, _I32, _P],

@@ -164,7 +164,7 @@ def run_round(state, bucket, error_mode):
 
     alpha = 1 - state.beta if error_mode in ("conef", "conef_v2") else 0.0
     residual = None
-    if error_mode == "conef_v2" and work:
+    if work and (error_mode == "conef_v2" or (error_mode == "conef" and state.matrix_approximation_rank > 8)):
         residual = _scratch_f32(device, stream, max(n * m for _, n, m, _ in work))
     errs = state.error_dict.get(bucket_index)
 
@@ -174,7 +174,7 @@ def run_round(state, bucket, error_mode):
             off = (matrix.data_ptr() - base_ptr) // 4
             e = dense_err[off: off + n * m]
             rc = lib.conef_psgd_mq_ef_f32(matrix.data_ptr(), e.data_ptr(), q.data_ptr(), p.data_ptr(), n, m, rank,
-                                          stream)
+                                          ws_ptr, ws_len, stream)
         elif error_mode == "conef":
             if cnt not in errs:
                 errs[cnt] = DenseCS(n, m, state.sketch_size, device=device)
@@ -183,24 +183,27 @@ def run_round(state, bucket, error_mode):
             if plan is not None:
                 rc = lib.conef_psgd_mq_conef_planned_f32(matrix.data_ptr(), cs.cs.data_ptr(), q.data_ptr(),
                                                          p.data_ptr(), plan.host_ptr, plan.device.data_ptr(), n, m,
-                                                         rank, cs.range, float(alpha), cs.a, cs.b, stream)
+                                                         rank, cs.range, float(alpha), cs.a, cs.b, ws_ptr, ws_len,
+                                                         stream)
             else:
                 rc = lib.conef_psgd_mq_conef_f32(matrix.data_ptr(), cs.cs.data_ptr(), q.data_ptr(), p.data_ptr(), n,
-                                                 m, rank, cs.range, float(alpha), cs.a, cs.b, stream)
+                                                 m, rank, cs.range, float(alpha), cs.a, cs.b, ws_ptr, ws_len, stream)
         elif error_mode == "conef_v2":
             # the sketch sees the same memory as m rows of n columns, so its rows are not the
             # matrix rows: query as a pass of its own, then the plain product
             if cnt not in errs:
                 errs[cnt] = DenseCS(m, n, state.sketch_size, device=device)
             errs[cnt].query(matrix.view(m, n), alpha)
-            rc = lib.conef_psgd_mq_f32(matrix.data_ptr(), q.data_ptr(), p.data_ptr(), n, m, rank, stream)
+            rc = lib.conef_psgd_mq_f32(matrix.data_ptr(), q.data_ptr(), p.data_ptr(), n, m, rank, ws_ptr, ws_len,
+                                       stream)
         elif error_mode == "topk":
             if cnt not in errs:
                 errs[cnt] = torch.zeros_like(matrix)
             rc = lib.conef_psgd_mq_ef_f32(matrix.data_ptr(), errs[cnt].data_ptr(), q.data_ptr(), p.data_ptr(), n, m,
-                                          rank, stream)
+                                          rank, ws_ptr, ws_len, stream)
         else:
-            rc = lib.conef_psgd_mq_f32(matrix.data_ptr(), q.data_ptr(), p.data_ptr(), n, m, rank, stream)
+            rc = lib.conef_psgd_mq_f32(matrix.data_ptr(), q.data_ptr(), p.data_ptr(), n, m, rank, ws_ptr, ws_len,
+                                       stream)
         _lib.check(rc, "conef_psgd_mq")
 
     if error_mode == "ef":
@@ -227,6 +230,15 @@ def run_round(state, bucket, error_mode):
             e = dense_err[off: off + n * m]
             rc = lib.conef_psgd_pqt_ef_f32(matrix.data_ptr(), e.data_ptr(), p.data_ptr(), q.data_ptr(), n, m, rank,
                                            stream)
+        elif error_mode == "conef" and rank > 8:
+            # at these ranks the low-rank product belongs on the matrix cores: M = P Q^T with the
+            # residual written out (MFMA kernel), then the sketch update as a pass of its own
+            res = residual[: n * m]
+            rc = lib.conef_psgd_pqt_ef_f32(matrix.data_ptr(), res.data_ptr(), p.data_ptr(), q.data_ptr(), n, m, rank,
+                                           stream)
+            _lib.check(rc, "conef_psgd_pqt_ef_f32")
+            errs[cnt].update(res.view(n, m), state.beta)
+            rc = 0
         elif error_mode == "conef":
             cs = errs[cnt]
             plan = cs.plan()
@@ -333,9 +345,10 @@ def run_batched_round(state, bucket):
                "conef_gram_schmidt_f32")
     if err is not None:
         rc = lib.conef_psgd_mq_ef_f32(square.data_ptr(), err.data_ptr(), q.data_ptr(), p.data_ptr(), side, side, rank,
-                                      stream)
+                                      ws_ptr, ws_len, stream)
     else:
-        rc = lib.conef_psgd_mq_f32(square.data_ptr(), q.data_ptr(), p.data_ptr(), side, side, rank, stream)
+        rc = lib.conef_psgd_mq_f32(square.data_ptr(), q.data_ptr(), p.data_ptr(), side, side, rank, ws_ptr, ws_len,
+                                   stream)
     _lib.check(rc, "conef_psgd_mq")
     _lib.check(lib.conef_gram_schmidt_f32(p.data_ptr(), side, rank, eps, ws_ptr, ws_len, stream),
                "conef_gram_schmidt_f32")

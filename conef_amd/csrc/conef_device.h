@@ -127,3 +127,17 @@ __device__ __forceinline__ float conef_wave_sum(float v)
     v += __shfl_xor(v, 32, 64);
     return v;
 }
+
+// Sum over the 64 lanes that ends in lane 63 only, all six steps on the vector ALU: four butterfly
+// steps inside each row of 16 lanes, then lane 15 of rows 0 and 2 is added into rows 1 and 3
+// (row_bcast15) and lane 31 into rows 2 and 3 (row_bcast31).
+__device__ __forceinline__ float conef_wave_sum_to_last(float v)
+{
+    v += conef_dpp<0xB1>(v);
+    v += conef_dpp<0x4E>(v);
+    v += conef_dpp<0x141>(v);
+    v += conef_dpp<0x140>(v);
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xa, 0xf, false));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xc, 0xf, false));
+    return v;
+}

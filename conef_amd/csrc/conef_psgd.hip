@@ -13,6 +13,10 @@
 #include "conef_device.h"
 #include "conef_sketch_core.h"
 #include "conef_plan.h"
+#include "conef_psgd_mfma.h"
+
+extern "C" int conef_cs_query_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
+                                  int32_t b, void* stream);
 
 namespace {
 
@@ -265,8 +269,16 @@ psgd_sum_partials_kernel(const float* __restrict__ partial, float* __restrict__ 
 {
     int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
     if (i >= count) return;
-    float s = partial[i];
-    for (int k = 1; k < slabs; ++k) s += partial[(int64_t)k * count + i];
+    float s = 0.f;
+    int k = 0;
+    for (; k + 8 <= slabs; k += 8) {        // eight loads in flight, added in slab order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = partial[(int64_t)(k + u) * count + i];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    for (; k < slabs; ++k) s += partial[(int64_t)k * count + i];
     out[i] = s;
 }
 
@@ -531,6 +543,261 @@ gram_schmidt_lds_kernel(float* __restrict__ a, int rows, int r, float eps)
     }
 }
 
+// Matrices of up to 32768 elements: one workgroup of four waves keeps the whole matrix in
+// registers (thread t owns rows t, t+256, ...: 128 / RP of them at most), so a column step is the
+// thread's own multiply-adds, one DPP reduction per remaining column, one barrier, and four LDS
+// reads per remaining column (the waves' sums, added in wave order by every thread alike).
+constexpr int kGsRegThreads = 256;
+constexpr int kGsRegFloats = 128;      // matrix elements a thread may hold
+
+// one column step; I is a template argument so that every register index is a constant
+template <int RP, int RPT, int I>
+__device__ __forceinline__ void gs_reg_step(float (&v)[RPT][RP], float (&red)[2][4][RP], int nrt, float eps, int wave,
+                                            int lane)
+{
+    float acc[RP];
+#pragma unroll
+    for (int c = I; c < RP; ++c) acc[c] = 0.f;
+#pragma unroll
+    for (int t = 0; t < RPT; ++t) {
+        if (t < nrt) {
+#pragma unroll
+            for (int c = I; c < RP; ++c) acc[c] = fmaf(v[t][I], v[t][c], acc[c]);
+        }
+    }
+#pragma unroll
+    for (int c = I; c < RP; ++c) {
+        float s = conef_wave_sum_to_last(acc[c]);
+        if (lane == 63) red[I & 1][wave][c] = s;
+    }
+    __syncthreads();
+    float tot[RP];
+#pragma unroll
+    for (int c = I; c < RP; ++c) tot[c] = (red[I & 1][0][c] + red[I & 1][1][c]) + (red[I & 1][2][c] + red[I & 1][3][c]);
+    const float nrm = sqrtf(tot[I]);
+    const float inv = 1.f / (eps == 0.f ? nrm : nrm + eps);     // one division per column, products after
+    float coef[RP];
+#pragma unroll
+    for (int c = I + 1; c < RP; ++c) coef[c] = __fmul_rn(tot[c], inv);
+#pragma unroll
+    for (int t = 0; t < RPT; ++t) {
+        if (t < nrt) {
+            const float ci = __fmul_rn(v[t][I], inv);
+            v[t][I] = ci;
+#pragma unroll
+            for (int c = I + 1; c < RP; ++c) v[t][c] = fmaf(-coef[c], ci, v[t][c]);
+        }
+    }
+}
+
+template <int RP, int RPT, int I>
+__device__ __forceinline__ void gs_reg_steps(float (&v)[RPT][RP], float (&red)[2][4][RP], int r, int nrt, float eps,
+                                             int wave, int lane)
+{
+    if constexpr (I < RP) {
+        if (I < r) {                    // uniform: columns past r hold zeros and are not stored
+            gs_reg_step<RP, RPT, I>(v, red, nrt, eps, wave, lane);
+            gs_reg_steps<RP, RPT, I + 1>(v, red, r, nrt, eps, wave, lane);
+        }
+    }
+}
+
+template <int RP, int RPT>
+__global__ void __launch_bounds__(kGsRegThreads)
+gram_schmidt_reg_kernel(float* __restrict__ a, int rows, int r, float eps)
+{
+    __shared__ float red[2][4][RP];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nrt = (rows + kGsRegThreads - 1) / kGsRegThreads;      // row slots in use (uniform)
+    float v[RPT][RP];
+#pragma unroll
+    for (int t = 0; t < RPT; ++t) {
+        const int k = threadIdx.x + t * kGsRegThreads;
+#pragma unroll
+        for (int c = 0; c < RP; ++c) v[t][c] = 0.f;
+        if (t < nrt && k < rows) {
+            const float* row = a + (int64_t)k * r;
+            if (RP >= 4 && r == RP) {
+#pragma unroll
+                for (int c = 0; c < RP; c += 4) ld4(row + c, &v[t][c]);
+            } else {
+#pragma unroll
+                for (int c = 0; c < RP; ++c)
+                    if (c < r) v[t][c] = row[c];
+            }
+        }
+    }
+    gs_reg_steps<RP, RPT, 0>(v, red, r, nrt, eps, wave, lane);
+#pragma unroll
+    for (int t = 0; t < RPT; ++t) {
+        const int k = threadIdx.x + t * kGsRegThreads;
+        if (t < nrt && k < rows) {
+            float* row = a + (int64_t)k * r;
+            if (RP >= 4 && r == RP) {
+#pragma unroll
+                for (int c = 0; c < RP; c += 4) st4(row + c, &v[t][c]);
+            } else {
+#pragma unroll
+                for (int c = 0; c < RP; ++c)
+                    if (c < r) row[c] = v[t][c];
+            }
+        }
+    }
+}
+
+// Matrices beyond one workgroup's registers: the same register-resident scheme over up to 128
+// workgroups launched cooperatively (all resident at once).  A column step ends with every
+// workgroup leaving its partial sums in the workspace and meeting the others at a counter; after
+// that every workgroup adds all partials in the same order.  The wait is bounded: a workgroup that
+// does not see the others arrive within about a second gives up and the kernel ends (the matrix
+// is then garbage; with a cooperative launch this cannot happen unless the device is lost).
+constexpr int kGsGridMaxWgs = 128;
+constexpr unsigned kGsSpinLimit = 1u << 22;
+
+struct GsGridWs {
+    unsigned arrived;      // workgroups that have reached a barrier, over all steps so far
+    unsigned gave_up;
+    unsigned pad[62];
+    float sums[2][kGsGridMaxWgs][32];
+};
+
+__global__ void gs_grid_reset_kernel(GsGridWs* ws)
+{
+    ws->arrived = 0;
+    ws->gave_up = 0;
+}
+
+template <int RP, int RPT, int I>
+__device__ __forceinline__ bool gs_grid_step(float (&v)[RPT][RP], float (&red)[4][RP], float* part, float* tot_l,
+                                             GsGridWs* ws, int nrt, float eps, int wave, int lane)
+{
+    float acc[RP];
+#pragma unroll
+    for (int c = I; c < RP; ++c) acc[c] = 0.f;
+#pragma unroll
+    for (int t = 0; t < RPT; ++t) {
+        if (t < nrt) {
+#pragma unroll
+            for (int c = I; c < RP; ++c) acc[c] = fmaf(v[t][I], v[t][c], acc[c]);
+        }
+    }
+#pragma unroll
+    for (int c = I; c < RP; ++c) {
+        float s = conef_wave_sum_to_last(acc[c]);
+        if (lane == 63) red[wave][c] = s;
+    }
+    __syncthreads();
+    const int nwg = (int)gridDim.x;
+    float* mine = ws->sums[I & 1][blockIdx.x];
+    if ((int)threadIdx.x >= I && (int)threadIdx.x < RP)
+        mine[threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+    __syncthreads();      // the partials are out before thread 0 announces the workgroup (release below)
+    if (threadIdx.x == 0) {
+        const unsigned target = (unsigned)(I + 1) * (unsigned)nwg;
+        __hip_atomic_fetch_add(&ws->arrived, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        unsigned spins = 0;
+        bool ok = true;
+        while (__hip_atomic_load(&ws->arrived, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < target) {
+            __builtin_amdgcn_s_sleep(1);
+            if (++spins > kGsSpinLimit || __hip_atomic_load(&ws->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+                ok = false;
+                __hip_atomic_store(&ws->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                break;
+            }
+        }
+        tot_l[RP] = ok ? 1.f : 0.f;
+    }
+    __syncthreads();
+    if (tot_l[RP] == 0.f) return false;      // thread 0's acquire, handed on by the barrier, covers the reads below
+    // all partials of this step: thread (g, c) reads one, one thread per column adds them in order
+    for (int e = threadIdx.x; e < nwg * RP; e += kGsRegThreads) {
+        const int g = e / RP, c = e - g * RP;
+        part[e] = c >= I ? ws->sums[I & 1][g][c] : 0.f;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x >= I && (int)threadIdx.x < RP) {
+        float s = 0.f;
+        for (int g = 0; g < nwg; ++g) s += part[g * RP + threadIdx.x];
+        tot_l[threadIdx.x] = s;
+    }
+    __syncthreads();
+    const float nrm = sqrtf(tot_l[I]);
+    const float inv = 1.f / (eps == 0.f ? nrm : nrm + eps);
+    float coef[RP];
+#pragma unroll
+    for (int c = I + 1; c < RP; ++c) coef[c] = __fmul_rn(tot_l[c], inv);
+#pragma unroll
+    for (int t = 0; t < RPT; ++t) {
+        if (t < nrt) {
+            const float ci = __fmul_rn(v[t][I], inv);
+            v[t][I] = ci;
+#pragma unroll
+            for (int c = I + 1; c < RP; ++c) v[t][c] = fmaf(-coef[c], ci, v[t][c]);
+        }
+    }
+    return true;
+}
+
+template <int RP, int RPT, int I>
+__device__ __forceinline__ void gs_grid_steps(float (&v)[RPT][RP], float (&red)[4][RP], float* part, float* tot_l,
+                                              GsGridWs* ws, int r, int nrt, float eps, int wave, int lane)
+{
+    if constexpr (I < RP) {
+        if (I < r) {
+            if (gs_grid_step<RP, RPT, I>(v, red, part, tot_l, ws, nrt, eps, wave, lane))
+                gs_grid_steps<RP, RPT, I + 1>(v, red, part, tot_l, ws, r, nrt, eps, wave, lane);
+        }
+    }
+}
+
+// workgroup b owns rows [b * rows_per_wg, +rows_per_wg); thread t its rows t, t+256, ...
+template <int RP, int RPT>
+__global__ void __launch_bounds__(kGsRegThreads)
+gram_schmidt_grid_kernel(float* __restrict__ a, int64_t rows, int r, float eps, int rows_per_wg, GsGridWs* ws)
+{
+    __shared__ float red[4][RP];
+    __shared__ float part[kGsGridMaxWgs * RP];
+    __shared__ float tot_l[RP + 1];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t k0 = (int64_t)blockIdx.x * rows_per_wg;
+    const int mine = (int)(rows - k0 < rows_per_wg ? rows - k0 : rows_per_wg);
+    const int nrt = (mine + kGsRegThreads - 1) / kGsRegThreads;
+    float v[RPT][RP];
+#pragma unroll
+    for (int t = 0; t < RPT; ++t) {
+        const int k = threadIdx.x + t * kGsRegThreads;
+#pragma unroll
+        for (int c = 0; c < RP; ++c) v[t][c] = 0.f;
+        if (t < nrt && k < mine) {
+            const float* row = a + (k0 + k) * r;
+            if (RP >= 4 && r == RP) {
+#pragma unroll
+                for (int c = 0; c < RP; c += 4) ld4(row + c, &v[t][c]);
+            } else {
+#pragma unroll
+                for (int c = 0; c < RP; ++c)
+                    if (c < r) v[t][c] = row[c];
+            }
+        }
+    }
+    gs_grid_steps<RP, RPT, 0>(v, red, part, tot_l, ws, r, nrt, eps, wave, lane);
+#pragma unroll
+    for (int t = 0; t < RPT; ++t) {
+        const int k = threadIdx.x + t * kGsRegThreads;
+        if (t < nrt && k < mine) {
+            float* row = a + (k0 + k) * r;
+            if (RP >= 4 && r == RP) {
+#pragma unroll
+                for (int c = 0; c < RP; c += 4) st4(row + c, &v[t][c]);
+            } else {
+#pragma unroll
+                for (int c = 0; c < RP; ++c)
+                    if (c < r) row[c] = v[t][c];
+            }
+        }
+    }
+}
+
 // Large matrices: r+1 launches over all CUs.  Launch i first finishes column i-1 on its own rows
 // (normalise it, take its projection off the later columns) from the sums launch i-1 left, then
 // sums column i against the later columns over its rows and leaves one partial per workgroup.
@@ -542,13 +809,31 @@ gram_schmidt_step_kernel(float* __restrict__ a, int64_t rows, int r, float eps, 
 {
     __shared__ float red[4][RP];
     __shared__ float tot[RP];
+    __shared__ float part[256];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     float coef[RP];
     float den = 1.f;
     if (i > 0) {
-        if (threadIdx.x < RP) {
+        // the workgroups' partial sums of the previous launch: 256 / RP threads per column take
+        // every (256 / RP)-th workgroup, then one thread per column adds their sums in order
+        {
+            constexpr int G = 256 / RP;
+            const int c = threadIdx.x % RP, g0 = threadIdx.x / RP;
             float s = 0.f;
-            for (int g = 0; g < (int)gridDim.x; ++g) s += sums_in[g * RP + threadIdx.x];
+            int g = g0;
+            for (; g + 3 * G < (int)gridDim.x; g += 4 * G) {
+                float v0 = sums_in[g * RP + c], v1 = sums_in[(g + G) * RP + c];
+                float v2 = sums_in[(g + 2 * G) * RP + c], v3 = sums_in[(g + 3 * G) * RP + c];
+                s += v0; s += v1; s += v2; s += v3;
+            }
+            for (; g < (int)gridDim.x; g += G) s += sums_in[g * RP + c];
+            part[threadIdx.x] = s;
+        }
+        __syncthreads();
+        if (threadIdx.x < RP) {
+            constexpr int G = 256 / RP;
+            float s = 0.f;
+            for (int g = 0; g < G; ++g) s += part[g * RP + threadIdx.x];
             tot[threadIdx.x] = s;
         }
         __syncthreads();
@@ -615,11 +900,67 @@ inline int rank_bound(int r) { return r <= 1 ? 1 : r <= 2 ? 2 : r <= 4 ? 4 : r <
         default: CALL(32); break;       \
     }
 
+// Column splits of the MFMA P = X Q kernel: enough workgroups for the machine, each at least 128
+// columns wide; the partial tiles of a row tile are added in split order by a second kernel.
+struct MfmaMqShape {
+    int row_tiles, splits, cols_per_split;
+};
+
+inline MfmaMqShape mfma_mq_shape(int64_t n, int64_t m)
+{
+    MfmaMqShape g;
+    g.row_tiles = (int)((n + 31) / 32);
+    int64_t want = (512 + g.row_tiles - 1) / g.row_tiles;
+    int64_t most = (m + 127) / 128;
+    int64_t splits = want < most ? want : most;
+    if (splits > 64) splits = 64;
+    if (splits < 1) splits = 1;
+    int64_t cps = ((m + splits - 1) / splits + 127) / 128 * 128;
+    g.cols_per_split = (int)cps;
+    g.splits = (int)((m + cps - 1) / cps);
+    return g;
+}
+
+constexpr size_t kMfmaMqLdsLimit = 144 * 1024;
+
 template <int MODE>
 int launch_mq(float* x, const float* err, const float* cs, const uint32_t* pktab, const float* q, float* p, int64_t n,
-              int64_t m, int r, int32_t w, float alpha, ConefSeeds hs, hipStream_t s)
+              int64_t m, int r, int32_t w, float alpha, ConefSeeds hs, void* workspace, int64_t workspace_bytes,
+              hipStream_t s)
 {
     ConefMod mod = conef_make_mod(w > 0 ? w : 1);
+    if (rank_bound(r) >= 16 && m % 4 == 0 && aligned16(x) && (MODE != 1 || aligned16(err)) &&
+        (!pktab || aligned16(pktab))) {
+        size_t lds = (size_t)kMfmaWaves * 16 * 64 * 4 + (MODE == 2 ? (size_t)32 * w * 4 : 0);
+        if (MODE == 2 && (mfma_mq_shape(n, m).splits > 1 || lds > kMfmaMqLdsLimit)) {
+            // Parking 32 sketch rows per workgroup costs more than the tile's share of M once the
+            // matrix is split over columns: unsketch in a launch of its own, then the plain product.
+            int rc = conef_cs_query_f32(x, cs, n, m, w, alpha, hs.a, hs.b, (void*)s);
+            if (rc != CONEF_OK) return rc;
+            return launch_mq<0>(x, nullptr, nullptr, nullptr, q, p, n, m, r, 1, 0.f, hs, workspace, workspace_bytes, s);
+        }
+        if (lds <= kMfmaMqLdsLimit) {
+            MfmaMqShape g = mfma_mq_shape(n, m);
+            if (g.splits > 1 && (!workspace || workspace_bytes < (int64_t)g.splits * n * r * 4)) {
+                g.splits = 1;
+                g.cols_per_split = (int)((m + 127) / 128 * 128);
+            }
+            float* out = g.splits > 1 ? (float*)workspace : p;
+            auto k = psgd_mfma_mq_kernel<MODE>;
+            if (lds > 48 * 1024) {
+                hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                if (e != hipSuccess) return (int)e;
+            }
+            hipLaunchKernelGGL(k, dim3((unsigned)g.row_tiles, (unsigned)g.splits), dim3(kMfmaThreads), lds, s, x, err, cs,
+                               pktab, q, out, n, (int)m, r, g.cols_per_split, mod, alpha, hs);
+            if (g.splits > 1) {
+                int64_t count = n * r;
+                hipLaunchKernelGGL(psgd_sum_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s, out,
+                                   p, count, g.splits);
+            }
+            return (int)hipGetLastError();
+        }
+    }
     const bool fast = r == rank_bound(r) && m % 4 == 0 && aligned16(x) && aligned16(q) && (MODE != 1 || aligned16(err)) &&
                       (!pktab || aligned16(pktab));
     // rows per workgroup: 4 amortises the Q traffic, but small matrices need the workgroups
@@ -668,7 +1009,39 @@ inline MtpShape mtp_shape(int64_t n, int64_t m)
     return g;
 }
 
-inline int64_t gs_sums_floats(int64_t rows, int r) { return 2 * (int64_t)kGsMaxWorkgroups * rank_bound(r); }
+// MFMA Q = X^T P: V floats per lane (column tile 32 V), row slabs whose partials cost at most a
+// quarter of the matrix's own bytes.
+struct MfmaMtpShape {
+    int v, col_tiles, slabs, rows_per_slab;
+};
+
+inline MfmaMtpShape mfma_mtp_shape(int64_t n, int64_t m, int r, int vmax)
+{
+    MfmaMtpShape g = {1, 0, 1, 0};
+    int64_t slabs_most = n / (4 * (int64_t)r);
+    if (slabs_most < 1) slabs_most = 1;
+    if (slabs_most > (n + 7) / 8) slabs_most = (n + 7) / 8;
+    for (int v = vmax; v >= 1; v >>= 1) {
+        int64_t tiles = (m + 32 * v - 1) / (32 * v);
+        int64_t want = (512 + tiles - 1) / tiles;
+        int64_t slabs = want < slabs_most ? want : slabs_most;
+        g.v = v;
+        g.col_tiles = (int)tiles;
+        g.slabs = (int)slabs;
+        if (tiles * slabs >= 512 || v == 1) break;
+    }
+    int64_t rps = ((n + g.slabs - 1) / g.slabs + 7) / 8 * 8;
+    g.rows_per_slab = (int)rps;
+    g.slabs = (int)((n + rps - 1) / rps);
+    return g;
+}
+
+inline int64_t gs_sums_floats(int64_t rows, int r)
+{
+    int64_t steps = 2 * (int64_t)kGsMaxWorkgroups * rank_bound(r);
+    int64_t grid = (int64_t)(sizeof(GsGridWs) + 3) / 4;
+    return steps > grid ? steps : grid;
+}
 
 inline bool gs_fits_lds(int64_t rows, int r)
 {
@@ -684,40 +1057,45 @@ inline bool psgd_args_ok(int64_t n, int64_t m, int32_t r)
 
 extern "C" {
 
-int conef_psgd_mq_f32(float* x, const float* q, float* p, int64_t n, int64_t m, int32_t r, void* stream)
+int conef_psgd_mq_f32(float* x, const float* q, float* p, int64_t n, int64_t m, int32_t r, void* workspace,
+                      int64_t workspace_bytes, void* stream)
 {
     if (!psgd_args_ok(n, m, r) || !x || !q || !p) return CONEF_ERR_INVALID;
     ConefSeeds hs = {0, 0, 0, 0};
-    return launch_mq<0>(x, nullptr, nullptr, nullptr, q, p, n, m, r, 1, 0.f, hs, (hipStream_t)stream);
+    return launch_mq<0>(x, nullptr, nullptr, nullptr, q, p, n, m, r, 1, 0.f, hs, workspace, workspace_bytes,
+                        (hipStream_t)stream);
 }
 
 int conef_psgd_mq_ef_f32(float* x, const float* err, const float* q, float* p, int64_t n, int64_t m, int32_t r,
-                         void* stream)
+                         void* workspace, int64_t workspace_bytes, void* stream)
 {
     if (!psgd_args_ok(n, m, r) || !x || !err || !q || !p) return CONEF_ERR_INVALID;
     ConefSeeds hs = {0, 0, 0, 0};
-    return launch_mq<1>(x, err, nullptr, nullptr, q, p, n, m, r, 1, 0.f, hs, (hipStream_t)stream);
+    return launch_mq<1>(x, err, nullptr, nullptr, q, p, n, m, r, 1, 0.f, hs, workspace, workspace_bytes,
+                        (hipStream_t)stream);
 }
 
 int conef_psgd_mq_conef_f32(float* x, const float* cs, const float* q, float* p, int64_t n, int64_t m, int32_t r,
-                            int32_t w, float alpha, int32_t a, int32_t b, void* stream)
+                            int32_t w, float alpha, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
+                            void* stream)
 {
     if (!psgd_args_ok(n, m, r) || !x || !cs || !q || !p || w < 1 || w > (1 << 30)) return CONEF_ERR_INVALID;
     ConefSeeds hs = {a, b, a + 2, b + 3};
-    return launch_mq<2>(x, nullptr, cs, nullptr, q, p, n, m, r, w, alpha, hs, (hipStream_t)stream);
+    return launch_mq<2>(x, nullptr, cs, nullptr, q, p, n, m, r, w, alpha, hs, workspace, workspace_bytes,
+                        (hipStream_t)stream);
 }
 
 // The same with the (bucket, sign) of every column read from a plan's table instead of hashed.
 int conef_psgd_mq_conef_planned_f32(float* x, const float* cs, const float* q, float* p, const void* plan_host,
                                     const void* plan_dev, int64_t n, int64_t m, int32_t r, int32_t w, float alpha,
-                                    int32_t a, int32_t b, void* stream)
+                                    int32_t a, int32_t b, void* workspace, int64_t workspace_bytes, void* stream)
 {
     const ConefPlanHeader* hp = (const ConefPlanHeader*)plan_host;
     if (!psgd_args_ok(n, m, r) || !x || !cs || !q || !p || !plan_dev || !conef_plan_matches(hp, n, m, w, a, b))
         return CONEF_ERR_INVALID;
     ConefSeeds hs = {a, b, a + 2, b + 3};
     const uint32_t* pk = (const uint32_t*)((const char*)plan_dev + hp->off_pk);
-    return launch_mq<2>(x, nullptr, cs, pk, q, p, n, m, r, w, alpha, hs, (hipStream_t)stream);
+    return launch_mq<2>(x, nullptr, cs, pk, q, p, n, m, r, w, alpha, hs, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 // Bytes of device workspace conef_psgd_mtp_f32 and conef_gram_schmidt_f32 may need for an [n,m]
@@ -726,10 +1104,21 @@ int64_t conef_psgd_workspace_bytes(int64_t n, int64_t m, int32_t r)
 {
     if (!psgd_args_ok(n, m, r)) return -1;
     MtpShape g = mtp_shape(n, m);
-    int64_t mtp = g.slabs > 1 ? (int64_t)g.slabs * m * r : 0;
+    int64_t need = g.slabs > 1 ? (int64_t)g.slabs * m * r : 0;
     int64_t rows = n > m ? n : m;
     int64_t gs = gs_sums_floats(rows, r);
-    return conef_align256(4 * (mtp > gs ? mtp : gs));
+    if (gs > need) need = gs;
+    if (rank_bound(r) >= 16) {
+        for (int v = 4; v >= 1; v >>= 1) {      // which one runs depends on the alignment of the call's pointers
+            MfmaMtpShape t = mfma_mtp_shape(n, m, r, v);
+            int64_t b = t.slabs > 1 ? (int64_t)t.slabs * m * r : 0;
+            if (b > need) need = b;
+        }
+        MfmaMqShape q = mfma_mq_shape(n, m);
+        int64_t b = q.splits > 1 ? (int64_t)q.splits * n * r : 0;
+        if (b > need) need = b;
+    }
+    return conef_align256(4 * need);
 }
 
 int conef_psgd_mtp_f32(const float* x, const float* p, float* q, int64_t n, int64_t m, int32_t r, void* workspace,
@@ -737,6 +1126,26 @@ int conef_psgd_mtp_f32(const float* x, const float* p, float* q, int64_t n, int6
 {
     if (!psgd_args_ok(n, m, r) || !x || !q || !p) return CONEF_ERR_INVALID;
     hipStream_t s = (hipStream_t)stream;
+    if (rank_bound(r) >= 16) {
+        const uintptr_t xa = reinterpret_cast<uintptr_t>(x);
+        int vmax = (m % 4 == 0 && (xa & 15u) == 0) ? 4 : (m % 2 == 0 && (xa & 7u) == 0) ? 2 : 1;
+        MfmaMtpShape t = mfma_mtp_shape(n, m, r, vmax);
+        float* dst = q;
+        if (t.slabs > 1) {
+            if (!workspace || workspace_bytes < (int64_t)t.slabs * m * r * 4) return CONEF_ERR_INVALID;
+            dst = (float*)workspace;
+        }
+        dim3 grid((unsigned)t.col_tiles, (unsigned)t.slabs);
+        if (t.v == 4) hipLaunchKernelGGL(psgd_mfma_mtp_kernel<4>, grid, dim3(kMfmaThreads), 0, s, x, p, dst, n, (int)m, r, t.rows_per_slab);
+        else if (t.v == 2) hipLaunchKernelGGL(psgd_mfma_mtp_kernel<2>, grid, dim3(kMfmaThreads), 0, s, x, p, dst, n, (int)m, r, t.rows_per_slab);
+        else hipLaunchKernelGGL(psgd_mfma_mtp_kernel<1>, grid, dim3(kMfmaThreads), 0, s, x, p, dst, n, (int)m, r, t.rows_per_slab);
+        if (t.slabs > 1) {
+            int64_t count = m * r;
+            hipLaunchKernelGGL(psgd_sum_partials_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, s, dst, q,
+                               count, t.slabs);
+        }
+        return (int)hipGetLastError();
+    }
     MtpShape g = mtp_shape(n, m);
     float* out = q;
     if (g.slabs > 1) {
@@ -765,6 +1174,25 @@ int conef_psgd_mtp_f32(const float* x, const float* p, float* q, int64_t n, int6
 static int launch_pqt(float* x, float* err, const float* p, const float* q, int64_t n, int64_t m, int32_t r,
                       hipStream_t s)
 {
+    if ((r == 16 || r == 32) && aligned16(p) && aligned16(q)) {
+        int64_t col_wgs = (m + 32 * kMfmaWaves - 1) / (32 * kMfmaWaves);
+        int64_t slabs = (1024 + col_wgs - 1) / col_wgs;
+        int64_t rps = ((n + slabs - 1) / slabs + 31) / 32 * 32;
+        slabs = (n + rps - 1) / rps;
+        if (slabs > 65535) {
+            rps = ((n + 65534) / 65535 + 31) / 32 * 32;
+            slabs = (n + rps - 1) / rps;
+        }
+        dim3 grid((unsigned)col_wgs, (unsigned)slabs);
+        if (r == 32) {
+            if (err) hipLaunchKernelGGL((psgd_mfma_pqt_kernel<32, 1>), grid, dim3(kMfmaThreads), 0, s, x, err, p, q, n, (int)m, (int)rps);
+            else hipLaunchKernelGGL((psgd_mfma_pqt_kernel<32, 0>), grid, dim3(kMfmaThreads), 0, s, x, err, p, q, n, (int)m, (int)rps);
+        } else {
+            if (err) hipLaunchKernelGGL((psgd_mfma_pqt_kernel<16, 1>), grid, dim3(kMfmaThreads), 0, s, x, err, p, q, n, (int)m, (int)rps);
+            else hipLaunchKernelGGL((psgd_mfma_pqt_kernel<16, 0>), grid, dim3(kMfmaThreads), 0, s, x, err, p, q, n, (int)m, (int)rps);
+        }
+        return (int)hipGetLastError();
+    }
     const bool fast = r == rank_bound(r) && m % 4 == 0 && aligned16(x) && aligned16(q) && (!err || aligned16(err));
     int64_t col_tiles = (m + 1023) / 1024;
     int64_t slabs = (1024 + col_tiles - 1) / col_tiles;       // about a thousand workgroups ...
@@ -851,6 +1279,28 @@ int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* w
     if (rows < 1 || rows > 0x7fffffffLL || r < 1 || r > kMaxRank || !a) return CONEF_ERR_INVALID;
     hipStream_t s = (hipStream_t)stream;
     const int rp = rank_bound(r);
+    if (rows <= (int64_t)kGsRegThreads * (kGsRegFloats / rp)) {
+        const bool vec_ok = rp < 4 || r != rp || aligned16(a);
+        if (vec_ok) {
+            // row slots per thread: the smallest of 1, 4, 16, all that holds the matrix (the unrolled
+            // code grows with the slots, and a small kernel is mostly instruction fetch)
+            const int nrt = (int)((rows + kGsRegThreads - 1) / kGsRegThreads);
+#define CONEF_GSR_GO(RP, RPT) \
+    hipLaunchKernelGGL((gram_schmidt_reg_kernel<RP, (RPT)>), dim3(1), dim3(kGsRegThreads), 0, s, a, (int)rows, r, eps)
+#define CONEF_GSR(RP)                                                                  \
+    do {                                                                               \
+        constexpr int kAll = kGsRegFloats / RP;                                        \
+        if (nrt <= 1) CONEF_GSR_GO(RP, 1);                                             \
+        else if (nrt <= 4 && kAll >= 4) CONEF_GSR_GO(RP, (kAll >= 4 ? 4 : kAll));      \
+        else if (nrt <= 16 && kAll >= 16) CONEF_GSR_GO(RP, (kAll >= 16 ? 16 : kAll));  \
+        else CONEF_GSR_GO(RP, kAll);                                                   \
+    } while (0)
+            CONEF_RANK_SWITCH(r, CONEF_GSR)
+#undef CONEF_GSR
+#undef CONEF_GSR_GO
+            return (int)hipGetLastError();
+        }
+    }
     if (gs_fits_lds(rows, r)) {
         size_t lds = (size_t)(rows * (r + 1) + 17 * rp) * 4;
         int threads = (int)((rows + 63) / 64 * 64);
@@ -869,7 +1319,37 @@ int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* w
         return (int)hipGetLastError();
     }
     if (!workspace || workspace_bytes < gs_sums_floats(rows, r) * 4) return CONEF_ERR_INVALID;
-    int64_t wgs = (rows + 255) / 256;
+    {
+        // cooperative register-resident kernel.  A step costs a trip through the barrier whatever
+        // the arithmetic, and the barrier grows with the workgroups: as many row slots per thread
+        // as the registers hold (4 at rank 32, 16 below rank 16), hence few workgroups
+        const int slots = rp >= 32 ? 4 : rp >= 16 ? 4 : 16;
+        const bool vec_ok = rp < 4 || r != rp || aligned16(a);
+        if (vec_ok && rows <= (int64_t)kGsGridMaxWgs * kGsRegThreads * slots &&
+            (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0) {
+            int64_t per = (int64_t)kGsRegThreads * slots;
+            int64_t wgs = (rows + per - 1) / per;
+            // fewer, fuller workgroups do not help: the step is bound by the barrier, not by arithmetic
+            int rows_per_wg = (int)((rows + wgs - 1) / wgs);
+            GsGridWs* gws = (GsGridWs*)workspace;
+            hipLaunchKernelGGL(gs_grid_reset_kernel, dim3(1), dim3(1), 0, s, gws);
+            void* args[] = {(void*)&a, (void*)&rows, (void*)&r, (void*)&eps, (void*)&rows_per_wg, (void*)&gws};
+            hipError_t e = hipErrorInvalidValue;
+#define CONEF_GSG(RP)                                                                                                 \
+    do {                                                                                                              \
+        constexpr int kSlots = RP >= 16 ? 4 : 16;                                                                     \
+        e = hipLaunchCooperativeKernel((const void*)gram_schmidt_grid_kernel<RP, kSlots>, dim3((unsigned)wgs),        \
+                                       dim3(kGsRegThreads), args, 0, s);                                              \
+    } while (0)
+            CONEF_RANK_SWITCH(r, CONEF_GSG)
+#undef CONEF_GSG
+            if (e == hipSuccess) return (int)hipGetLastError();
+            (void)hipGetLastError();       // cooperative launch refused: fall through to the multi-launch path
+        }
+    }
+    // a thread walks whole rows (r strided floats), so the launch is bound by the number of CUs
+    // it reaches rather than by threads: 64 rows per workgroup until the workgroup cap
+    int64_t wgs = (rows + 63) / 64;
     if (wgs > kGsMaxWorkgroups) wgs = kGsMaxWorkgroups;
     int rows_per_wg = (int)((rows + wgs - 1) / wgs);
     wgs = (rows + rows_per_wg - 1) / rows_per_wg;

@@ -14,6 +14,7 @@ import numpy as np
 import torch
 
 from . import _bucket, _lib
+from ._psgd_engine import _workspace
 from ._psgd_engine import should_compress as _should_compress
 
 
@@ -109,6 +110,7 @@ def UnbiasedMtrx_hook(state: unbiasedMtrxState, bucket) -> torch.futures.Future[
         state.p_memory_dict[bucket_index] = torch.empty(total_ps, device=device, dtype=dtype)
         state.q_memory_dict[bucket_index] = torch.empty(total_qs, device=device, dtype=dtype)
     p_mem, q_mem = state.p_memory_dict[bucket_index], state.q_memory_dict[bucket_index]
+    ws = _workspace(device, stream, max([lib.conef_psgd_workspace_bytes(n, m, rank) for _, n, m, rank in work] or [256]))
     p_idx = q_idx = 0
     for matrix, n, m, rank in work:
         p = p_mem[p_idx: p_idx + n * rank].view(n, rank)
@@ -116,7 +118,8 @@ def UnbiasedMtrx_hook(state: unbiasedMtrxState, bucket) -> torch.futures.Future[
         p_idx += n * rank
         q_idx += m * rank
         set_random(q, state, device)                                                      # :231
-        _lib.check(lib.conef_psgd_mq_f32(matrix.data_ptr(), q.data_ptr(), p.data_ptr(), n, m, rank, stream),
+        _lib.check(lib.conef_psgd_mq_f32(matrix.data_ptr(), q.data_ptr(), p.data_ptr(), n, m, rank, ws.data_ptr(),
+                                         ws.numel(), stream),
                    "conef_psgd_mq_f32")                                                   # :232
         _lib.check(lib.conef_psgd_pqt_f32(matrix.data_ptr(), p.data_ptr(), q.data_ptr(), n, m, rank, stream),
                    "conef_psgd_pqt_f32")                                                  # :292

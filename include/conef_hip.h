@@ -181,24 +181,28 @@ int conef_randblock_scatter_f32(float* x, const float* payload, int64_t numel, i
 int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* workspace, int64_t workspace_bytes,
                            void* stream);
 
-/* Bytes of device workspace conef_gram_schmidt_f32 (matrices too large for LDS) and
- * conef_psgd_mtp_f32 (sums across row slabs) may need for an [n,m] matrix at rank r.  The sums
- * meet in a fixed order: no atomics, results do not change from run to run. */
+/* Bytes of device workspace conef_gram_schmidt_f32 (matrices too large for LDS), conef_psgd_mtp_f32
+ * (sums across row slabs) and the conef_psgd_mq_* family (sums across column splits at rank >= 16)
+ * may need for an [n,m] matrix at rank r.  The sums meet in a fixed order: no atomics, results do
+ * not change from run to run.  The mq entry points also run without a workspace (null, 0): they
+ * then keep every row tile's sum inside one workgroup. */
 int64_t conef_psgd_workspace_bytes(int64_t n, int64_t m, int32_t r);
 
 /* P = M Q.  Replaces: torch.matmul(tensor, q, out=p), powerSGD_hook.py:498. */
-int conef_psgd_mq_f32(float* x, const float* q, float* p, int64_t n, int64_t m, int32_t r, void* stream);
+int conef_psgd_mq_f32(float* x, const float* q, float* p, int64_t n, int64_t m, int32_t r, void* workspace,
+                      int64_t workspace_bytes, void* stream);
 /* M += E (kept in M), then P = M Q.  Replaces: input_tensor.add_(error) :361 + :498 for one matrix
  * (also hPowerSGD_hook.py:399). */
 int conef_psgd_mq_ef_f32(float* x, const float* err, const float* q, float* p, int64_t n, int64_t m, int32_t r,
-                         void* stream);
+                         void* workspace, int64_t workspace_bytes, void* stream);
 /* M += alpha*unsketch(cs) (kept in M), then P = M Q.  Replaces: DenseCS.query :409 + :498. */
 int conef_psgd_mq_conef_f32(float* x, const float* cs, const float* q, float* p, int64_t n, int64_t m,
-                            int32_t r, int32_t w, float alpha, int32_t a, int32_t b, void* stream);
+                            int32_t r, int32_t w, float alpha, int32_t a, int32_t b, void* workspace,
+                            int64_t workspace_bytes, void* stream);
 /* The same with bucket and sign of every column read from a plan's table instead of hashed. */
 int conef_psgd_mq_conef_planned_f32(float* x, const float* cs, const float* q, float* p, const void* plan_host,
                                     const void* plan_dev, int64_t n, int64_t m, int32_t r, int32_t w, float alpha,
-                                    int32_t a, int32_t b, void* stream);
+                                    int32_t a, int32_t b, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Q = M^T P.  Replaces: torch.matmul(tensor.t(), p, out=q), powerSGD_hook.py:532. */
 int conef_psgd_mtp_f32(const float* x, const float* p, float* q, int64_t n, int64_t m, int32_t r, void* workspace,

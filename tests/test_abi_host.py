@@ -62,7 +62,7 @@ def test_argument_validation_without_gpu(lib):
     assert lib.conef_psgd_mtp_f32(1, 1, 1, 640, 5760, 4, 0, 0, 0) == -1         # several row slabs: needs the workspace
     assert lib.conef_psgd_workspace_bytes(640, 5760, 4) >= 4 * 5760 * 4
     assert lib.conef_psgd_workspace_bytes(0, 5, 1) == -1
-    assert lib.conef_psgd_mq_f32(1, 1, 1, 4, 4, 0, 0) == -1
+    assert lib.conef_psgd_mq_f32(1, 1, 1, 4, 4, 0, 0, 0, 0) == -1
     assert lib.conef_topk_sparsify_f32(1, 100, 10, 0, 0, 0) == -1               # no workspace
     assert lib.conef_topk_sparsify_f32(1, 100, 100, 0, 0, 0) == 0               # k >= numel: nothing to do
     assert lib.conef_topk_workspace_bytes(1 << 20) >= 4 * 1024

@@ -138,15 +138,20 @@ def test_unbiased_randomblock_bit_exact(oracle, shapes, ratio):
 
 def test_gram_schmidt_parity(oracle):
     from conef_amd.powerSGD_hook import _orthogonalize
-    # one workgroup with the matrix in LDS up to about 36K padded elements, r+1 launches above
+    # one workgroup with the matrix in registers up to 32768 elements, in LDS up to about 36K
+    # padded elements, r+1 launches above; unaligned starts take the scalar-access paths
     for rows, r, eps in [(27, 1, 0.0), (576, 2, 0.0), (5760, 4, 0.0), (1024, 8, 0.0), (4096, 8, 0.0), (4096, 32, 0.0),
                          (300, 3, 1e-8), (33278, 4, 0.0), (2000, 13, 0.0), (30522, 8, 0.0), (70001, 3, 1e-8),
-                         (64, 32, 0.0), (1, 1, 0.0)]:
+                         (64, 32, 0.0), (1, 1, 0.0), (1024, 32, 0.0), (1000, 32, 1e-8), (2048, 16, 0.0), (2047, 9, 0.0),
+                         (8192, 4, 0.0), (8200, 4, 0.0), (32768, 1, 0.0), (16384, 2, 0.0), (4500, 8, 0.0), (255, 5, 0.0),
+                         (257, 7, 0.0)]:
         g = torch.Generator().manual_seed(rows + r)
         a = torch.randn(rows, r, generator=g)
         want = a.numpy().copy()
         oracle.gram_schmidt(want, eps)
-        got = a.cuda()
+        off = (rows + r) % 3                       # 0: 16-byte aligned start, else not
+        got = torch.zeros(rows * r + off, device="cuda")[off:].view(rows, r)
+        got.copy_(a)
         _orthogonalize(got, eps)
         assert_close(got, want, what="gram-schmidt %dx%d" % (rows, r))
         gg = to_np(got).astype(np.float64)
@@ -162,7 +167,11 @@ def test_products_parity(oracle):
     for n, m, r, off in [(16, 27, 2, 0), (64, 576, 2, 0), (640, 5760, 4, 0), (13, 29, 3, 0), (1024, 1024, 8, 0),
                          (300, 4096, 32, 0), (1000, 77, 1, 0), (9, 4100, 16, 0), (2049, 1024, 8, 0),
                          (4099, 260, 4, 0), (640, 5760, 4, 3), (37, 4096, 8, 2), (5000, 64, 1, 0),
-                         (30522, 128, 8, 0), (515, 1028, 5, 0)]:
+                         (30522, 128, 8, 0), (515, 1028, 5, 0),
+                         # ranks 9..32 run on the matrix cores when the shapes allow
+                         (1024, 1024, 32, 0), (1000, 516, 32, 0), (33, 4096, 16, 0), (2049, 1000, 20, 0),
+                         (4096, 1024, 32, 0), (30522, 128, 32, 0), (100, 130, 32, 0), (77, 129, 16, 0),
+                         (640, 5760, 32, 3), (64, 64, 17, 0), (31, 8192, 9, 0), (1024, 4096, 32, 4)]:
         M = rng.randn(n, m).astype(np.float32)
         Q = rng.randn(m, r).astype(np.float32)
         P = rng.randn(n, r).astype(np.float32)
@@ -172,7 +181,8 @@ def test_products_parity(oracle):
         ws = torch.empty(lib.conef_psgd_workspace_bytes(n, m, r), dtype=torch.uint8, device="cuda")
         what = str((n, m, r, off))
         out = torch.empty(n, r, device="cuda")
-        assert lib.conef_psgd_mq_f32(Md.data_ptr(), Qd.data_ptr(), out.data_ptr(), n, m, r, 0) == 0
+        assert lib.conef_psgd_mq_f32(Md.data_ptr(), Qd.data_ptr(), out.data_ptr(), n, m, r, ws.data_ptr(), ws.numel(),
+                                     0) == 0
         assert_close(out, oracle.mq(M, Q), what="MQ " + what)
         outq = torch.empty(m, r, device="cuda")
         assert lib.conef_psgd_mtp_f32(Md.data_ptr(), Pd.data_ptr(), outq.data_ptr(), n, m, r, ws.data_ptr(),
@@ -181,7 +191,8 @@ def test_products_parity(oracle):
         # dense error feedback fused into the products
         E = rng.randn(n, m).astype(np.float32)
         Ed = torch.from_numpy(E).cuda()
-        assert lib.conef_psgd_mq_ef_f32(Md.data_ptr(), Ed.data_ptr(), Qd.data_ptr(), out.data_ptr(), n, m, r, 0) == 0
+        assert lib.conef_psgd_mq_ef_f32(Md.data_ptr(), Ed.data_ptr(), Qd.data_ptr(), out.data_ptr(), n, m, r,
+                                        ws.data_ptr(), ws.numel(), 0) == 0
         ME = M + E
         np.testing.assert_array_equal(to_np(Md), ME)
         assert_close(out, oracle.mq(ME, Q), what="MQ+EF " + what)
@@ -216,7 +227,7 @@ def test_products_with_sketch_on_a_plan(oracle):
         out = torch.empty(n, r, device="cuda")
         rc = lib.conef_psgd_mq_conef_planned_f32(Md.data_ptr(), cs.cs.data_ptr(), Qd.data_ptr(), out.data_ptr(),
                                                  plan.host_ptr, plan.device.data_ptr(), n, m, r, cs.range, 0.1,
-                                                 cs.a, cs.b, 0)
+                                                 cs.a, cs.b, 0, 0, 0)
         assert rc == 0
         MQ = M.copy()
         ocs.query(MQ, 0.1)
