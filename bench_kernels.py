@@ -118,6 +118,12 @@ def main():
            lambda: [(rnd(n, d), rnd(n, w).half()) for _ in range(nset)],
            lambda s: ck(lib.conef_cs_update_f16(s[0].data_ptr(), s[1].data_ptr(), s[1].data_ptr(), n, d, w, 0.9, A, B,
                                                 stream), "u16"))
+    plan16 = SketchPlan(n, d, w, A, B, dev)
+    timeit("cs_update_planned_f16 (row lists) cfg3 [640,5760] W=1152", 4 * n * d + 4 * n * w,
+           lambda: [(rnd(n, d), rnd(n, w).half()) for _ in range(nset)],
+           lambda s: ck(lib.conef_cs_update_planned_f16(s[0].data_ptr(), s[1].data_ptr(), s[1].data_ptr(),
+                                                        plan16.host_ptr, plan16.device.data_ptr(), n, d, w, 0.9, A, B,
+                                                        stream), "u16 planned"))
     timeit("cs3_query_f32 cfg3 [640,5760] W=1152", 8 * n * d + 12 * n * w,
            lambda: [(rnd(n, d), rnd(n, w), rnd(n, w), rnd(n, w)) for _ in range(nset)],
            lambda s: ck(lib.conef_cs3_query_f32(s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(), s[3].data_ptr(), n,
@@ -127,6 +133,12 @@ def main():
            lambda s: ck(lib.conef_cs3_update_f32(s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(), s[3].data_ptr(),
                                                  s[4].data_ptr(), s[5].data_ptr(), s[6].data_ptr(), n, d, w, 0.9,
                                                  stream), "u3"))
+
+    from conef_amd.compressors.CountSketchHash3 import DenseCSHash3
+    sk3 = [DenseCSHash3(n, d, 0.2) for _ in range(4)]
+    timeit("DenseCSHash3.update on plans (value pass + 3 row-list updates) cfg3 [640,5760] W=1152",
+           4 * n * d + 24 * n * w, lambda: [(rnd(n, d), sk3[i % 4]) for i in range(nset)],
+           lambda s: s[1].update(s[0], 0.9))
 
     # ------------------------------------------------------------------ random block
     L = 6_500_000

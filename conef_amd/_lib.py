@@ -56,6 +56,8 @@ SIGNATURES = {
     "conef_ef_passthrough_f32": [_P, _P, _I64, _P],
     "conef_plan_bytes": [_I64, _I64, _I32, _I32, _I32],
     "conef_plan_build_host": [_P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32],
+    "conef_plan_build_host_seeded": [_P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _I32],
+    "conef_cs3_value_f32": [_P, _P, _P, _P, _P, _I64, _I64, _I32, _F32, _P],
     "conef_plan_workspace_bytes": [_P],
     "conef_plan_kind": [_P],
     "conef_cs_update_planned_f16": [_P, _P, _P, _P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],

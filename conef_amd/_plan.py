@@ -15,14 +15,17 @@ class SketchPlan:
     """plan bytes on the host (read for launch geometry), the same bytes on the device, and the
     staging buffer the two passes hand records through."""
 
-    def __init__(self, n, d, w, a, b, device, chunk_cols=0, bin_buckets=0):
+    def __init__(self, n, d, w, a, b, device, chunk_cols=0, bin_buckets=0, sign_seeds=None):
+        """``sign_seeds``: (sa, sb) of the sign hash; None means the single-hash sketch's (a + 2, b + 3)."""
         lib = _lib.load()
         nbytes = lib.conef_plan_bytes(n, d, w, chunk_cols, bin_buckets)
         if nbytes <= 0:
             raise ValueError("no plan for shape n=%d d=%d w=%d" % (n, d, w))
         self.host = np.zeros(nbytes, dtype=np.uint8)
-        rc = lib.conef_plan_build_host(self.host.ctypes.data, nbytes, n, d, w, a, b, chunk_cols, bin_buckets)
-        _lib.check(rc, "conef_plan_build_host")
+        sa, sb = sign_seeds if sign_seeds is not None else (a + 2, b + 3)
+        rc = lib.conef_plan_build_host_seeded(self.host.ctypes.data, nbytes, n, d, w, a, b, sa, sb, chunk_cols,
+                                              bin_buckets)
+        _lib.check(rc, "conef_plan_build_host_seeded")
         self.device = torch.from_numpy(self.host).to(device)
         ws = lib.conef_plan_workspace_bytes(self.host.ctypes.data)
         self.workspace = torch.empty(max(ws, 16), dtype=torch.uint8, device=device)

@@ -2,9 +2,12 @@
 (reference: communication/compressors/CountSketchHash3.py:152-238).  Kept for comparison, as in
 the reference; the hash constants and the update/query disagreement on the third sign seed are
 the reference's (:40-41,:85,:137)."""
+import os
+
 import torch
 
 from .. import _lib
+from .._plan import SketchPlan
 
 
 class DenseCSHash3:
@@ -18,6 +21,8 @@ class DenseCSHash3:
         self.cs0, self.cs1, self.cs2 = (torch.zeros(self.N, self.range, dtype=torch.float32, device=device)
                                         for _ in range(3))
         self._spare = None
+        self._plans = None
+        self._value = None
         self._lib = _lib.load()
 
     def state_dict(self):
@@ -38,8 +43,44 @@ class DenseCSHash3:
             raise ValueError("%s has %d elements, the sketch was built for %d x %d" % (
                 name, t.numel(), self.N, self.D))
 
+    # (a, b) of the three bucket hashes and the seeds of their sign hashes in update
+    # (CountSketchHash3.py:40-41,68,77,85)
+    HASHES = ((994443, 609478, 994443 + 2, 609478 + 3), (4113759, 2949676, 4113759 + 4, 2949676 + 5),
+              (9171025, 2171464, 9171025 + 8, 2171464 + 4))
+
+    def plans(self):
+        """One accumulation plan per sketch (built on first use), or None when the shape has none
+        or CONEF_PLAN=0: the update then accumulates with float atomics."""
+        if self._plans is None:
+            self._plans = False
+            if os.environ.get("CONEF_PLAN", "1") != "0" and SketchPlan.applicable(self.N, self.D, self.range):
+                try:
+                    self._plans = [SketchPlan(self.N, self.D, self.range, a, b, self.cs0.device, sign_seeds=(sa, sb))
+                                   for a, b, sa, sb in self.HASHES]
+                except ValueError:
+                    self._plans = False
+        return self._plans or None
+
     def update(self, vec, beta):
         self._check(vec, "vec")
+        plans = self.plans()
+        if plans is not None:
+            # t = median of the three decays + value, then every sketch adds sign * t (an update
+            # with beta = 1) along its plan: no atomics, the serial definition's order
+            s = _lib.stream_ptr(vec)
+            if self._value is None:
+                self._value = torch.empty(self.N, self.D, dtype=torch.float32, device=self.cs0.device)
+            rc = self._lib.conef_cs3_value_f32(vec.data_ptr(), self.cs0.data_ptr(), self.cs1.data_ptr(),
+                                               self.cs2.data_ptr(), self._value.data_ptr(), self.N, self.D, self.range,
+                                               float(beta), s)
+            _lib.check(rc, "conef_cs3_value_f32")
+            for cs, plan, (a, b, _, _) in zip((self.cs0, self.cs1, self.cs2), plans, self.HASHES):
+                rc = self._lib.conef_cs_update_planned_f32(self._value.data_ptr(), cs.data_ptr(), cs.data_ptr(),
+                                                           plan.host_ptr, plan.device.data_ptr(),
+                                                           plan.workspace.data_ptr(), self.N, self.D, self.range, 1.0,
+                                                           a, b, s)
+                _lib.check(rc, "conef_cs_update_planned_f32")
+            return
         if self._spare is None:
             self._spare = [torch.empty_like(self.cs0) for _ in range(3)]
         o = self._spare

@@ -131,11 +131,12 @@ inline bool conef_plan_shape(int64_t n, int64_t d, int32_t w, int32_t hint_chunk
 
 // Fills a host buffer of header.total_bytes with the plan.  Returns false when a bin would hold
 // more records than a slot index can name.
-inline bool conef_plan_fill(void* buf, const ConefPlanHeader& shape, int32_t a, int32_t b)
+inline bool conef_plan_fill(void* buf, const ConefPlanHeader& shape, int32_t a, int32_t b, int32_t sa, int32_t sb)
 {
     ConefPlanHeader h = shape;
     h.a = a;
     h.b = b;
+    h.reserved[0] = ((int64_t)(uint32_t)sa << 32) | (uint32_t)sb;      // sign-hash seeds the tables were built with
     const int64_t d = h.d;
     if (h.kind == kConefPlanRowlist) {
         char* rbase = (char*)buf;
@@ -145,7 +146,7 @@ inline bool conef_plan_fill(void* buf, const ConefPlanHeader& shape, int32_t a, 
         ConefMod rmod = conef_make_mod(h.w);
         std::vector<uint32_t> count((size_t)h.w + 1, 0);
         for (int64_t i = 0; i < d; ++i) {
-            rpk[i] = conef_bucket_sign((int32_t)i, rmod, a, b, a + 2, b + 3);
+            rpk[i] = conef_bucket_sign((int32_t)i, rmod, a, b, sa, sb);
             count[(rpk[i] & 0x7fffffffu) + 1]++;
         }
         rcsr[0] = 0;
@@ -164,7 +165,7 @@ inline bool conef_plan_fill(void* buf, const ConefPlanHeader& shape, int32_t a, 
     uint16_t* ent = (uint16_t*)(base + h.off_ent);
     ConefMod mod = conef_make_mod(w);
     uint32_t* packed = (uint32_t*)(base + h.off_pk);
-    for (int64_t i = 0; i < d; ++i) packed[(size_t)i] = conef_bucket_sign((int32_t)i, mod, a, b, a + 2, b + 3);
+    for (int64_t i = 0; i < d; ++i) packed[(size_t)i] = conef_bucket_sign((int32_t)i, mod, a, b, sa, sb);
 
     // pass-A side: inside every chunk, records grouped by bin (stable in column order)
     std::vector<uint32_t> bin_fill((size_t)nbins, 0);          // records of each bin so far (earlier chunks)

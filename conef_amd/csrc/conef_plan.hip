@@ -21,16 +21,24 @@ int64_t conef_plan_bytes(int64_t n, int64_t d, int32_t w, int32_t chunk_cols, in
 
 // Builds the plan into HOST memory.  The caller copies the same bytes to the device and passes
 // both copies to the *_planned entry points (the host copy is read for launch geometry only).
-int conef_plan_build_host(void* plan_host, int64_t plan_bytes, int64_t n, int64_t d, int32_t w, int32_t a, int32_t b,
-                          int32_t chunk_cols, int32_t bin_buckets)
+// The same for a sketch whose sign hash uses the seeds (sa, sb) instead of (a + 2, b + 3): the
+// second and third sketch of the three-hash compressor (CountSketchHash3.py:77,85).
+int conef_plan_build_host_seeded(void* plan_host, int64_t plan_bytes, int64_t n, int64_t d, int32_t w, int32_t a,
+                                 int32_t b, int32_t sa, int32_t sb, int32_t chunk_cols, int32_t bin_buckets)
 {
     ConefPlanHeader h;
     if (!plan_host || !conef_plan_shape(n, d, w, chunk_cols, bin_buckets, &h)) return CONEF_ERR_INVALID;
     if (plan_bytes < h.total_bytes) return CONEF_ERR_INVALID;
-    if (!conef_plan_fill(plan_host, h, a, b)) return CONEF_ERR_INVALID;
+    if (!conef_plan_fill(plan_host, h, a, b, sa, sb)) return CONEF_ERR_INVALID;
     const ConefPlanHeader* built = (const ConefPlanHeader*)plan_host;
     if (built->kind == kConefPlanBinned && conef_binned_lds_b(built, (int)n) > 160 * 1024) return CONEF_ERR_INVALID;
     return CONEF_OK;
+}
+
+int conef_plan_build_host(void* plan_host, int64_t plan_bytes, int64_t n, int64_t d, int32_t w, int32_t a, int32_t b,
+                          int32_t chunk_cols, int32_t bin_buckets)
+{
+    return conef_plan_build_host_seeded(plan_host, plan_bytes, n, d, w, a, b, a + 2, b + 3, chunk_cols, bin_buckets);
 }
 
 int64_t conef_plan_workspace_bytes(const void* plan_host)

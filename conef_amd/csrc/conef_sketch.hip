@@ -119,6 +119,38 @@ cs3_update_kernel(const float* __restrict__ vec, const float* __restrict__ in0, 
     }
 }
 
+// The value all three sketches accumulate for an element (CountSketchHash3.py:70-93):
+// t = median(u0, u1, u2) + v with u_k = -(1 - beta) * s_k * cs_k[h_k] taken from the snapshots.
+// With t in hand, each sketch's update is the one-hash update of t with beta = 1 (no decay of its
+// own), which the planned kernels do without atomics and in the serial definition's order.
+__global__ void __launch_bounds__(256)
+cs3_value_kernel(const float* __restrict__ vec, const float* __restrict__ in0, const float* __restrict__ in1,
+                 const float* __restrict__ in2, float* __restrict__ out_t, int64_t n, int64_t d, ConefMod mod, float beta,
+                 int rows_per_block)
+{
+    int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+    if (i >= d) return;
+    uint32_t pk[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        ConefSeeds s = conef_hash3_seeds(k, /*for_query=*/false);
+        pk[k] = conef_bucket_sign((int32_t)i, mod, s.a, s.b, s.sa, s.sb);
+    }
+    const double bm1 = (double)beta - 1.0;
+    const double neg_omb = -(1. - (double)beta);
+    const uint32_t j0 = pk[0] & 0x7fffffffu, j1 = pk[1] & 0x7fffffffu, j2 = pk[2] & 0x7fffffffu;
+    int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
+    for (int64_t r = r0; r < r1; ++r) {
+        int64_t base = r * (int64_t)mod.w;
+        float value = vec[r * d + i];
+        float u0 = (float)__dmul_rn((double)conef_apply_sign(in0[base + j0], pk[0]), bm1);
+        float u1 = (float)__dmul_rn(neg_omb, (double)conef_apply_sign(in1[base + j1], pk[1]));
+        float u2 = (float)__dmul_rn(neg_omb, (double)conef_apply_sign(in2[base + j2], pk[2]));
+        out_t[r * d + i] = __fadd_rn(conef_median3(u0, u1, u2), value);
+    }
+}
+
 // -------------------------------------------------------------- utilities ----
 template <typename T>
 __global__ void scale_kernel(T* x, int64_t count, float alpha)
@@ -294,6 +326,20 @@ int conef_cs3_update_f32(const float* vec, const float* in0, const float* in1, c
     int rpb = rows_per_block_for(n, col_blocks);
     dim3 grid((unsigned)col_blocks, (unsigned)((n + rpb - 1) / rpb));
     hipLaunchKernelGGL(cs3_update_kernel, grid, dim3(256), 0, s, vec, in0, in1, in2, out0, out1, out2, n, d,
+                       conef_make_mod(w), beta, rpb);
+    return (int)hipGetLastError();
+}
+
+int conef_cs3_value_f32(const float* vec, const float* in0, const float* in1, const float* in2, float* out_t,
+                        int64_t n, int64_t d, int32_t w, float beta, void* stream)
+{
+    if (n < 0 || d < 0 || w < 1 || w > (1 << 30) || d > 0x7fffffffLL) return CONEF_ERR_INVALID;
+    if (n == 0 || d == 0) return CONEF_OK;
+    if (!vec || !in0 || !in1 || !in2 || !out_t) return CONEF_ERR_INVALID;
+    int64_t col_blocks = (d + 255) / 256;
+    int rpb = rows_per_block_for(n, col_blocks);
+    dim3 grid((unsigned)col_blocks, (unsigned)((n + rpb - 1) / rpb));
+    hipLaunchKernelGGL(cs3_value_kernel, grid, dim3(256), 0, (hipStream_t)stream, vec, in0, in1, in2, out_t, n, d,
                        conef_make_mod(w), beta, rpb);
     return (int)hipGetLastError();
 }

@@ -94,6 +94,13 @@ int conef_cs3_query_f32(float* x, const float* cs0, const float* cs1, const floa
  * sign seed (a2+8, b2+4) for the third hash).  out_k must differ from in_k. */
 int conef_cs3_update_f32(const float* vec, const float* in0, const float* in1, const float* in2, float* out0,
                          float* out1, float* out2, int64_t n, int64_t d, int32_t w, float beta, void* stream);
+/* First half of the same update without atomics: out_t[r,i] = median_k(-(1 - beta) * sign_k,i *
+ * in_k[r, bucket_k,i]) + vec[r,i], the value all three sketches accumulate for element (r,i)
+ * (CountSketchHash3.py:70-93).  The second half is conef_cs_update_planned_f32(out_t, cs_k, ...,
+ * beta = 1) once per sketch, on plans built with that sketch's hash seeds
+ * (conef_plan_build_host_seeded): same terms, same order as the serial definition. */
+int conef_cs3_value_f32(const float* vec, const float* in0, const float* in1, const float* in2, float* out_t,
+                        int64_t n, int64_t d, int32_t w, float beta, void* stream);
 
 /* ------------------------------------------------ planned accumulation (no atomics) ---- */
 /* The hash is a fixed function of (column, w, a, b), so where every column of an [n,d] tensor
@@ -115,6 +122,10 @@ int64_t conef_plan_bytes(int64_t n, int64_t d, int32_t w, int32_t chunk_cols, in
  * is only read for the launch geometry.  Host function, O(d). */
 int conef_plan_build_host(void* plan_host, int64_t plan_bytes, int64_t n, int64_t d, int32_t w, int32_t a,
                           int32_t b, int32_t chunk_cols, int32_t bin_buckets);
+/* The same for a sketch whose sign hash is seeded (sa, sb) rather than (a + 2, b + 3): the second
+ * and third sketch of the three-hash compressor (CountSketchHash3.py:77,85). */
+int conef_plan_build_host_seeded(void* plan_host, int64_t plan_bytes, int64_t n, int64_t d, int32_t w, int32_t a,
+                                 int32_t b, int32_t sa, int32_t sb, int32_t chunk_cols, int32_t bin_buckets);
 /* Bytes of device staging memory the planned entry points need (binned: n*d floats, rounded up;
  * row lists: 0, the workspace argument may then be null). */
 int64_t conef_plan_workspace_bytes(const void* plan_host);

@@ -157,6 +157,40 @@ def test_hash3_parity(oracle, n, d, ss):
     np.testing.assert_array_equal(to_np(xd), x)
 
 
+@pytest.mark.parametrize("n,d,ss", [(3, 17, 0.3), (64, 576, 0.2), (640, 5760, 0.2), (5, 50_000, 0.1), (2100, 650, 0.1),
+                                    (1, 1, 0.5), (7, 24_576, 0.05)])
+def test_hash3_update_on_plans_is_bit_exact(oracle, n, d, ss):
+    """With a plan per sketch the three-hash update has no atomics: every cell receives the
+    serial definition's terms in its order, so all three sketches match the oracle bit for bit,
+    step after step."""
+    from conef_amd.compressors.CountSketchHash3 import DenseCSHash3
+    rng = np.random.RandomState(n + d)
+    cs = DenseCSHash3(n, d, ss)
+    assert cs.plans() is not None and len(cs.plans()) == 3
+    o = oracle.DenseCSHash3(n, d, ss)
+    for step in range(3):
+        v = (rng.randn(n, d) * 1e-3).astype(np.float32)
+        cs.update(dev(v), 0.9)
+        o.update(v, 0.9)
+        for k, (g, want) in enumerate(zip((cs.cs0, cs.cs1, cs.cs2), (o.cs0, o.cs1, o.cs2))):
+            np.testing.assert_array_equal(to_np(g), want, err_msg="cs%d step %d" % (k, step))
+
+
+def test_hash3_without_plans_uses_atomics(oracle, monkeypatch):
+    from conef_amd.compressors.CountSketchHash3 import DenseCSHash3
+    monkeypatch.setenv("CONEF_PLAN", "0")
+    rng = np.random.RandomState(3)
+    n, d, ss = 6, 3000, 0.2
+    cs = DenseCSHash3(n, d, ss)
+    assert cs.plans() is None
+    o = oracle.DenseCSHash3(n, d, ss)
+    v = (rng.randn(n, d) * 1e-3).astype(np.float32)
+    cs.update(dev(v), 0.9)
+    o.update(v, 0.9)
+    for g, want in zip((cs.cs0, cs.cs1, cs.cs2), (o.cs0, o.cs1, o.cs2)):
+        assert_close(g, want, what="atomic three-hash update")
+
+
 def test_state_dict_round_trip():
     from conef_amd.compressors.CountSketch import DenseCS
     cs = DenseCS(4, 100, 0.2)
