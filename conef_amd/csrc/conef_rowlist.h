@@ -40,7 +40,8 @@ inline size_t conef_rowlist_lds(int rb, int64_t d, int32_t w, bool cells)
     size_t vals = (((size_t)rb * d + 3) & ~(size_t)3) * 4;
     size_t ent = (((size_t)d + 7) & ~(size_t)7) * 2;
     size_t csr = (((size_t)w + 1 + 3) & ~(size_t)3) * 4;
-    return vals + ent + csr + (cells ? (size_t)rb * w * 4 : 0);
+    (void)cells;      // every front parks the tile's old sketch rows in LDS
+    return vals + ent + csr + (size_t)rb * w * 4;
 }
 
 // Rows per tile: about 32 KB of values (several tiles per CU), but no more than leaves a
@@ -258,16 +259,36 @@ conef_rowlist_kernel(Front front, ConefRowlistView plan, const CsT* cs_in, CsT* 
         }
         __syncthreads();
     }
+    // The tile's cells are rows * w consecutive values; thread t owns cells t, t + 256, ...  Fronts
+    // that do not need the old rows for staging request their cells now, so that the values arrive
+    // while the tile is staged, and park them in LDS before the barrier.
+    const int total = rows * w;
+    constexpr int kPre = 8;
+    float aux_pre[kPre];
+    if (!Front::kNeedsCells) {
+#pragma unroll
+        for (int u = 0; u < kPre; ++u) {
+            const int p = threadIdx.x + u * kConefRowlistThreads;
+            aux_pre[u] = conef_ld(cs_in + row0 * w + (p < total ? p : total - 1));
+        }
+    }
     front.stage(row0, rows, d, w, vals, cells, plan.pk);
+    if (!Front::kNeedsCells) {
+#pragma unroll
+        for (int u = 0; u < kPre; ++u) {
+            const int p = threadIdx.x + u * kConefRowlistThreads;
+            if (p < total) cells[p] = aux_pre[u];
+        }
+        for (int p = threadIdx.x + kPre * kConefRowlistThreads; p < total; p += kConefRowlistThreads)
+            cells[p] = conef_ld(cs_in + row0 * w + p);
+    }
     __syncthreads();
 
-    const int total = rows * w;
     int row = threadIdx.x / w, j = threadIdx.x - row * w;
     const int srow = kConefRowlistThreads / w, sj = kConefRowlistThreads - srow * w;
     for (int p = threadIdx.x; p < total; p += kConefRowlistThreads) {
         const uint32_t e0 = csr_l[j], e1 = csr_l[j + 1];
-        const int64_t cell = (row0 + row) * w + j;
-        const float aux = Front::kNeedsCells ? cells[row * w + j] : conef_ld(cs_in + cell);
+        const float aux = cells[p];
         const double decay = __dmul_rn(one_minus_beta, (double)aux);
         const float* vr = vals + row * d;
         float acc = aux;
@@ -277,7 +298,7 @@ conef_rowlist_kernel(Front front, ConefRowlistView plan, const CsT* cs_in, CsT* 
             double sv = (double)__uint_as_float(__float_as_uint(vr[en & 0x7fffu]) ^ flip);
             acc = __fadd_rn(acc, (float)__dsub_rn(sv, decay));
         }
-        conef_st(cs_out + cell, acc);
+        conef_st(cs_out + row0 * w + p, acc);
         row += srow;
         j += sj;
         if (j >= w) {
