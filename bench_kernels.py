@@ -240,8 +240,125 @@ def main():
                                                                   for _ in range(nset)],
                lambda s, numel=numel, kk=kk: ck(lib.conef_topk_sparsify_f32(s[0].data_ptr(), numel, kk, s[1].data_ptr(),
                                                                             s[1].numel(), stream), "topk"))
+    # ------------------------------------------------------------------ whole hook steps
+    # One training step's worth of buckets through the Python hooks, per benchmark configuration:
+    # host work included (one ctypes call per kernel launch), so small-matrix models show what the
+    # launch path costs next to what the kernels cost.
+    if not args.filter or "hook" in args.filter:
+        hook_steps(args, results)
     if not args.json:
         print("done: %d cases" % len(results))
+
+
+def hook_steps(args, results):
+    import time
+
+    import numpy as np
+    import torch
+
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from _helpers import FakeGradBucket
+    from conef_amd.powerSGD_hook import PowerSGDState, powerSGD_hook
+    from conef_amd.hPowerSGD_hook import hPowerSGDState, hpowerSGD_hook
+    from conef_amd.RandomBlock_hook import RandomBlock_hook, RandomBlockState
+    from conef_amd.UnbiasedRandomBlock_hook import UnbiasedRandomBlock_hook, UnbiasedRandomBlockState
+
+    cap = 25 * 1024 * 1024 // 4
+
+    def numel(s):
+        return int(np.prod(s))
+
+    def buckets_of(shapes):
+        out, cur, size = [], [], 0
+        for s in reversed(shapes):
+            if cur and size + numel(s) > cap:
+                out.append(cur)
+                cur, size = [], 0
+            cur.append(s)
+            size += numel(s)
+        if cur:
+            out.append(cur)
+        return out
+
+    resnet20 = ([(16, 3, 3, 3), (16,), (16,)] + [(16, 16, 3, 3), (16,), (16,)] * 6 + [(32, 16, 3, 3), (32,), (32,)] +
+                [(32, 32, 3, 3), (32,), (32,)] * 5 + [(64, 32, 3, 3), (64,), (64,)] + [(64, 64, 3, 3), (64,), (64,)] * 5 +
+                [(10, 64), (10,)])
+    wrn = [(16, 3, 3, 3)]
+    widths = [16, 160, 320, 640]
+    for stage in range(3):
+        cin, cout = widths[stage], widths[stage + 1]
+        for block in range(4):
+            a = cin if block == 0 else cout
+            wrn += [(a,), (a,), (cout, a, 3, 3), (cout,), (cout,), (cout, cout, 3, 3)]
+            if block == 0:
+                wrn.append((cout, a, 1, 1))
+    wrn += [(640,), (640,), (10, 640), (10,)]
+    v, h = 33278, 650
+    lstm = [(v, h), (4 * h, h), (4 * h, h), (4 * h,), (4 * h,), (4 * h, h), (4 * h, h), (4 * h,), (4 * h,), (v, h), (v,)]
+    hh, ff, vv = 1024, 4096, 30522
+    bert = [(vv, hh), (512, hh), (2, hh), (hh,), (hh,)]
+    for _ in range(24):
+        bert += [(hh, hh), (hh,)] * 4 + [(hh,), (hh,), (ff, hh), (ff,), (hh, ff), (hh,), (hh,), (hh,)]
+    bert += [(hh, hh), (hh,), (hh, hh), (hh,), (hh,), (hh,), (vv,), (2, hh), (2,)]
+
+    def psgd(rank, ss):
+        return lambda: (PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2,
+                                      use_error_compression=True, sketch_size=ss, beta=0.9), powerSGD_hook)
+
+    cases = [
+        ("hook cfg1 ResNet-20, PowerSGD r=2 + sketch 50%", resnet20, psgd(2, 0.5)),
+        ("hook cfg2 flat 25 MB bucket, RandomBlock 10% + sketch 10%", [(5, 1_300_000)],
+         lambda: (RandomBlockState(None, compression_ratio=0.1, start_compression_iter=2, use_error_compression=True,
+                                   sketch_size=0.1, beta=0.9), RandomBlock_hook)),
+        ("hook cfg3 WRN-28-10, PowerSGD r=4 + sketch 20%", wrn, psgd(4, 0.2)),
+        ("hook cfg4 LSTM, UnbiasedRandomBlock 5%", lstm,
+         lambda: (UnbiasedRandomBlockState(None, compression_ratio=0.05, start_compression_iter=2),
+                  UnbiasedRandomBlock_hook)),
+        ("hook cfg4 LSTM, RandomBlock 5% + sketch 10%", lstm,
+         lambda: (RandomBlockState(None, compression_ratio=0.05, start_compression_iter=2, use_error_compression=True,
+                                   sketch_size=0.1, beta=0.9), RandomBlock_hook)),
+        ("hook cfg5 BERT-large, PowerSGD r=8 + sketch 10%", bert, psgd(8, 0.1)),
+        ("hook cfg5 BERT-large, PowerSGD r=32 + sketch 10%", bert, psgd(32, 0.1)),
+        ("hook cfg5 BERT-large, hPowerSGD r=8 + top-k error", bert,
+         lambda: (hPowerSGDState(None, matrix_approximation_rank=8, start_powerSGD_iter=2, use_error_compression=True,
+                                 topk_ratio=0.4), hpowerSGD_hook)),
+    ]
+    dev = torch.device("cuda", 0)
+    for name, shapes, make in cases:
+        if args.filter and args.filter not in name and args.filter != "hook":
+            continue
+        state, hook = make()
+        state.iter = 2
+        buckets = buckets_of(shapes)
+        total = sum(numel(s) for s in shapes)
+        grads = [torch.randn(sum(numel(s) for s in b), device=dev) * 1e-3 for b in buckets]
+
+        def step():
+            for i, (b, g) in enumerate(zip(buckets, grads)):
+                hook(state, FakeGradBucket(g, b, index=i, is_last=i == len(buckets) - 1)).wait()
+
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+        reps = 5
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(reps):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) / reps * 1e3
+        gpu = e0.elapsed_time(e1) / reps
+        rec = {"case": name, "ms_per_step_wall": round(wall, 3), "ms_per_step_gpu_events": round(gpu, 3),
+               "gradient_MB": round(4 * total / 1e6, 1), "buckets": len(buckets),
+               "gradient_GBs": round(4 * total / 1e6 / max(wall, gpu), 1)}
+        results.append(rec)
+        if args.json:
+            print(json.dumps(rec), flush=True)
+        else:
+            print("%-58s %8.3f ms/step wall  %8.3f ms gpu  %8.1f MB gradient in %2d buckets  %7.1f GB/s of gradient" % (
+                name, wall, gpu, rec["gradient_MB"], len(buckets), rec["gradient_GBs"]), flush=True)
 
 
 if __name__ == "__main__":

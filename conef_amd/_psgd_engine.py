@@ -37,6 +37,20 @@ def orthogonalize(matrix, epsilon=0, workspace=None):
     return workspace
 
 
+def orthogonalize_all(matrices, epsilon, ws_ptr, ws_len, stream):
+    """Gram-Schmidt of independent [rows, r] device matrices, side by side in as few launches as
+    their shapes allow."""
+    import ctypes
+    count = len(matrices)
+    if count == 0:
+        return
+    ptrs = (ctypes.c_void_p * count)(*[m.data_ptr() for m in matrices])
+    rows = (ctypes.c_int64 * count)(*[m.shape[0] for m in matrices])
+    ranks = (ctypes.c_int32 * count)(*[m.shape[1] for m in matrices])
+    rc = _lib.load().conef_gram_schmidt_batch_f32(ptrs, rows, ranks, count, float(epsilon), ws_ptr, ws_len, stream)
+    _lib.check(rc, "conef_gram_schmidt_batch_f32")
+
+
 _WORKSPACES = {}
 
 
@@ -158,9 +172,7 @@ def run_round(state, bucket, error_mode):
             host_q = [torch.randn(*q.shape, device="cpu", dtype=dtype) for q in qs]
         for q, hq in zip(qs, host_q):
             q.copy_(hq)
-    for q in qs:
-        rc = lib.conef_gram_schmidt_f32(q.data_ptr(), q.shape[0], q.shape[1], eps, ws_ptr, ws_len, stream)
-        _lib.check(rc, "conef_gram_schmidt_f32")
+    orthogonalize_all(qs, eps, ws_ptr, ws_len, stream)
 
     alpha = 1 - state.beta if error_mode in ("conef", "conef_v2") else 0.0
     residual = None
@@ -215,10 +227,9 @@ def run_round(state, bucket, error_mode):
                                               stream)
             _lib.check(rc, "conef_ef_passthrough_f32")
 
-    # pass 2: orthogonalise P, Q = M^T P
+    # pass 2: orthogonalise all P side by side, then Q = M^T P
+    orthogonalize_all(ps, eps, ws_ptr, ws_len, stream)
     for (matrix, n, m, rank), p, q in zip(work, ps, qs):
-        _lib.check(lib.conef_gram_schmidt_f32(p.data_ptr(), n, rank, eps, ws_ptr, ws_len, stream),
-                   "conef_gram_schmidt_f32")
         _lib.check(lib.conef_psgd_mtp_f32(matrix.data_ptr(), p.data_ptr(), q.data_ptr(), n, m, rank, ws_ptr, ws_len,
                                           stream), "conef_psgd_mtp_f32")
 

@@ -10,6 +10,8 @@
 // error-feedback add (before the first product) and the residual (after the last) are fused into
 // the passes that touch M anyway.  Sums that cross workgroups meet through a caller-provided
 // workspace in a fixed order: no atomics, results do not change from run to run.
+#include <vector>
+
 #include "conef_device.h"
 #include "conef_sketch_core.h"
 #include "conef_plan.h"
@@ -602,10 +604,20 @@ __device__ __forceinline__ void gs_reg_steps(float (&v)[RPT][RP], float (&red)[2
     }
 }
 
+// One launch orthogonalises up to kGsBatchMax matrices of the same rank, one workgroup each: the P
+// (or Q) factors of all tensors of a gradient bucket are independent of each other.
+constexpr int kGsBatchMax = 48;
+struct GsBatch {
+    float* a[kGsBatchMax];
+    int rows[kGsBatchMax];
+};
+
 template <int RP, int RPT>
 __global__ void __launch_bounds__(kGsRegThreads)
-gram_schmidt_reg_kernel(float* __restrict__ a, int rows, int r, float eps)
+gram_schmidt_reg_kernel(GsBatch batch, int r, float eps)
 {
+    float* __restrict__ a = batch.a[blockIdx.x];
+    const int rows = batch.rows[blockIdx.x];
     __shared__ float red[2][4][RP];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int nrt = (rows + kGsRegThreads - 1) / kGsRegThreads;      // row slots in use (uniform)
@@ -1048,6 +1060,41 @@ inline bool gs_fits_lds(int64_t rows, int r)
     return (size_t)(rows * (r + 1) + 17 * rank_bound(r)) * 4 <= kGsLdsLimit;
 }
 
+// Row slots per thread the register kernel needs for a matrix: the smallest of 1, 4, 16, all that
+// holds it (the unrolled code grows with the slots, and a small kernel is mostly instruction
+// fetch); -1 when the matrix does not fit one workgroup's registers or its rows are not 16-byte
+// aligned for the vector accesses.
+inline int gs_reg_class(const float* a, int64_t rows, int r)
+{
+    const int rp = rank_bound(r);
+    const int all = kGsRegFloats / rp;
+    if (rows > (int64_t)kGsRegThreads * all) return -1;
+    if (!(rp < 4 || r != rp || aligned16(a))) return -1;
+    const int nrt = (int)((rows + kGsRegThreads - 1) / kGsRegThreads);
+    if (nrt <= 1) return 1;
+    if (nrt <= 4 && all >= 4) return 4;
+    if (nrt <= 16 && all >= 16) return 16;
+    return all;
+}
+
+inline int gs_launch_reg_batch(const GsBatch& batch, int count, int r, int slots, float eps, hipStream_t s)
+{
+#define CONEF_GSR_GO(RP, RPT) \
+    hipLaunchKernelGGL((gram_schmidt_reg_kernel<RP, (RPT)>), dim3((unsigned)count), dim3(kGsRegThreads), 0, s, batch, r, eps)
+#define CONEF_GSR(RP)                                                       \
+    do {                                                                    \
+        constexpr int kAll = kGsRegFloats / RP;                             \
+        if (slots == 1) CONEF_GSR_GO(RP, 1);                                \
+        else if (slots == 4 && kAll >= 4) CONEF_GSR_GO(RP, (kAll >= 4 ? 4 : kAll));      \
+        else if (slots == 16 && kAll >= 16) CONEF_GSR_GO(RP, (kAll >= 16 ? 16 : kAll));  \
+        else CONEF_GSR_GO(RP, kAll);                                        \
+    } while (0)
+    CONEF_RANK_SWITCH(r, CONEF_GSR)
+#undef CONEF_GSR
+#undef CONEF_GSR_GO
+    return (int)hipGetLastError();
+}
+
 inline bool psgd_args_ok(int64_t n, int64_t m, int32_t r)
 {
     return n >= 1 && m >= 1 && r >= 1 && r <= kMaxRank && m <= 0x7fffffffLL && n <= 0x7fffffffLL;
@@ -1279,27 +1326,11 @@ int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* w
     if (rows < 1 || rows > 0x7fffffffLL || r < 1 || r > kMaxRank || !a) return CONEF_ERR_INVALID;
     hipStream_t s = (hipStream_t)stream;
     const int rp = rank_bound(r);
-    if (rows <= (int64_t)kGsRegThreads * (kGsRegFloats / rp)) {
-        const bool vec_ok = rp < 4 || r != rp || aligned16(a);
-        if (vec_ok) {
-            // row slots per thread: the smallest of 1, 4, 16, all that holds the matrix (the unrolled
-            // code grows with the slots, and a small kernel is mostly instruction fetch)
-            const int nrt = (int)((rows + kGsRegThreads - 1) / kGsRegThreads);
-#define CONEF_GSR_GO(RP, RPT) \
-    hipLaunchKernelGGL((gram_schmidt_reg_kernel<RP, (RPT)>), dim3(1), dim3(kGsRegThreads), 0, s, a, (int)rows, r, eps)
-#define CONEF_GSR(RP)                                                                  \
-    do {                                                                               \
-        constexpr int kAll = kGsRegFloats / RP;                                        \
-        if (nrt <= 1) CONEF_GSR_GO(RP, 1);                                             \
-        else if (nrt <= 4 && kAll >= 4) CONEF_GSR_GO(RP, (kAll >= 4 ? 4 : kAll));      \
-        else if (nrt <= 16 && kAll >= 16) CONEF_GSR_GO(RP, (kAll >= 16 ? 16 : kAll));  \
-        else CONEF_GSR_GO(RP, kAll);                                                   \
-    } while (0)
-            CONEF_RANK_SWITCH(r, CONEF_GSR)
-#undef CONEF_GSR
-#undef CONEF_GSR_GO
-            return (int)hipGetLastError();
-        }
+    if (gs_reg_class(a, rows, r) >= 0) {
+        GsBatch one;
+        one.a[0] = a;
+        one.rows[0] = (int)rows;
+        return gs_launch_reg_batch(one, 1, r, gs_reg_class(a, rows, r), eps, s);
     }
     if (gs_fits_lds(rows, r)) {
         size_t lds = (size_t)(rows * (r + 1) + 17 * rp) * 4;
@@ -1363,6 +1394,43 @@ int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* w
 #undef CONEF_GSS
     }
     return (int)hipGetLastError();
+}
+
+// Gram-Schmidt of `count` independent matrices (matrix k: mats[k], [rows[k], ranks[k]] row-major,
+// in place).  Matrices of equal rank that fit one workgroup's registers share launches, one
+// workgroup each; the others go through conef_gram_schmidt_f32 one by one.  mats / rows / ranks
+// are host arrays, read before the call returns.
+int conef_gram_schmidt_batch_f32(float* const* mats, const int64_t* rows, const int32_t* ranks, int32_t count, float eps,
+                                 void* workspace, int64_t workspace_bytes, void* stream)
+{
+    if (count < 0 || (count > 0 && (!mats || !rows || !ranks))) return CONEF_ERR_INVALID;
+    hipStream_t s = (hipStream_t)stream;
+    std::vector<char> done((size_t)count, 0);
+    for (int k = 0; k < count; ++k) {
+        if (rows[k] < 1 || rows[k] > 0x7fffffffLL || ranks[k] < 1 || ranks[k] > kMaxRank || !mats[k]) return CONEF_ERR_INVALID;
+    }
+    for (int k = 0; k < count; ++k) {
+        if (done[(size_t)k]) continue;
+        const int cls = gs_reg_class(mats[k], rows[k], ranks[k]);
+        if (cls < 0) {
+            int rc = conef_gram_schmidt_f32(mats[k], rows[k], ranks[k], eps, workspace, workspace_bytes, stream);
+            if (rc != CONEF_OK) return rc;
+            done[(size_t)k] = 1;
+            continue;
+        }
+        GsBatch batch;
+        int nb = 0;
+        for (int j = k; j < count && nb < kGsBatchMax; ++j) {
+            if (done[(size_t)j] || ranks[j] != ranks[k] || gs_reg_class(mats[j], rows[j], ranks[j]) != cls) continue;
+            batch.a[nb] = mats[j];
+            batch.rows[nb] = (int)rows[j];
+            ++nb;
+            done[(size_t)j] = 1;
+        }
+        int rc = gs_launch_reg_batch(batch, nb, ranks[k], cls, eps, s);
+        if (rc != CONEF_OK) return rc;
+    }
+    return CONEF_OK;
 }
 
 // dense error feedback on the parts of a bucket that are not compressed: x += e; e = 0

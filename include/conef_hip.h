@@ -192,6 +192,13 @@ int conef_randblock_scatter_f32(float* x, const float* payload, int64_t numel, i
 int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* workspace, int64_t workspace_bytes,
                            void* stream);
 
+/* The same for `count` independent matrices in as few launches as their shapes allow (matrix k:
+ * mats[k], [rows[k], ranks[k]]; host arrays, read before the call returns): the factors of all
+ * tensors of a bucket are orthogonalised side by side, one workgroup each, instead of one after
+ * the other.  Replaces: the `for p in ps: _orthogonalize(p)` loops, powerSGD_hook.py:475-477,527-528. */
+int conef_gram_schmidt_batch_f32(float* const* mats, const int64_t* rows, const int32_t* ranks, int32_t count,
+                                 float eps, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Bytes of device workspace conef_gram_schmidt_f32 (matrices too large for LDS), conef_psgd_mtp_f32
  * (sums across row slabs) and the conef_psgd_mq_* family (sums across column splits at rank >= 16)
  * may need for an [n,m] matrix at rank r.  The sums meet in a fixed order: no atomics, results do

@@ -158,6 +158,32 @@ def test_gram_schmidt_parity(oracle):
         np.testing.assert_allclose(gg.T @ gg, np.eye(r), atol=2e-5)
 
 
+def test_gram_schmidt_batch_parity(oracle):
+    """All factors of a bucket in one call: equal-rank matrices that fit one workgroup share
+    launches, the rest go one by one; every matrix must come out as from the single-matrix call."""
+    from conef_amd._psgd_engine import orthogonalize_all
+    from conef_amd import _lib
+    lib = _lib.load()
+    shapes = [(640, 4), (5760, 4), (27, 4), (1440, 4), (30522, 4), (1024, 8), (4096, 8), (64, 2), (4096, 32), (33, 4),
+              (300, 3), (1, 1)] + [(100 + 7 * k, 4) for k in range(60)]
+    gen = torch.Generator().manual_seed(9)
+    host = [torch.randn(rows, r, generator=gen) for rows, r in shapes]
+    arena = torch.zeros(sum(h.numel() for h in host) + 8, device="cuda")
+    mats, off = [], 0
+    for h in host:                       # back to back in one arena, as the hooks keep them
+        mats.append(arena[off:off + h.numel()].view(*h.shape))
+        mats[-1].copy_(h)
+        off += h.numel()
+    ws = torch.empty(max(lib.conef_psgd_workspace_bytes(rows, 1, r) for rows, r in shapes), dtype=torch.uint8,
+                     device="cuda")
+    orthogonalize_all(mats, 0.0, ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream)
+    for h, m in zip(host, mats):
+        want = h.numpy().copy()
+        oracle.gram_schmidt(want, 0.0)
+        assert_close(m, want, what="batched gram-schmidt %s" % (tuple(h.shape),))
+    assert float(arena[off:].abs().max()) == 0.0
+
+
 def test_products_parity(oracle):
     from conef_amd import _lib
     lib = _lib.load()
