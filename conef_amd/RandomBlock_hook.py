@@ -13,11 +13,13 @@ import numpy as np
 import torch
 import torch.distributed as dist
 
-from . import _bucket, _lib
+from . import _bucket
+from . import _lib
+from ._checkpoint import Checkpointable
 from .compressors.CountSketch import DenseCS
 
 
-class RandomBlockState(object):
+class RandomBlockState(Checkpointable):
     """Hyper-parameters and per-bucket state (reference: RandomBlock_hook.py:16-135).
 
     ``compression_ratio`` is the fraction of entries of every >=2-D gradient that is kept;
@@ -26,6 +28,8 @@ class RandomBlockState(object):
     ``use_error_compression`` stores the residual in a count sketch of ``sketch_size * columns``
     buckets per row with decay ``beta`` instead of a dense tensor.
     """
+
+    CHECKPOINT_FIELDS = ("iter", "rng", "error_dict")
 
     __slots__ = [
         "process_group",

@@ -11,10 +11,14 @@ import numpy as np
 import torch
 import torch.distributed as dist
 
-from . import _bucket, _lib
+from . import _bucket
+from . import _lib
+from ._checkpoint import Checkpointable
 
 
-class UnbiasedRandomBlockState(object):
+class UnbiasedRandomBlockState(Checkpointable):
+    CHECKPOINT_FIELDS = ("iter", "rng")
+
     __slots__ = [
         "process_group",
         "compression_ratio",

@@ -51,6 +51,16 @@ class DenseCS:
         self.a = int(d.get("a", HASH_A))
         self.b = int(d.get("b", HASH_B))
 
+    @classmethod
+    def from_state_dict(cls, d, device=None):
+        """A sketch rebuilt from ``state_dict()`` output (width taken from the state, not recomputed)."""
+        obj = cls(d["N"], d["D"], 0.0, device=device)
+        obj.range = int(d["range"])
+        obj.cs = torch.from_numpy(d["cs"]).to(obj.cs.device).contiguous()
+        obj.a, obj.b = int(d.get("a", HASH_A)), int(d.get("b", HASH_B))
+        obj._inplace = bool(obj._lib.conef_cs_update_inplace_ok(obj.N, obj.D, obj.range))
+        return obj
+
     __getstate__ = state_dict
 
     def __setstate__(self, d):

@@ -37,6 +37,14 @@ class DenseCSHash3:
         for k in ("cs0", "cs1", "cs2"):
             getattr(self, k).copy_(torch.from_numpy(d[k]).to(self.cs0.device))
 
+    @classmethod
+    def from_state_dict(cls, d, device=None):
+        obj = cls(d["N"], d["D"], 0.0, device=device)
+        obj.range = int(d["range"])
+        for k in ("cs0", "cs1", "cs2"):
+            setattr(obj, k, torch.from_numpy(d[k]).to(obj.cs0.device).contiguous())
+        return obj
+
     def _check(self, t, name):
         _lib.require_device_f32(t, name)
         if t.numel() != self.N * self.D:

@@ -46,6 +46,15 @@ class DenseCS:
             raise ValueError("sketch shape mismatch")
         self.cs.copy_(torch.from_numpy(d["cs"]).to(self.cs.device))
 
+    @classmethod
+    def from_state_dict(cls, d, device=None):
+        obj = cls(d["N"], d["D"], 0.0, device=device)
+        obj.range = int(d["range"])
+        obj.cs = torch.from_numpy(d["cs"]).to(obj.cs.device).contiguous()
+        obj.a, obj.b = int(d.get("a", HASH_A)), int(d.get("b", HASH_B))
+        obj._inplace = bool(obj._lib.conef_cs_update_inplace_ok(obj.N, obj.D, obj.range))
+        return obj
+
     def _check(self, t, name):
         _lib.require_device_f32(t, name)
         if t.numel() != self.N * self.D:

@@ -12,6 +12,7 @@ import numpy as np
 import torch
 
 from . import _bucket
+from ._checkpoint import Checkpointable
 from ._psgd_engine import orthogonalize as _orthogonalize  # noqa: F401
 from ._psgd_engine import run_round, topk_sparsify
 from ._psgd_engine import should_compress as _should_compress  # noqa: F401
@@ -22,7 +23,9 @@ def _topk(error_tensor, topk_ratio):
     topk_sparsify(error_tensor, topk_ratio)
 
 
-class hPowerSGDState(object):
+class hPowerSGDState(Checkpointable):
+    CHECKPOINT_FIELDS = ("iter", "rng", "error_dict", "p_memory_dict", "q_memory_dict", "total_numel_before_compression", "total_numel_after_compression")
+
     __slots__ = [
         "process_group",
         "matrix_approximation_rank",

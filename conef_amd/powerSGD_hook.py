@@ -12,12 +12,13 @@ import numpy as np
 import torch
 
 from . import _bucket
+from ._checkpoint import Checkpointable
 from ._psgd_engine import orthogonalize as _orthogonalize  # noqa: F401  (reference name, :12)
 from ._psgd_engine import run_batched_round, run_round
 from ._psgd_engine import should_compress as _should_compress  # noqa: F401  (reference name, :46)
 
 
-class PowerSGDState(object):
+class PowerSGDState(Checkpointable):
     """Hyper-parameters and cross-iteration state.
 
     ``matrix_approximation_rank`` is the rank r of the P [n,r] / Q [m,r] factors;
@@ -28,6 +29,8 @@ class PowerSGDState(object):
     ``use_error_compression`` keeps that residual in a count sketch (``sketch_size`` buckets per
     column, decay ``beta``) instead of a dense tensor; ``warm_start`` reuses P and Q.
     """
+
+    CHECKPOINT_FIELDS = ("iter", "rng", "error_dict", "p_memory_dict", "q_memory_dict", "total_numel_before_compression", "total_numel_after_compression")
 
     __slots__ = [
         "process_group",

@@ -13,7 +13,9 @@ import logging
 import numpy as np
 import torch
 
-from . import _bucket, _lib
+from . import _bucket
+from . import _lib
+from ._checkpoint import Checkpointable
 from ._psgd_engine import _workspace
 from ._psgd_engine import should_compress as _should_compress
 
@@ -27,7 +29,9 @@ def set_random(vector, state, device):
     torch.set_rng_state(cur_state)
 
 
-class unbiasedMtrxState(object):
+class unbiasedMtrxState(Checkpointable):
+    CHECKPOINT_FIELDS = ("iter", "rng", "total_numel_before_compression", "total_numel_after_compression")
+
     __slots__ = [
         "process_group",
         "matrix_approximation_rank",

@@ -429,3 +429,85 @@ def test_unbiased_mtrx_hook_parity(oracle):
     assert st.p_memory_dict == {} and st.q_memory_dict == {} and st.iter == 5
     rate, before, after = st.compression_stats()
     assert before == 3 * total and after < before
+
+
+# ------------------------------------------------------------------ checkpoints --
+
+def _resume_case(make_state, hook, shapes):
+    """Three steps, save, restore into a fresh state, two more steps on both: same results."""
+    import io
+    total = numel_of(shapes)
+    a = make_state()
+    a.iter = 2
+    for step in range(3):
+        hook(a, FakeGradBucket(grads(total, 700 + step).cuda(), shapes)).wait()
+    buf = io.BytesIO()
+    torch.save(a.state_dict(), buf)                       # plain scalars, lists, dicts, numpy arrays
+    buf.seek(0)
+    b = make_state()
+    b.load_state_dict(torch.load(buf, weights_only=False))
+    assert b.iter == a.iter == 5
+    for step in range(2):
+        ga, gb = grads(total, 800 + step).cuda(), grads(total, 800 + step).cuda()
+        hook(a, FakeGradBucket(ga, shapes)).wait()
+        hook(b, FakeGradBucket(gb, shapes)).wait()
+        assert torch.equal(ga, gb), "step %d after the restore differs" % step
+    return a, b
+
+
+def test_checkpoint_randomblock_states():
+    from conef_amd.RandomBlock_hook import RandomBlock_hook, RandomBlockState
+    from conef_amd.UnbiasedRandomBlock_hook import UnbiasedRandomBlock_hook, UnbiasedRandomBlockState
+    shapes = [(6, 5, 3), (7,), (40, 650), (5, 26_000)]
+    a, b = _resume_case(lambda: RandomBlockState(None, compression_ratio=0.1, start_compression_iter=2,
+                                                 use_error_compression=True, sketch_size=0.2, beta=0.9),
+                        RandomBlock_hook, shapes)
+    for x, y in zip(a.error_dict[0], b.error_dict[0]):
+        assert torch.equal(x.cs, y.cs) and (x.N, x.D, x.range, x.a, x.b) == (y.N, y.D, y.range, y.a, y.b)
+    a, b = _resume_case(lambda: RandomBlockState(None, compression_ratio=0.1, start_compression_iter=2),
+                        RandomBlock_hook, shapes)
+    for x, y in zip(a.error_dict[0], b.error_dict[0]):
+        assert torch.equal(x, y)
+    _resume_case(lambda: UnbiasedRandomBlockState(None, compression_ratio=0.1, start_compression_iter=2),
+                 UnbiasedRandomBlock_hook, shapes)
+
+
+@pytest.mark.parametrize("mode", ["ef", "conef", "topk", "conef_v2"])
+def test_checkpoint_powersgd_states(mode):
+    from conef_amd.hPowerSGD_hook import hPowerSGDState, hpowerSGD_hook
+    from conef_amd.powerSGD_hook import C2CS_hook_v2, PowerSGDState, powerSGD_hook
+    shapes = [(640, 1440), (640,), (320, 2880), (40, 33)]
+    if mode == "topk":
+        make, hook = (lambda: hPowerSGDState(None, matrix_approximation_rank=4, start_powerSGD_iter=2,
+                                             use_error_compression=True)), hpowerSGD_hook
+    else:
+        make = lambda: PowerSGDState(None, matrix_approximation_rank=4, start_powerSGD_iter=2,  # noqa: E731
+                                     use_error_compression=mode != "ef", sketch_size=0.2)
+        hook = C2CS_hook_v2 if mode == "conef_v2" else powerSGD_hook
+    a, b = _resume_case(make, hook, shapes)
+    assert torch.equal(a.p_memory_dict[0], b.p_memory_dict[0]) and torch.equal(a.q_memory_dict[0], b.q_memory_dict[0])
+    assert a.compression_stats() == b.compression_stats()
+
+
+def test_checkpoint_rejects_the_wrong_class():
+    from conef_amd.powerSGD_hook import PowerSGDState
+    from conef_amd.RandomBlock_hook import RandomBlockState
+    sd = RandomBlockState(None, start_compression_iter=2).state_dict()
+    with pytest.raises(ValueError, match="cannot be loaded into"):
+        PowerSGDState(None, start_powerSGD_iter=2).load_state_dict(sd)
+
+
+def test_sketch_variants_round_trip():
+    from conef_amd._checkpoint import pack, unpack
+    from conef_amd.compressors.CountSketchHash3 import DenseCSHash3
+    from conef_amd.compressors.halfCountSketch import DenseCS as HalfDenseCS
+    v = torch.randn(6, 3000, device="cuda") * 1e-3
+    for cls, names in ((DenseCSHash3, ("cs0", "cs1", "cs2")), (HalfDenseCS, ("cs",))):
+        sk = cls(6, 3000, 0.13)
+        sk.update(v, 0.9)
+        back = unpack(pack({"k": [sk]}), torch.device("cuda", 0))["k"][0]
+        assert type(back) is cls and (back.N, back.D, back.range) == (sk.N, sk.D, sk.range)
+        sk.update(v, 0.9)
+        back.update(v, 0.9)
+        for nme in names:
+            assert torch.equal(getattr(sk, nme), getattr(back, nme))
