@@ -74,3 +74,5 @@ class Checkpointable:
             raise ValueError("checkpoint lacks %s" % ", ".join(missing))
         for f in self.CHECKPOINT_FIELDS:
             setattr(self, f, unpack(state["fields"][f], device))
+        if hasattr(self, "round_cache"):
+            self.round_cache = {}        # launch tables hold pointers into the state just replaced

@@ -47,6 +47,10 @@ SIGNATURES = {
     "conef_psgd_mq_conef_planned_f32": [_P, _P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P, _I64,
                                         _P],
     "conef_psgd_workspace_bytes": [_I64, _I64, _I32],
+    "conef_psgd_batch_workspace_bytes": [_P, _I32],
+    "conef_psgd_mq_batch_f32": [_P, _I32, _I32, _F32, _I32, _I32, _P, _I64, _P],
+    "conef_psgd_mtp_batch_f32": [_P, _I32, _P, _I64, _P],
+    "conef_psgd_pqt_batch_f32": [_P, _I32, _I32, _F32, _I32, _I32, _P],
     "conef_psgd_mtp_f32": [_P, _P, _P, _I64, _I64, _I32, _P, _I64, _P],
     "conef_psgd_pqt_f32": [_P, _P, _P, _I64, _I64, _I32, _P],
     "conef_psgd_pqt_ef_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _P],
@@ -69,8 +73,14 @@ SIGNATURES = {
     "conef_topk_sparsify_f32": [_P, _I64, _I64, _P, _I64, _P],
 }
 
+class PsgdItem(ctypes.Structure):
+    """ConefPsgdItem of include/conef_hip.h: one matrix of a bucket for the batch entry points."""
+    _fields_ = [("x", _P), ("err", _P), ("cs", _P), ("plan_host", _P), ("plan_dev", _P), ("p", _P), ("q", _P),
+                ("n", _I64), ("m", _I64), ("r", _I32), ("w", _I32)]
+
+
 _RETURNS_I64 = ("conef_topk_workspace_bytes", "conef_plan_bytes", "conef_plan_workspace_bytes",
-                "conef_psgd_workspace_bytes")
+                "conef_psgd_workspace_bytes", "conef_psgd_batch_workspace_bytes")
 
 _handle = None
 

@@ -13,7 +13,7 @@ import torch
 import torch.distributed as dist
 
 from . import _bucket, _lib
-from .compressors.CountSketch import DenseCS
+from .compressors.CountSketch import HASH_A, HASH_B, DenseCS
 
 
 def should_compress(num_rows, num_cols, matrix_approximation_rank, min_compression_rate):
@@ -94,6 +94,60 @@ def topk_sparsify(err, topk_ratio, workspace=None):
     return workspace
 
 
+class _RoundPlan:
+    """What a bucket's round needs that does not change from step to step: which tensors are
+    compressed, the table of matrices the batch entry points read, the views into the P / Q
+    arenas.  Built on the first step of a bucket and reused while the bucket keeps its buffer
+    and layout, so that a step costs a handful of foreign calls however many tensors it has."""
+    __slots__ = ("key", "shapes", "work", "passthrough", "before", "after", "total_ps", "total_qs", "arena_key", "ps",
+                 "qs", "gs_p", "gs_q", "items", "count", "sketches", "fused_sketch", "residual_offsets")
+
+
+def _gs_table(matrices):
+    import ctypes
+    count = len(matrices)
+    ptrs = (ctypes.c_void_p * max(count, 1))(*[m.data_ptr() for m in matrices])
+    rows = (ctypes.c_int64 * max(count, 1))(*[m.shape[0] for m in matrices])
+    ranks = (ctypes.c_int32 * max(count, 1))(*[m.shape[1] for m in matrices])
+    return ptrs, rows, ranks, count
+
+
+def _build_round(state, grads, shapes, key, error_mode):
+    plan = _RoundPlan()
+    plan.key, plan.shapes = key, shapes
+    plan.work, plan.passthrough = [], []
+    plan.before = plan.after = plan.total_ps = plan.total_qs = 0
+    for tensor in grads:                                            # Step I (:394-418)
+        matrix = tensor.view(tensor.shape[0], -1)
+        n, m = matrix.shape
+        rank = min(n, m, state.matrix_approximation_rank)
+        ok, before, after = should_compress(n, m, rank, state.min_compression_rate)
+        plan.before += before
+        if ok:
+            plan.work.append((matrix, n, m, rank))
+            plan.total_ps += n * rank
+            plan.total_qs += m * rank
+            plan.after += after
+        else:
+            plan.passthrough.append(tensor)
+            plan.after += before
+    plan.count = len(plan.work)
+    plan.items = (_lib.PsgdItem * max(plan.count, 1))()
+    for cnt, (matrix, n, m, rank) in enumerate(plan.work):
+        it = plan.items[cnt]
+        it.x, it.n, it.m, it.r, it.w = matrix.data_ptr(), n, m, rank, 1
+    plan.arena_key = None
+    plan.sketches = []
+    plan.fused_sketch = False
+    plan.residual_offsets = []
+    off = 0
+    for _, n, m, _ in plan.work:
+        plan.residual_offsets.append(off)
+        off += n * m
+    plan.residual_offsets.append(off)
+    return plan
+
+
 def run_round(state, bucket, error_mode):
     """One hook call.  error_mode: None | 'ef' (dense, whole bucket) | 'conef' (count sketch per
     matrix) | 'conef_v2' (count sketch over the [m,n] re-view of each matrix's memory,
@@ -116,6 +170,7 @@ def run_round(state, bucket, error_mode):
     device, dtype = input_tensor.device, input_tensor.dtype
     bucket_index = _bucket.index(bucket)
     total_length = input_tensor.shape[0]
+    base_ptr = input_tensor.data_ptr()
 
     dense_err = None
     if error_mode == "ef":
@@ -125,45 +180,76 @@ def run_round(state, bucket, error_mode):
         dense_err = state.error_dict[bucket_index]
     elif error_mode in ("conef", "conef_v2", "topk"):
         state.error_dict.setdefault(bucket_index, {})
+    errs = state.error_dict.get(bucket_index)
 
-    # Step I: which tensors are worth compressing (:394-418)
-    base_ptr = input_tensor.data_ptr()
-    work, passthrough = [], []
-    total_ps, total_qs = 0, 0
-    for tensor in _bucket.gradients(bucket):
-        matrix = tensor.view(tensor.shape[0], -1)
-        n, m = matrix.shape
-        rank = min(n, m, state.matrix_approximation_rank)
-        ok, before, after = should_compress(n, m, rank, state.min_compression_rate)
-        state.total_numel_before_compression += before
-        if ok:
-            work.append((matrix, n, m, rank))
-            total_ps += n * rank
-            total_qs += m * rank
-            state.total_numel_after_compression += after
-        else:
-            passthrough.append(tensor)
-            state.total_numel_after_compression += before
+    grads = _bucket.gradients(bucket)
+    shapes = [t.shape for t in grads]
+    key = (base_ptr, total_length, error_mode, state.matrix_approximation_rank, state.min_compression_rate,
+           getattr(state, "sketch_size", None), dense_err.data_ptr() if dense_err is not None else 0)
+    plan = state.round_cache.get(bucket_index)
+    if plan is None or plan.key != key or plan.shapes != shapes:
+        plan = _build_round(state, grads, shapes, key, error_mode)
+        state.round_cache[bucket_index] = plan
+    work, items, count = plan.work, plan.items, plan.count
+    state.total_numel_before_compression += plan.before
+    state.total_numel_after_compression += plan.after
 
     # Step III: P and Q arenas, reused across iterations under warm start (:434-471)
     need_randomize_qs = (not state.warm_start) or bucket_index not in state.p_memory_dict
     if need_randomize_qs:
         if state.warm_start:
             logging.info("Allocating contiguous memory of length {} for Ps, and of length {} for Qs, "
-                         "respectively.".format(total_ps, total_qs))
-        state.p_memory_dict[bucket_index] = torch.empty(total_ps, device=device, dtype=dtype)
-        state.q_memory_dict[bucket_index] = torch.empty(total_qs, device=device, dtype=dtype)
+                         "respectively.".format(plan.total_ps, plan.total_qs))
+        state.p_memory_dict[bucket_index] = torch.empty(plan.total_ps, device=device, dtype=dtype)
+        state.q_memory_dict[bucket_index] = torch.empty(plan.total_qs, device=device, dtype=dtype)
     p_mem, q_mem = state.p_memory_dict[bucket_index], state.q_memory_dict[bucket_index]
-    ps, qs, p_idx, q_idx = [], [], 0, 0
-    for matrix, n, m, rank in work:
-        ps.append(p_mem[p_idx: p_idx + n * rank].view(n, rank))
-        qs.append(q_mem[q_idx: q_idx + m * rank].view(m, rank))
-        p_idx += n * rank
-        q_idx += m * rank
+    if plan.arena_key != (p_mem.data_ptr(), q_mem.data_ptr()):
+        plan.ps, plan.qs, p_idx, q_idx = [], [], 0, 0
+        for cnt, (matrix, n, m, rank) in enumerate(work):
+            plan.ps.append(p_mem[p_idx: p_idx + n * rank].view(n, rank))
+            plan.qs.append(q_mem[q_idx: q_idx + m * rank].view(m, rank))
+            items[cnt].p, items[cnt].q = plan.ps[-1].data_ptr(), plan.qs[-1].data_ptr()
+            p_idx += n * rank
+            q_idx += m * rank
+        plan.gs_p, plan.gs_q = _gs_table(plan.ps), _gs_table(plan.qs)
+        plan.arena_key = (p_mem.data_ptr(), q_mem.data_ptr())
+    qs = plan.qs
+
+    # error memory of every matrix in the table (created on first use; pointers that can move
+    # between steps are refreshed)
+    alpha = 1 - state.beta if error_mode in ("conef", "conef_v2") else 0.0
+    if error_mode == "ef":
+        if items[0].err is None and count:
+            for cnt, (matrix, n, m, rank) in enumerate(work):
+                items[cnt].err = dense_err.data_ptr() + (matrix.data_ptr() - base_ptr)
+    elif error_mode == "topk":
+        for cnt, (matrix, n, m, rank) in enumerate(work):
+            if cnt not in errs:
+                errs[cnt] = torch.zeros_like(matrix)
+            items[cnt].err = errs[cnt].data_ptr()
+    elif error_mode == "conef":
+        if len(plan.sketches) != count or any(errs.get(cnt) is not cs for cnt, (cs, _) in enumerate(plan.sketches)):
+            plan.sketches = []
+            for cnt, (matrix, n, m, rank) in enumerate(work):
+                if cnt not in errs:
+                    errs[cnt] = DenseCS(n, m, state.sketch_size, device=device)
+                cs = errs[cnt]
+                sk_plan = cs.plan()
+                it = items[cnt]
+                it.w = cs.range
+                it.plan_host, it.plan_dev = (sk_plan.host_ptr, sk_plan.device.data_ptr()) if sk_plan is not None else (None, None)
+                plan.sketches.append((cs, sk_plan))
+            plan.fused_sketch = (state.matrix_approximation_rank <= 8 and
+                                 all(p is not None and p.in_place for _, p in plan.sketches))
+        for cnt, (cs, _) in enumerate(plan.sketches):
+            items[cnt].cs = cs.cs.data_ptr()
+    elif error_mode == "conef_v2":
+        for cnt, (matrix, n, m, rank) in enumerate(work):
+            if cnt not in errs:
+                errs[cnt] = DenseCS(m, n, state.sketch_size, device=device)
 
     eps = float(state.orthogonalization_epsilon)
-    ws_bytes = max([lib.conef_psgd_workspace_bytes(n, m, rank) for _, n, m, rank in work] or [256])
-    ws = _workspace(device, stream, ws_bytes)
+    ws = _workspace(device, stream, max(lib.conef_psgd_batch_workspace_bytes(items, count), 256))
     ws_ptr, ws_len = ws.data_ptr(), ws.numel()
     if need_randomize_qs:
         # same seeded CPU draws as the reference so every replica starts from the same Q (:479-494)
@@ -172,114 +258,61 @@ def run_round(state, bucket, error_mode):
             host_q = [torch.randn(*q.shape, device="cpu", dtype=dtype) for q in qs]
         for q, hq in zip(qs, host_q):
             q.copy_(hq)
-    orthogonalize_all(qs, eps, ws_ptr, ws_len, stream)
-
-    alpha = 1 - state.beta if error_mode in ("conef", "conef_v2") else 0.0
-    residual = None
-    if work and (error_mode == "conef_v2" or (error_mode == "conef" and state.matrix_approximation_rank > 8)):
-        residual = _scratch_f32(device, stream, max(n * m for _, n, m, _ in work))
-    errs = state.error_dict.get(bucket_index)
+    ptrs, rows, ranks, n_mats = plan.gs_q
+    _lib.check(lib.conef_gram_schmidt_batch_f32(ptrs, rows, ranks, n_mats, eps, ws_ptr, ws_len, stream),
+               "conef_gram_schmidt_batch_f32")
 
     # pass 1: error add fused into P = M Q
-    for cnt, ((matrix, n, m, rank), p, q) in enumerate(zip(work, ps, qs)):
-        if error_mode == "ef":
-            off = (matrix.data_ptr() - base_ptr) // 4
-            e = dense_err[off: off + n * m]
-            rc = lib.conef_psgd_mq_ef_f32(matrix.data_ptr(), e.data_ptr(), q.data_ptr(), p.data_ptr(), n, m, rank,
-                                          ws_ptr, ws_len, stream)
-        elif error_mode == "conef":
-            if cnt not in errs:
-                errs[cnt] = DenseCS(n, m, state.sketch_size, device=device)
-            cs = errs[cnt]
-            plan = cs.plan()
-            if plan is not None:
-                rc = lib.conef_psgd_mq_conef_planned_f32(matrix.data_ptr(), cs.cs.data_ptr(), q.data_ptr(),
-                                                         p.data_ptr(), plan.host_ptr, plan.device.data_ptr(), n, m,
-                                                         rank, cs.range, float(alpha), cs.a, cs.b, ws_ptr, ws_len,
-                                                         stream)
-            else:
-                rc = lib.conef_psgd_mq_conef_f32(matrix.data_ptr(), cs.cs.data_ptr(), q.data_ptr(), p.data_ptr(), n,
-                                                 m, rank, cs.range, float(alpha), cs.a, cs.b, ws_ptr, ws_len, stream)
-        elif error_mode == "conef_v2":
-            # the sketch sees the same memory as m rows of n columns, so its rows are not the
-            # matrix rows: query as a pass of its own, then the plain product
-            if cnt not in errs:
-                errs[cnt] = DenseCS(m, n, state.sketch_size, device=device)
+    if error_mode == "conef_v2":
+        # the sketch sees the same memory as m rows of n columns, so its rows are not the matrix
+        # rows: query as a pass of its own, then the plain product
+        for cnt, (matrix, n, m, rank) in enumerate(work):
             errs[cnt].query(matrix.view(m, n), alpha)
-            rc = lib.conef_psgd_mq_f32(matrix.data_ptr(), q.data_ptr(), p.data_ptr(), n, m, rank, ws_ptr, ws_len,
-                                       stream)
-        elif error_mode == "topk":
-            if cnt not in errs:
-                errs[cnt] = torch.zeros_like(matrix)
-            rc = lib.conef_psgd_mq_ef_f32(matrix.data_ptr(), errs[cnt].data_ptr(), q.data_ptr(), p.data_ptr(), n, m,
-                                          rank, ws_ptr, ws_len, stream)
-        else:
-            rc = lib.conef_psgd_mq_f32(matrix.data_ptr(), q.data_ptr(), p.data_ptr(), n, m, rank, ws_ptr, ws_len,
-                                       stream)
-        _lib.check(rc, "conef_psgd_mq")
+    mode1 = {"ef": 1, "topk": 1, "conef": 2}.get(error_mode, 0)
+    rc = lib.conef_psgd_mq_batch_f32(items, count, mode1, float(alpha), HASH_A, HASH_B, ws_ptr, ws_len, stream)
+    _lib.check(rc, "conef_psgd_mq_batch_f32")
 
     if error_mode == "ef":
         # tensors that are not compressed: g += e, and their new error is exactly zero (:361,:558)
-        for tensor in passthrough:
+        for tensor in plan.passthrough:
             off = (tensor.data_ptr() - base_ptr) // 4
             cnt_el = tensor.numel()
-            rc = lib.conef_ef_passthrough_f32(tensor.data_ptr(), dense_err[off: off + cnt_el].data_ptr(), cnt_el,
-                                              stream)
+            rc = lib.conef_ef_passthrough_f32(tensor.data_ptr(), dense_err.data_ptr() + 4 * off, cnt_el, stream)
             _lib.check(rc, "conef_ef_passthrough_f32")
 
     # pass 2: orthogonalise all P side by side, then Q = M^T P
-    orthogonalize_all(ps, eps, ws_ptr, ws_len, stream)
-    for (matrix, n, m, rank), p, q in zip(work, ps, qs):
-        _lib.check(lib.conef_psgd_mtp_f32(matrix.data_ptr(), p.data_ptr(), q.data_ptr(), n, m, rank, ws_ptr, ws_len,
-                                          stream), "conef_psgd_mtp_f32")
+    ptrs, rows, ranks, n_mats = plan.gs_p
+    _lib.check(lib.conef_gram_schmidt_batch_f32(ptrs, rows, ranks, n_mats, eps, ws_ptr, ws_len, stream),
+               "conef_gram_schmidt_batch_f32")
+    _lib.check(lib.conef_psgd_mtp_batch_f32(items, count, ws_ptr, ws_len, stream), "conef_psgd_mtp_batch_f32")
 
     # pass 3: M = P Q^T with the residual fused
-    topk_ws = None
-    for cnt, ((matrix, n, m, rank), p, q) in enumerate(zip(work, ps, qs)):
-        if error_mode == "ef":
-            off = (matrix.data_ptr() - base_ptr) // 4
-            e = dense_err[off: off + n * m]
-            rc = lib.conef_psgd_pqt_ef_f32(matrix.data_ptr(), e.data_ptr(), p.data_ptr(), q.data_ptr(), n, m, rank,
-                                           stream)
-        elif error_mode == "conef" and rank > 8:
-            # at these ranks the low-rank product belongs on the matrix cores: M = P Q^T with the
-            # residual written out (MFMA kernel), then the sketch update as a pass of its own
-            res = residual[: n * m]
-            rc = lib.conef_psgd_pqt_ef_f32(matrix.data_ptr(), res.data_ptr(), p.data_ptr(), q.data_ptr(), n, m, rank,
-                                           stream)
-            _lib.check(rc, "conef_psgd_pqt_ef_f32")
-            errs[cnt].update(res.view(n, m), state.beta)
-            rc = 0
-        elif error_mode == "conef":
-            cs = errs[cnt]
-            plan = cs.plan()
-            if plan is not None and plan.in_place:
-                rc = lib.conef_psgd_pqt_conef_planned_f32(matrix.data_ptr(), p.data_ptr(), q.data_ptr(),
-                                                          cs.cs.data_ptr(), cs.cs.data_ptr(), plan.host_ptr,
-                                                          plan.device.data_ptr(), n, m, rank, cs.range,
-                                                          float(state.beta), cs.a, cs.b, stream)
-            else:
-                out = cs.next_buffer()
-                rc = lib.conef_psgd_pqt_conef_f32(matrix.data_ptr(), p.data_ptr(), q.data_ptr(), cs.cs.data_ptr(),
-                                                  out.data_ptr(), n, m, rank, cs.range, float(state.beta), cs.a,
-                                                  cs.b, stream)
-                cs.commit(out)
-        elif error_mode == "conef_v2":
-            res = residual[: n * m]
-            rc = lib.conef_psgd_pqt_ef_f32(matrix.data_ptr(), res.data_ptr(), p.data_ptr(), q.data_ptr(), n, m, rank,
-                                           stream)
-            _lib.check(rc, "conef_psgd_pqt_ef_f32")
-            errs[cnt].update(res.view(m, n), state.beta)
-            rc = 0
-        elif error_mode == "topk":
-            rc = lib.conef_psgd_pqt_ef_f32(matrix.data_ptr(), errs[cnt].data_ptr(), p.data_ptr(), q.data_ptr(), n, m,
-                                           rank, stream)
-            _lib.check(rc, "conef_psgd_pqt_ef_f32")
+    residual = None
+    if error_mode in ("ef", "topk"):
+        mode3 = 1
+    elif error_mode == "conef" and plan.fused_sketch:
+        mode3 = 2
+    elif error_mode in ("conef", "conef_v2"):
+        # The residual goes out dense and every sketch is updated in a launch of its own: ranks
+        # above 8 (the low-rank product belongs on the matrix cores), sketches whose plan is not a
+        # row list, and the re-viewed sketches of C2CS_hook_v2.
+        mode3 = 1
+        residual = _scratch_f32(device, stream, max(plan.residual_offsets[-1], 1))
+        for cnt in range(count):
+            items[cnt].err = residual.data_ptr() + 4 * plan.residual_offsets[cnt]
+    else:
+        mode3 = 0
+    rc = lib.conef_psgd_pqt_batch_f32(items, count, mode3, float(state.beta) if mode3 == 2 else 0.0, HASH_A, HASH_B,
+                                      stream)
+    _lib.check(rc, "conef_psgd_pqt_batch_f32")
+    if error_mode == "topk":
+        topk_ws = None
+        for cnt in range(count):
             topk_ws = topk_sparsify(errs[cnt], state.topk_ratio, topk_ws)
-            rc = 0
-        else:
-            rc = lib.conef_psgd_pqt_f32(matrix.data_ptr(), p.data_ptr(), q.data_ptr(), n, m, rank, stream)
-        _lib.check(rc, "conef_psgd_pqt")
+    elif residual is not None:
+        for cnt, (matrix, n, m, rank) in enumerate(work):
+            res = residual[plan.residual_offsets[cnt]: plan.residual_offsets[cnt + 1]]
+            errs[cnt].update(res.view(n, m) if error_mode == "conef" else res.view(m, n), state.beta)
 
     if not state.warm_start:
         state.p_memory_dict.clear()

@@ -16,6 +16,7 @@
 #include "conef_sketch_core.h"
 #include "conef_plan.h"
 #include "conef_psgd_mfma.h"
+#include "conef_hip.h"      // ConefPsgdItem, and a check of this file's definitions against the public header
 
 extern "C" int conef_cs_query_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
                                   int32_t b, void* stream);
@@ -40,6 +41,30 @@ __device__ __forceinline__ void st4(float* p, const float* v)
 // pointer 16-byte aligned: 16-byte accesses, Q rows of a column quad are one contiguous run) and a
 // general form (any r <= RP, any alignment, 4-byte accesses).
 
+// ------------------------------------------------------------ batched launches ----
+// A gradient bucket holds several matrices whose products are independent of each other, and most
+// of them are too small to fill 256 CUs on their own.  Every product kernel therefore exists in
+// two forms: one matrix per launch, and up to kPsgdBatchMax matrices per launch with the
+// per-matrix arguments in a table passed by value; a workgroup finds its matrix from the table's
+// running workgroup count and then does exactly what it would do in a launch of its own.
+constexpr int kPsgdBatchMax = 24;
+
+template <typename Item>
+struct PsgdBatch {
+    Item item[kPsgdBatchMax];
+    int first[kPsgdBatchMax + 1];   // first workgroup of item i; first[count] = workgroups in all
+    int count;
+};
+
+template <typename Item>
+__device__ __forceinline__ int psgd_batch_locate(const PsgdBatch<Item>& b, int* local)
+{
+    int i = 0;
+    while (i + 1 < b.count && (int)blockIdx.x >= b.first[i + 1]) ++i;
+    *local = (int)blockIdx.x - b.first[i];
+    return i;
+}
+
 // ---------------------------------------------------------------- P = X Q ----
 // MODE 0: X = M as stored.  MODE 1: X = M + E (dense error), written back into M.
 // MODE 2: X = M + alpha * unsketch(cs), written back into M (DenseCS.query fused); the sketch rows
@@ -47,15 +72,15 @@ __device__ __forceinline__ void st4(float* p, const float* v)
 // A workgroup owns RB consecutive rows and all columns; a thread owns column quads tid, tid+256, ...
 // and keeps RB x RP partial sums, reduced over the workgroup at the end in a fixed order.
 template <int RB, int RP, int MODE, bool FAST>
-__global__ void __launch_bounds__(256)
-psgd_mq_kernel(float* __restrict__ x, const float* __restrict__ err, const float* __restrict__ cs,
-               const uint32_t* __restrict__ pktab, const float* __restrict__ q, float* __restrict__ p, int64_t n,
-               int m, int r, ConefMod mod, float alpha, ConefSeeds hs)
+__device__ __forceinline__ void
+psgd_mq_body(float* __restrict__ x, const float* __restrict__ err, const float* __restrict__ cs,
+             const uint32_t* __restrict__ pktab, const float* __restrict__ q, float* __restrict__ p, int64_t n,
+             int m, int r, ConefMod mod, float alpha, ConefSeeds hs, int bx)
 {
     extern __shared__ float mq_lds[];
     float* red = mq_lds;                    // [4][RB*RP]
     float* cells = mq_lds + 4 * RB * RP;    // [RB][w], MODE 2 only
-    const int64_t row0 = (int64_t)blockIdx.x * RB;
+    const int64_t row0 = (int64_t)bx * RB;
     const int w = (int)mod.w;
     int64_t rowc[RB];                       // rows past the end are clamped for loads, their stores are skipped
 #pragma unroll
@@ -166,6 +191,36 @@ psgd_mq_kernel(float* __restrict__ x, const float* __restrict__ err, const float
     }
 }
 
+template <int RB, int RP, int MODE, bool FAST>
+__global__ void __launch_bounds__(256)
+psgd_mq_kernel(float* __restrict__ x, const float* __restrict__ err, const float* __restrict__ cs,
+               const uint32_t* __restrict__ pktab, const float* __restrict__ q, float* __restrict__ p, int64_t n,
+               int m, int r, ConefMod mod, float alpha, ConefSeeds hs)
+{
+    psgd_mq_body<RB, RP, MODE, FAST>(x, err, cs, pktab, q, p, n, m, r, mod, alpha, hs, (int)blockIdx.x);
+}
+
+struct MqItem {
+    float* x;
+    const float* err;
+    const float* cs;
+    const uint32_t* pktab;
+    const float* q;
+    float* p;
+    int64_t n;
+    int m, r;
+    ConefMod mod;
+};
+
+template <int RB, int RP, int MODE, bool FAST>
+__global__ void __launch_bounds__(256)
+psgd_mq_batch_kernel(PsgdBatch<MqItem> b, float alpha, ConefSeeds hs)
+{
+    int local;
+    const MqItem& it = b.item[psgd_batch_locate(b, &local)];
+    psgd_mq_body<RB, RP, MODE, FAST>(it.x, it.err, it.cs, it.pktab, it.q, it.p, it.n, it.m, it.r, it.mod, alpha, hs, local);
+}
+
 // -------------------------------------------------------------- Q = X^T P ----
 // A workgroup of 8 waves owns 256 columns and a slab of rows.  A lane owns a column quad, wave v
 // takes rows v, v+8, ... of the slab (one contiguous kilobyte per row), the 8 waves meet in LDS.
@@ -175,15 +230,15 @@ constexpr int kMtpWaves = 8;
 constexpr int kMtpThreads = 64 * kMtpWaves;
 
 template <int RP, bool FAST>
-__global__ void __launch_bounds__(kMtpThreads)
-psgd_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, float* __restrict__ out, int64_t n, int m,
-                int r, int rows_per_slab)
+__device__ __forceinline__ void
+psgd_mtp_body(const float* __restrict__ x, const float* __restrict__ p, float* __restrict__ out, int64_t n, int m,
+              int r, int rows_per_slab, int bx, int by)
 {
     constexpr int CH = RP < 4 ? RP : 4;            // ranks reduced per LDS round
     __shared__ float red[kMtpWaves][CH][256];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int c0 = blockIdx.x * 256 + lane * 4;    // first column of my quad
-    const int64_t i0 = (int64_t)blockIdx.y * rows_per_slab;
+    const int c0 = bx * 256 + lane * 4;            // first column of my quad
+    const int64_t i0 = (int64_t)by * rows_per_slab;
     const int64_t i1 = i0 + rows_per_slab < n ? i0 + rows_per_slab : n;
     float acc[4][RP];
 #pragma unroll
@@ -233,7 +288,7 @@ psgd_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, float*
             }
         }
     }
-    float* dst = out + (int64_t)blockIdx.y * m * r;   // partial of this slab (or Q itself with one slab)
+    float* dst = out + (int64_t)by * m * r;           // partial of this slab (or Q itself with one slab)
 #pragma unroll
     for (int cb = 0; cb < RP; cb += CH) {
         if (cb) __syncthreads();
@@ -243,7 +298,7 @@ psgd_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, float*
             for (int k = 0; k < 4; ++k) red[wave][c][lane * 4 + k] = acc[k][cb + c];
         __syncthreads();
         if (threadIdx.x < 256) {
-            const int col = blockIdx.x * 256 + threadIdx.x;
+            const int col = bx * 256 + threadIdx.x;
             float s[CH];
 #pragma unroll
             for (int c = 0; c < CH; ++c) {
@@ -265,11 +320,37 @@ psgd_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, float*
     }
 }
 
-// out[i] = sum over slabs of partial[s][i], slabs in ascending order
-__global__ void __launch_bounds__(256)
-psgd_sum_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, int64_t count, int slabs)
+template <int RP, bool FAST>
+__global__ void __launch_bounds__(kMtpThreads)
+psgd_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, float* __restrict__ out, int64_t n, int m,
+                int r, int rows_per_slab)
 {
-    int64_t i = blockIdx.x * (int64_t)256 + threadIdx.x;
+    psgd_mtp_body<RP, FAST>(x, p, out, n, m, r, rows_per_slab, (int)blockIdx.x, (int)blockIdx.y);
+}
+
+struct MtpItem {
+    const float* x;
+    const float* p;
+    float* out;
+    int64_t n;
+    int m, r, rows_per_slab, col_tiles;
+};
+
+template <int RP, bool FAST>
+__global__ void __launch_bounds__(kMtpThreads)
+psgd_mtp_batch_kernel(PsgdBatch<MtpItem> b)
+{
+    int local;
+    const MtpItem& it = b.item[psgd_batch_locate(b, &local)];
+    psgd_mtp_body<RP, FAST>(it.x, it.p, it.out, it.n, it.m, it.r, it.rows_per_slab, local % it.col_tiles,
+                            local / it.col_tiles);
+}
+
+// out[i] = sum over slabs of partial[s][i], slabs in ascending order
+__device__ __forceinline__ void
+psgd_sum_partials_body(const float* __restrict__ partial, float* __restrict__ out, int64_t count, int slabs, int bx)
+{
+    int64_t i = bx * (int64_t)256 + threadIdx.x;
     if (i >= count) return;
     float s = 0.f;
     int k = 0;
@@ -284,18 +365,39 @@ psgd_sum_partials_kernel(const float* __restrict__ partial, float* __restrict__ 
     out[i] = s;
 }
 
+__global__ void __launch_bounds__(256)
+psgd_sum_partials_kernel(const float* __restrict__ partial, float* __restrict__ out, int64_t count, int slabs)
+{
+    psgd_sum_partials_body(partial, out, count, slabs, (int)blockIdx.x);
+}
+
+struct SumItem {
+    const float* partial;
+    float* out;
+    int64_t count;
+    int slabs;
+};
+
+__global__ void __launch_bounds__(256)
+psgd_sum_partials_batch_kernel(PsgdBatch<SumItem> b)
+{
+    int local;
+    const SumItem& it = b.item[psgd_batch_locate(b, &local)];
+    psgd_sum_partials_body(it.partial, it.out, it.count, it.slabs, local);
+}
+
 // ------------------------------------------------------------ M = P Q^T ----
 // MODE 0: write M.  MODE 1: also write the dense residual E = X - M (X = what M held on entry).
 // A thread owns a column quad (its 4 x r slice of Q stays in registers), the workgroup walks a slab
 // of rows; the row of P is uniform over the workgroup.
 template <int RP, int MODE, bool FAST>
-__global__ void __launch_bounds__(256)
-psgd_pqt_kernel(float* __restrict__ x, float* __restrict__ err, const float* __restrict__ p,
-                const float* __restrict__ q, int64_t n, int m, int r, int rows_per_slab)
+__device__ __forceinline__ void
+psgd_pqt_body(float* __restrict__ x, float* __restrict__ err, const float* __restrict__ p,
+              const float* __restrict__ q, int64_t n, int m, int r, int rows_per_slab, int bx, int by)
 {
-    const int c0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+    const int c0 = (bx * 256 + threadIdx.x) * 4;
     if (c0 >= m) return;
-    const int64_t i0 = (int64_t)blockIdx.y * rows_per_slab;
+    const int64_t i0 = (int64_t)by * rows_per_slab;
     const int64_t i1 = i0 + rows_per_slab < n ? i0 + rows_per_slab : n;
     float qf[4][RP];
     if (FAST) {
@@ -357,6 +459,33 @@ psgd_pqt_kernel(float* __restrict__ x, float* __restrict__ err, const float* __r
     }
 }
 
+template <int RP, int MODE, bool FAST>
+__global__ void __launch_bounds__(256)
+psgd_pqt_kernel(float* __restrict__ x, float* __restrict__ err, const float* __restrict__ p,
+                const float* __restrict__ q, int64_t n, int m, int r, int rows_per_slab)
+{
+    psgd_pqt_body<RP, MODE, FAST>(x, err, p, q, n, m, r, rows_per_slab, (int)blockIdx.x, (int)blockIdx.y);
+}
+
+struct PqtItem {
+    float* x;
+    float* err;
+    const float* p;
+    const float* q;
+    int64_t n;
+    int m, r, rows_per_slab, col_tiles;
+};
+
+template <int RP, int MODE, bool FAST>
+__global__ void __launch_bounds__(256)
+psgd_pqt_batch_kernel(PsgdBatch<PqtItem> b)
+{
+    int local;
+    const PqtItem& it = b.item[psgd_batch_locate(b, &local)];
+    psgd_pqt_body<RP, MODE, FAST>(it.x, it.err, it.p, it.q, it.n, it.m, it.r, it.rows_per_slab, local % it.col_tiles,
+                                  local / it.col_tiles);
+}
+
 // Front of the row-list sketch kernel: the value to sketch is the residual X - P Q^T, and M is
 // overwritten with P Q^T on the way (powerSGD_hook.py:551,563-564).
 template <int RP, bool FAST>
@@ -371,48 +500,48 @@ struct ListPsgdResidual {
     {
         float* base = x + row0 * d;
         if (FAST) {
-            const int d4 = d >> 2, total4 = rows * d4;
-            int row = threadIdx.x / d4, c4 = threadIdx.x - row * d4;
-            const int srow = kConefRowlistThreads / d4, sc = kConefRowlistThreads - srow * d4;
-            constexpr int U = RP <= 8 ? 4 : 2;         // quads in flight per thread
-            for (int t0 = threadIdx.x; t0 < total4; t0 += U * kConefRowlistThreads) {
-                float xv[U][4], flat[U][4 * RP], pr[U][RP];
+            // A thread owns column quads c4 = t, t + 256, ... and walks the tile's rows with the
+            // quad's slice of Q (4 x RP floats) in registers: Q is read once per quad and tile, not
+            // once per element.  Two rows are in flight; the row of P is uniform over the workgroup.
+            // Narrow matrices (fewer quads than threads) split the rows over thread groups instead.
+            const int d4 = d >> 2;
+            const int lanes = d4 < kConefRowlistThreads ? d4 : kConefRowlistThreads;
+            const int groups = kConefRowlistThreads / lanes, grp = threadIdx.x / lanes;
+            for (int c4 = threadIdx.x - grp * lanes; c4 < d4 && grp < groups; c4 += lanes) {
+                float flat[4 * RP];
 #pragma unroll
-                for (int u = 0; u < U; ++u) {           // past the end: a valid address, result unused
-                    const bool in = t0 + u * kConefRowlistThreads < total4;
-                    const int t = in ? t0 + u * kConefRowlistThreads : total4 - 1;
-                    const int cq = in ? c4 : 0, rq = in ? row : 0;
-                    ld4(base + 4 * t, xv[u]);
+                for (int v = 0; v < RP; ++v) ld4(q + (int64_t)c4 * 4 * RP + 4 * v, flat + 4 * v);
+                for (int rw = 2 * grp; rw < rows; rw += 2 * groups) {
+                    const int r1 = rw + 1 < rows ? rw + 1 : rw;
+                    float x0[4], x1[4], p0[RP], p1[RP];
+                    ld4(base + (int64_t)rw * d + 4 * c4, x0);
+                    ld4(base + (int64_t)r1 * d + 4 * c4, x1);
+                    const float* pa = p + (row0 + rw) * RP;
+                    const float* pb = p + (row0 + r1) * RP;
 #pragma unroll
-                    for (int v = 0; v < RP; ++v) ld4(q + (int64_t)cq * 4 * RP + 4 * v, flat[u] + 4 * v);
-                    const float* pi = p + (row0 + rq) * RP;
-                    if (RP >= 4) {
-#pragma unroll
-                        for (int v = 0; v < RP / 4; ++v) ld4(pi + 4 * v, pr[u] + 4 * v);
-                    } else {
-#pragma unroll
-                        for (int c = 0; c < RP; ++c) pr[u][c] = pi[c];
+                    for (int c = 0; c < RP; ++c) {
+                        p0[c] = pa[c];
+                        p1[c] = pb[c];
                     }
-                    row += srow;
-                    c4 += sc;
-                    if (c4 >= d4) {
-                        c4 -= d4;
-                        ++row;
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int t = t0 + u * kConefRowlistThreads;
-                    if (t >= total4) break;
-                    float mh[4] = {0.f, 0.f, 0.f, 0.f}, v[4];
+                    float m0[4] = {0.f, 0.f, 0.f, 0.f}, m1[4] = {0.f, 0.f, 0.f, 0.f}, v0[4], v1[4];
 #pragma unroll
                     for (int c = 0; c < RP; ++c)
 #pragma unroll
-                        for (int k = 0; k < 4; ++k) mh[k] = fmaf(pr[u][c], flat[u][k * RP + c], mh[k]);
+                        for (int k = 0; k < 4; ++k) {
+                            m0[k] = fmaf(p0[c], flat[k * RP + c], m0[k]);
+                            m1[k] = fmaf(p1[c], flat[k * RP + c], m1[k]);
+                        }
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) v[k] = __fsub_rn(xv[u][k], mh[k]);
-                    st4(base + 4 * t, mh);
-                    st4(vals + 4 * t, v);
+                    for (int k = 0; k < 4; ++k) {
+                        v0[k] = __fsub_rn(x0[k], m0[k]);
+                        v1[k] = __fsub_rn(x1[k], m1[k]);
+                    }
+                    st4(base + (int64_t)rw * d + 4 * c4, m0);
+                    st4(vals + rw * d + 4 * c4, v0);
+                    if (rw + 1 < rows) {
+                        st4(base + (int64_t)r1 * d + 4 * c4, m1);
+                        st4(vals + r1 * d + 4 * c4, v1);
+                    }
                 }
             }
         } else {
@@ -1431,6 +1560,404 @@ int conef_gram_schmidt_batch_f32(float* const* mats, const int64_t* rows, const 
         if (rc != CONEF_OK) return rc;
     }
     return CONEF_OK;
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------ batch dispatch ----
+namespace {
+
+// Launches `table` (workgroup counts in `blocks`) in runs of kPsgdBatchMax with `go(batch, grid)`.
+template <typename Item, typename Go>
+int run_batches(const std::vector<Item>& table, const std::vector<int>& blocks, Go go)
+{
+    size_t k = 0;
+    while (k < table.size()) {
+        PsgdBatch<Item> b;
+        int nb = 0, total = 0;
+        while (k < table.size() && nb < kPsgdBatchMax) {
+            b.item[nb] = table[k];
+            b.first[nb] = total;
+            total += blocks[k];
+            ++nb;
+            ++k;
+        }
+        b.first[nb] = total;
+        b.count = nb;
+        if (total > 0) go(b, total);
+    }
+    return (int)hipGetLastError();
+}
+
+inline bool item_ok(const ConefPsgdItem& it)
+{
+    return psgd_args_ok(it.n, it.m, it.r) && it.x && it.p && it.q;
+}
+
+inline const uint32_t* item_pktab(const ConefPsgdItem& it)
+{
+    const ConefPlanHeader* hp = (const ConefPlanHeader*)it.plan_host;
+    return (hp && it.plan_dev) ? (const uint32_t*)((const char*)it.plan_dev + hp->off_pk) : nullptr;
+}
+
+// rows per workgroup of the streaming P = X Q kernel inside a batch: four amortise the Q traffic
+// once the batch as a whole has workgroups to spare
+inline int mq_rows_per_wg(int64_t total_rows) { return total_rows / 4 >= 256 ? 4 : 1; }
+
+template <int MODE>
+int mq_batch(const ConefPsgdItem* items, int count, float alpha, int32_t a, int32_t b, void* workspace,
+             int64_t workspace_bytes, hipStream_t s)
+{
+    ConefSeeds hs = {a, b, a + 2, b + 3};
+    std::vector<char> done((size_t)count, 0);
+    for (int k = 0; k < count; ++k) {
+        if (done[(size_t)k]) continue;
+        const ConefPsgdItem& lead = items[k];
+        const int rp = rank_bound(lead.r);
+        auto fast_of = [&](const ConefPsgdItem& it) {
+            return it.r == rank_bound(it.r) && it.m % 4 == 0 && aligned16(it.x) && aligned16(it.q) &&
+                   (MODE != 1 || aligned16(it.err)) && (MODE != 2 || !item_pktab(it) || aligned16(item_pktab(it)));
+        };
+        const bool fast = fast_of(lead);
+        // ranks on the matrix cores, and sketch rows too wide for LDS, go one by one
+        auto alone = [&](const ConefPsgdItem& it) {
+            return rank_bound(it.r) >= 16 || (MODE == 2 && (size_t)4 * it.w * 4 + 4 * 4 * 8 * 4 > 64 * 1024);
+        };
+        if (alone(lead)) {
+            int rc = launch_mq<MODE>(lead.x, lead.err, lead.cs, item_pktab(lead), lead.q, lead.p, lead.n, lead.m, lead.r,
+                                     MODE == 2 ? lead.w : 1, alpha, hs, workspace, workspace_bytes, s);
+            if (rc != CONEF_OK) return rc;
+            done[(size_t)k] = 1;
+            continue;
+        }
+        std::vector<int> members;
+        int64_t rows = 0;
+        for (int j = k; j < count; ++j) {
+            if (done[(size_t)j] || alone(items[j]) || rank_bound(items[j].r) != rp || fast_of(items[j]) != fast) continue;
+            members.push_back(j);
+            rows += items[j].n;
+            done[(size_t)j] = 1;
+        }
+        const int rb = mq_rows_per_wg(rows);
+        std::vector<MqItem> table;
+        std::vector<int> blocks;
+        size_t lds = 0;
+        for (int j : members) {
+            const ConefPsgdItem& it = items[j];
+            MqItem t = {it.x, it.err, it.cs, item_pktab(it), it.q, it.p, it.n, (int)it.m, it.r,
+                        conef_make_mod(MODE == 2 ? it.w : 1)};
+            table.push_back(t);
+            blocks.push_back((int)((it.n + rb - 1) / rb));
+            size_t need = (size_t)4 * rb * rp * 4 + (MODE == 2 ? (size_t)rb * it.w * 4 : 0);
+            if (need > lds) lds = need;
+        }
+#define CONEF_MQB_GO(RB, RP, F)                                                                                    \
+    run_batches(table, blocks, [&](const PsgdBatch<MqItem>& bt, int grid) {                                        \
+        hipLaunchKernelGGL((psgd_mq_batch_kernel<RB, RP, MODE, F>), dim3((unsigned)grid), dim3(256), lds, s, bt, alpha, hs); \
+    })
+#define CONEF_MQB(RP)                                                  \
+    do {                                                               \
+        if (RP >= 16) break;                                           \
+        if (rb == 4) {                                                 \
+            if (fast) rc = CONEF_MQB_GO(4, (RP < 16 ? RP : 8), true);  \
+            else rc = CONEF_MQB_GO(4, (RP < 16 ? RP : 8), false);      \
+        } else {                                                       \
+            if (fast) rc = CONEF_MQB_GO(1, (RP < 16 ? RP : 8), true);  \
+            else rc = CONEF_MQB_GO(1, (RP < 16 ? RP : 8), false);      \
+        }                                                              \
+    } while (0)
+        int rc = CONEF_OK;
+        CONEF_RANK_SWITCH(lead.r, CONEF_MQB)
+#undef CONEF_MQB
+#undef CONEF_MQB_GO
+        if (rc != CONEF_OK) return rc;
+    }
+    return CONEF_OK;
+}
+
+// per item: slabs of the streaming Q = X^T P kernel and where its partials start in the workspace
+struct MtpPlan {
+    MtpShape g;
+    int64_t partial_off;    // floats; -1: one slab, the result goes straight to q
+};
+
+inline int64_t mtp_batch_layout(const ConefPsgdItem* items, int count, std::vector<MtpPlan>* plans)
+{
+    int64_t off = 0;
+    for (int k = 0; k < count; ++k) {
+        MtpPlan pl;
+        pl.g = mtp_shape(items[k].n, items[k].m);
+        pl.partial_off = -1;
+        if (rank_bound(items[k].r) < 16 && pl.g.slabs > 1) {
+            pl.partial_off = off;
+            off += ((int64_t)pl.g.slabs * items[k].m * items[k].r + 63) / 64 * 64;     // 256-byte aligned regions
+        }
+        if (plans) plans->push_back(pl);
+    }
+    return off;
+}
+
+int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    std::vector<MtpPlan> plans;
+    const int64_t floats = mtp_batch_layout(items, count, &plans);
+    int64_t single = 0;       // the matrix-core items run one by one and share the front of the workspace
+    for (int k = 0; k < count; ++k)
+        if (rank_bound(items[k].r) >= 16) {
+            int64_t b = conef_psgd_workspace_bytes(items[k].n, items[k].m, items[k].r);
+            if (b > single) single = b;
+        }
+    if ((floats > 0 || single > 0) && (!workspace || workspace_bytes < floats * 4 + single)) return CONEF_ERR_INVALID;
+    float* partial_base = (float*)((char*)workspace + single);
+    std::vector<char> done((size_t)count, 0);
+    std::vector<SumItem> sums;
+    std::vector<int> sum_blocks;
+    for (int k = 0; k < count; ++k) {
+        if (done[(size_t)k]) continue;
+        const ConefPsgdItem& lead = items[k];
+        const int rp = rank_bound(lead.r);
+        if (rp >= 16) {
+            int rc = conef_psgd_mtp_f32(lead.x, lead.p, lead.q, lead.n, lead.m, lead.r, workspace, single, (void*)s);
+            if (rc != CONEF_OK) return rc;
+            done[(size_t)k] = 1;
+            continue;
+        }
+        auto fast_of = [&](int j) {
+            const ConefPsgdItem& it = items[j];
+            const float* out = plans[(size_t)j].partial_off >= 0 ? partial_base + plans[(size_t)j].partial_off : it.q;
+            return it.r == rank_bound(it.r) && it.m % 4 == 0 && aligned16(it.x) && aligned16(it.p) && aligned16(out);
+        };
+        const bool fast = fast_of(k);
+        std::vector<MtpItem> table;
+        std::vector<int> blocks;
+        for (int j = k; j < count; ++j) {
+            if (done[(size_t)j] || rank_bound(items[j].r) != rp || fast_of(j) != fast) continue;
+            const ConefPsgdItem& it = items[j];
+            const MtpPlan& pl = plans[(size_t)j];
+            float* out = pl.partial_off >= 0 ? partial_base + pl.partial_off : it.q;
+            MtpItem t = {it.x, it.p, out, it.n, (int)it.m, it.r, pl.g.rows_per_slab, pl.g.col_tiles};
+            table.push_back(t);
+            blocks.push_back(pl.g.col_tiles * pl.g.slabs);
+            if (pl.partial_off >= 0) {
+                int64_t cnt = it.m * it.r;
+                SumItem si = {out, it.q, cnt, pl.g.slabs};
+                sums.push_back(si);
+                sum_blocks.push_back((int)((cnt + 255) / 256));
+            }
+            done[(size_t)j] = 1;
+        }
+        int rc = CONEF_OK;
+#define CONEF_MTPB(RP)                                                                                              \
+    do {                                                                                                            \
+        if (RP >= 16) break;                                                                                        \
+        if (fast) rc = run_batches(table, blocks, [&](const PsgdBatch<MtpItem>& bt, int grid) {                     \
+            hipLaunchKernelGGL((psgd_mtp_batch_kernel<(RP < 16 ? RP : 8), true>), dim3((unsigned)grid), dim3(kMtpThreads), 0, s, bt); \
+        });                                                                                                         \
+        else rc = run_batches(table, blocks, [&](const PsgdBatch<MtpItem>& bt, int grid) {                          \
+            hipLaunchKernelGGL((psgd_mtp_batch_kernel<(RP < 16 ? RP : 8), false>), dim3((unsigned)grid), dim3(kMtpThreads), 0, s, bt); \
+        });                                                                                                         \
+    } while (0)
+        CONEF_RANK_SWITCH(lead.r, CONEF_MTPB)
+#undef CONEF_MTPB
+        if (rc != CONEF_OK) return rc;
+    }
+    if (!sums.empty()) {
+        int rc = run_batches(sums, sum_blocks, [&](const PsgdBatch<SumItem>& bt, int grid) {
+            hipLaunchKernelGGL(psgd_sum_partials_batch_kernel, dim3((unsigned)grid), dim3(256), 0, s, bt);
+        });
+        if (rc != CONEF_OK) return rc;
+    }
+    return CONEF_OK;
+}
+
+template <int RP, bool FAST>
+struct RowlistResidualItem {
+    ListPsgdResidual<RP, FAST> front;
+    ConefRowlistView plan;
+    const float* cs_in;
+    float* cs_out;
+    int64_t n;
+    int d, w, rb;
+};
+
+template <int RP, bool FAST>
+__global__ void __launch_bounds__(kConefRowlistThreads)
+psgd_residual_rowlist_batch_kernel(PsgdBatch<RowlistResidualItem<RP, FAST>> b, double one_minus_beta)
+{
+    int local;
+    const RowlistResidualItem<RP, FAST>& it = b.item[psgd_batch_locate(b, &local)];
+    conef_rowlist_body<float, ListPsgdResidual<RP, FAST>>(it.front, it.plan, it.cs_in, it.cs_out, it.n, it.d, it.w, it.rb,
+                                                          one_minus_beta, local);
+}
+
+template <int RP, bool FAST>
+int pqt_sketch_group(const ConefPsgdItem* items, const std::vector<int>& members, float beta, hipStream_t s)
+{
+    std::vector<RowlistResidualItem<RP, FAST>> table;
+    std::vector<int> blocks;
+    size_t lds = 0;
+    for (int j : members) {
+        const ConefPsgdItem& it = items[j];
+        ConefRowlistShape shape;
+        if (!conef_rowlist_shape(it.n, it.m, it.w, false, &shape, (int)members.size())) return CONEF_ERR_INVALID;
+        RowlistResidualItem<RP, FAST> t = {{it.x, it.p, it.q, it.r},
+                                           conef_rowlist_view((const ConefPlanHeader*)it.plan_host, it.plan_dev),
+                                           it.cs, it.cs, it.n, (int)it.m, it.w, shape.rb};
+        table.push_back(t);
+        blocks.push_back((int)shape.tiles);
+        if (shape.lds > lds) lds = shape.lds;
+    }
+    auto kern = psgd_residual_rowlist_batch_kernel<RP, FAST>;
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    const double omb = 1. - (double)beta;
+    return run_batches(table, blocks, [&](const PsgdBatch<RowlistResidualItem<RP, FAST>>& bt, int grid) {
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kConefRowlistThreads), lds, s, bt, omb);
+    });
+}
+
+int pqt_batch(const ConefPsgdItem* items, int count, int mode, float beta, int32_t a, int32_t b, hipStream_t s)
+{
+    std::vector<char> done((size_t)count, 0);
+    for (int k = 0; k < count; ++k) {
+        if (done[(size_t)k]) continue;
+        const ConefPsgdItem& lead = items[k];
+        const int rp = rank_bound(lead.r);
+        if (rp >= 16 || mode == 2) {
+            if (mode == 2 && rp < 16) {
+                // residual sketch on row-list plans: items of one rank class share launches
+                auto fast_of = [&](const ConefPsgdItem& it) {
+                    return it.r == rank_bound(it.r) && it.m % 4 == 0 && aligned16(it.x) && aligned16(it.q) && aligned16(it.p);
+                };
+                const bool fast = fast_of(lead);
+                std::vector<int> members;
+                for (int j = k; j < count; ++j) {
+                    if (done[(size_t)j] || rank_bound(items[j].r) != rp || fast_of(items[j]) != fast) continue;
+                    const ConefPlanHeader* hp = (const ConefPlanHeader*)items[j].plan_host;
+                    if (!conef_plan_matches(hp, items[j].n, items[j].m, items[j].w, a, b) || hp->kind != kConefPlanRowlist ||
+                        !items[j].plan_dev || !items[j].cs)
+                        return CONEF_ERR_INVALID;
+                    members.push_back(j);
+                    done[(size_t)j] = 1;
+                }
+                int rc = CONEF_ERR_INVALID;
+#define CONEF_PQS(RP)                                                                  \
+    do {                                                                               \
+        if (RP >= 16) break;                                                           \
+        if (fast) rc = pqt_sketch_group<(RP < 16 ? RP : 8), true>(items, members, beta, s);  \
+        else rc = pqt_sketch_group<(RP < 16 ? RP : 8), false>(items, members, beta, s);      \
+    } while (0)
+                CONEF_RANK_SWITCH(lead.r, CONEF_PQS)
+#undef CONEF_PQS
+                if (rc != CONEF_OK) return rc;
+                continue;
+            }
+            int rc;
+            if (mode == 2)
+                rc = conef_psgd_pqt_conef_planned_f32(lead.x, lead.p, lead.q, lead.cs, lead.cs, lead.plan_host, lead.plan_dev,
+                                                      lead.n, lead.m, lead.r, lead.w, beta, a, b, (void*)s);
+            else
+                rc = launch_pqt(lead.x, mode == 1 ? lead.err : nullptr, lead.p, lead.q, lead.n, lead.m, lead.r, s);
+            if (rc != CONEF_OK) return rc;
+            done[(size_t)k] = 1;
+            continue;
+        }
+        auto fast_of = [&](const ConefPsgdItem& it) {
+            return it.r == rank_bound(it.r) && it.m % 4 == 0 && aligned16(it.x) && aligned16(it.q) &&
+                   (mode != 1 || aligned16(it.err));
+        };
+        const bool fast = fast_of(lead);
+        std::vector<PqtItem> table;
+        std::vector<int> blocks;
+        for (int j = k; j < count; ++j) {
+            if (done[(size_t)j] || rank_bound(items[j].r) != rp || fast_of(items[j]) != fast) continue;
+            const ConefPsgdItem& it = items[j];
+            // about a thousand workgroups for the batch as a whole, slabs of at least four rows
+            int64_t col_tiles = (it.m + 1023) / 1024;
+            int64_t slabs = (256 + col_tiles - 1) / col_tiles;
+            int64_t rps = (it.n + slabs - 1) / slabs;
+            if (rps < 4) rps = 4;
+            slabs = (it.n + rps - 1) / rps;
+            PqtItem t = {it.x, mode == 1 ? it.err : nullptr, it.p, it.q, it.n, (int)it.m, it.r, (int)rps, (int)col_tiles};
+            table.push_back(t);
+            blocks.push_back((int)(col_tiles * slabs));
+            done[(size_t)j] = 1;
+        }
+        int rc = CONEF_OK;
+#define CONEF_PQB_GO(RP, MODE, F)                                                                                  \
+    run_batches(table, blocks, [&](const PsgdBatch<PqtItem>& bt, int grid) {                                       \
+        hipLaunchKernelGGL((psgd_pqt_batch_kernel<RP, MODE, F>), dim3((unsigned)grid), dim3(256), 0, s, bt);       \
+    })
+#define CONEF_PQB(RP)                                                          \
+    do {                                                                       \
+        if (RP >= 16) break;                                                   \
+        if (mode == 1) {                                                       \
+            if (fast) rc = CONEF_PQB_GO((RP < 16 ? RP : 8), 1, true);          \
+            else rc = CONEF_PQB_GO((RP < 16 ? RP : 8), 1, false);              \
+        } else {                                                               \
+            if (fast) rc = CONEF_PQB_GO((RP < 16 ? RP : 8), 0, true);          \
+            else rc = CONEF_PQB_GO((RP < 16 ? RP : 8), 0, false);              \
+        }                                                                      \
+    } while (0)
+        CONEF_RANK_SWITCH(lead.r, CONEF_PQB)
+#undef CONEF_PQB
+#undef CONEF_PQB_GO
+        if (rc != CONEF_OK) return rc;
+    }
+    return CONEF_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t conef_psgd_batch_workspace_bytes(const ConefPsgdItem* items, int32_t count)
+{
+    if (count < 0 || (count > 0 && !items)) return -1;
+    int64_t single = 256;
+    for (int k = 0; k < count; ++k) {
+        if (!psgd_args_ok(items[k].n, items[k].m, items[k].r)) return -1;
+        int64_t b = conef_psgd_workspace_bytes(items[k].n, items[k].m, items[k].r);
+        if (b > single) single = b;
+    }
+    return conef_align256(single) + conef_align256(4 * mtp_batch_layout(items, count, nullptr));
+}
+
+int conef_psgd_mq_batch_f32(const ConefPsgdItem* items, int32_t count, int32_t mode, float alpha, int32_t a, int32_t b,
+                            void* workspace, int64_t workspace_bytes, void* stream)
+{
+    if (count < 0 || (count > 0 && !items) || mode < 0 || mode > 2) return CONEF_ERR_INVALID;
+    for (int k = 0; k < count; ++k) {
+        const ConefPsgdItem& it = items[k];
+        if (!item_ok(it) || (mode == 1 && !it.err) || (mode == 2 && (!it.cs || it.w < 1 || it.w > (1 << 30))))
+            return CONEF_ERR_INVALID;
+        if (mode == 2 && it.plan_host && !conef_plan_matches((const ConefPlanHeader*)it.plan_host, it.n, it.m, it.w, a, b))
+            return CONEF_ERR_INVALID;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    if (mode == 0) return mq_batch<0>(items, count, 0.f, a, b, workspace, workspace_bytes, s);
+    if (mode == 1) return mq_batch<1>(items, count, 0.f, a, b, workspace, workspace_bytes, s);
+    return mq_batch<2>(items, count, alpha, a, b, workspace, workspace_bytes, s);
+}
+
+int conef_psgd_mtp_batch_f32(const ConefPsgdItem* items, int32_t count, void* workspace, int64_t workspace_bytes,
+                             void* stream)
+{
+    if (count < 0 || (count > 0 && !items)) return CONEF_ERR_INVALID;
+    for (int k = 0; k < count; ++k)
+        if (!item_ok(items[k])) return CONEF_ERR_INVALID;
+    return mtp_batch(items, count, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int conef_psgd_pqt_batch_f32(const ConefPsgdItem* items, int32_t count, int32_t mode, float beta, int32_t a, int32_t b,
+                             void* stream)
+{
+    if (count < 0 || (count > 0 && !items) || mode < 0 || mode > 2) return CONEF_ERR_INVALID;
+    for (int k = 0; k < count; ++k)
+        if (!item_ok(items[k]) || (mode == 1 && !items[k].err)) return CONEF_ERR_INVALID;
+    return pqt_batch(items, count, mode, beta, a, b, (hipStream_t)stream);
 }
 
 // dense error feedback on the parts of a bucket that are not compressed: x += e; e = 0

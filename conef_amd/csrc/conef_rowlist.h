@@ -46,11 +46,13 @@ inline size_t conef_rowlist_lds(int rb, int64_t d, int32_t w, bool cells)
 
 // Rows per tile: about 32 KB of values (several tiles per CU), but no more than leaves a
 // thousand tiles for the 256 CUs.
-inline bool conef_rowlist_shape(int64_t n, int64_t d, int32_t w, bool cells, ConefRowlistShape* s)
+// `companions`: matrices of about this size that share the launch (a batch leaves enough tiles
+// for the machine with taller tiles per matrix).
+inline bool conef_rowlist_shape(int64_t n, int64_t d, int32_t w, bool cells, ConefRowlistShape* s, int companions = 1)
 {
     if (d < 1 || d > kConefRowlistMaxCols || n < 1 || w < 1) return false;
     int64_t rb = 8192 / d;
-    if (rb > n / 1024) rb = n / 1024;
+    if (rb > n * companions / 1024) rb = n * companions / 1024;
     if (rb > 16) rb = 16;
     if (rb < 1) rb = 1;
     while (rb > 1 && conef_rowlist_lds((int)rb, d, w, cells) > 64 * 1024) --rb;
@@ -226,16 +228,16 @@ __device__ __forceinline__ void conef_copy_words_to_lds(uint32_t* dst, const uin
 }
 
 template <typename CsT, typename Front>
-__global__ void __launch_bounds__(kConefRowlistThreads)
-conef_rowlist_kernel(Front front, ConefRowlistView plan, const CsT* cs_in, CsT* cs_out, int64_t n, int d, int w,
-                     int rb, double one_minus_beta)
+__device__ __forceinline__ void
+conef_rowlist_body(const Front& front, ConefRowlistView plan, const CsT* cs_in, CsT* cs_out, int64_t n, int d, int w,
+                   int rb, double one_minus_beta, int bx)
 {
     extern __shared__ float conef_rl[];
     float* vals = conef_rl;
     uint16_t* ent_l = reinterpret_cast<uint16_t*>(vals + ((rb * d + 3) & ~3));
     uint32_t* csr_l = reinterpret_cast<uint32_t*>(ent_l + ((d + 7) & ~7));
     float* cells = reinterpret_cast<float*>(csr_l + ((w + 1 + 3) & ~3));
-    const int64_t row0 = (int64_t)blockIdx.x * rb;
+    const int64_t row0 = (int64_t)bx * rb;
     const int rows = n - row0 < rb ? (int)(n - row0) : rb;
 
     // the bucket lists, two entries per load (the table is padded to a multiple of 256 bytes)
@@ -306,6 +308,14 @@ conef_rowlist_kernel(Front front, ConefRowlistView plan, const CsT* cs_in, CsT* 
             ++row;
         }
     }
+}
+
+template <typename CsT, typename Front>
+__global__ void __launch_bounds__(kConefRowlistThreads)
+conef_rowlist_kernel(Front front, ConefRowlistView plan, const CsT* cs_in, CsT* cs_out, int64_t n, int d, int w,
+                     int rb, double one_minus_beta)
+{
+    conef_rowlist_body<CsT, Front>(front, plan, cs_in, cs_out, n, d, w, rb, one_minus_beta, (int)blockIdx.x);
 }
 
 template <typename CsT, typename Front>

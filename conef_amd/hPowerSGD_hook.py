@@ -45,6 +45,7 @@ class hPowerSGDState(Checkpointable):
         "total_numel_after_compression",
         "compression_stats_logging_frequency",
         "next_stats_report",
+        "round_cache",
     ]
 
     def __init__(
@@ -82,6 +83,7 @@ class hPowerSGDState(Checkpointable):
         self.total_numel_after_compression = 0
         self.compression_stats_logging_frequency = max(1, compression_stats_logging_frequency)
         self.next_stats_report = 0
+        self.round_cache = {}            # per-bucket launch tables of the engine, rebuilt when a bucket changes
         self.use_error_compression = use_error_compression
         self.topk_ratio = topk_ratio
 

@@ -52,6 +52,7 @@ class PowerSGDState(Checkpointable):
         "total_numel_after_compression",
         "compression_stats_logging_frequency",
         "next_stats_report",
+        "round_cache",
         "batched_square_dict",
     ]
 
@@ -97,6 +98,7 @@ class PowerSGDState(Checkpointable):
         self.total_numel_after_compression = 0
         self.compression_stats_logging_frequency = max(1, compression_stats_logging_frequency)
         self.next_stats_report = 0
+        self.round_cache = {}            # per-bucket launch tables of the engine, rebuilt when a bucket changes
         self.use_error_compression = use_error_compression
         self.beta = beta
         self.sketch_size = sketch_size

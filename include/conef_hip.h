@@ -242,6 +242,39 @@ int conef_psgd_pqt_conef_planned_f32(float* x, const float* p, const float* q, c
                                      const void* plan_host, const void* plan_dev, int64_t n, int64_t m, int32_t r,
                                      int32_t w, float beta, int32_t a, int32_t b, void* stream);
 
+/* ---- all matrices of a bucket per launch -------------------------------------------------- */
+/* The tensors of a gradient bucket are independent of each other and most are too small to fill
+ * the GPU alone, so the three products also come as batch calls: one table entry per matrix
+ * (host array, read before the call returns), matrices of one kernel class share launches of up
+ * to 24, a workgroup finds its matrix from the table.  Results are those of the per-matrix calls.
+ * Replaces: the `for tensor, q, p in zip(...)` loops, powerSGD_hook.py:497-498,530-532,550-551,
+ * 561-564. */
+typedef struct ConefPsgdItem {
+    float* x;               /* the matrix [n,m], inside the bucket */
+    float* err;             /* dense error / residual [n,m], or NULL */
+    float* cs;              /* sketch [n,w] (updated in place by pqt mode 2), or NULL */
+    const void* plan_host;  /* row-list plan of the sketch (host and device copy), or NULL */
+    const void* plan_dev;
+    float* p;               /* [n,r] */
+    float* q;               /* [m,r] */
+    int64_t n, m;
+    int32_t r, w;
+} ConefPsgdItem;
+
+/* Bytes of workspace conef_psgd_mtp_batch_f32 needs for these items (sums across row slabs). */
+int64_t conef_psgd_batch_workspace_bytes(const ConefPsgdItem* items, int32_t count);
+/* mode 0: P = M Q.  mode 1: M += err first.  mode 2: M += alpha*unsketch(cs) first (bucket and
+ * sign from the plan's table when a plan is given).  Per item as conef_psgd_mq_f32 / _ef_ / _conef_. */
+int conef_psgd_mq_batch_f32(const ConefPsgdItem* items, int32_t count, int32_t mode, float alpha, int32_t a, int32_t b,
+                            void* workspace, int64_t workspace_bytes, void* stream);
+/* Q = M^T P for every item. */
+int conef_psgd_mtp_batch_f32(const ConefPsgdItem* items, int32_t count, void* workspace, int64_t workspace_bytes,
+                             void* stream);
+/* mode 0: M = P Q^T.  mode 1: err = M - P Q^T as well.  mode 2: cs = update(cs, M - P Q^T, beta) in
+ * place on the item's row-list plan (every item needs one) as well. */
+int conef_psgd_pqt_batch_f32(const ConefPsgdItem* items, int32_t count, int32_t mode, float beta, int32_t a, int32_t b,
+                             void* stream);
+
 /* Dense error feedback on a stretch of the bucket that is not compressed: x += err; err = 0
  * (the copy-minus-result of powerSGD_hook.py:558 is exactly zero there). */
 int conef_ef_passthrough_f32(float* x, float* err, int64_t count, void* stream);

@@ -231,6 +231,53 @@ def test_products_parity(oracle):
         np.testing.assert_array_equal(to_np(outm), to_np(Md))
 
 
+def test_batch_products_parity(oracle):
+    """All matrices of a bucket per launch: mixed shapes, ranks on both sides of the matrix-core
+    threshold, an unaligned matrix, dense error and plain modes - every matrix must come out as
+    the oracle's products of that matrix alone."""
+    from conef_amd import _lib
+    lib = _lib.load()
+    rng = np.random.RandomState(4)
+    specs = [(64, 576, 2, 0), (640, 1440, 4, 0), (1024, 1024, 8, 0), (13, 29, 3, 0), (300, 4096, 32, 0), (37, 4096, 8, 2),
+             (2049, 260, 4, 0), (16, 27, 2, 0), (5000, 64, 1, 0), (128, 128, 16, 0)] + [(96 + k, 200, 4, 0) for k in range(30)]
+    for mode in (0, 1):
+        items = (_lib.PsgdItem * len(specs))()
+        keep, host = [], []
+        for k, (n, m, r, off) in enumerate(specs):
+            M = rng.randn(n, m).astype(np.float32)
+            E = rng.randn(n, m).astype(np.float32)
+            Q = rng.randn(m, r).astype(np.float32)
+            Md = torch.zeros(n * m + off, device="cuda")[off:].view(n, m)
+            Md.copy_(torch.from_numpy(M))
+            Ed, Qd = torch.from_numpy(E).cuda(), torch.from_numpy(Q).cuda()
+            Pd = torch.empty(n, r, device="cuda")
+            it = items[k]
+            it.x, it.err, it.p, it.q, it.n, it.m, it.r, it.w = (Md.data_ptr(), Ed.data_ptr(), Pd.data_ptr(), Qd.data_ptr(),
+                                                                n, m, r, 1)
+            keep.append((Md, Ed, Qd, Pd))
+            host.append((M, E, Q))
+        ws = torch.empty(lib.conef_psgd_batch_workspace_bytes(items, len(specs)), dtype=torch.uint8, device="cuda")
+        assert lib.conef_psgd_mq_batch_f32(items, len(specs), mode, 0.0, 1, 1, ws.data_ptr(), ws.numel(), 0) == 0
+        xs = []
+        for (Md, Ed, Qd, Pd), (M, E, Q), spec in zip(keep, host, specs):
+            X = M + E if mode == 1 else M
+            np.testing.assert_array_equal(to_np(Md), X)
+            assert_close(Pd, oracle.mq(X, Q), what="batch MQ %s mode %d" % (spec, mode))
+            xs.append(X)
+        # Q = M^T P with the P just computed
+        assert lib.conef_psgd_mtp_batch_f32(items, len(specs), ws.data_ptr(), ws.numel(), 0) == 0
+        for (Md, Ed, Qd, Pd), X, spec in zip(keep, xs, specs):
+            assert_close(Qd, oracle.mtp(X, to_np(Pd)), what="batch MtP %s" % (spec,))
+        assert lib.conef_psgd_pqt_batch_f32(items, len(specs), mode, 0.0, 1, 1, 0) == 0
+        for (Md, Ed, Qd, Pd), X, spec in zip(keep, xs, specs):
+            low = oracle.pqt(to_np(Pd), to_np(Qd))
+            assert_close(Md, low, what="batch PQt %s" % (spec,))
+            if mode == 1:
+                np.testing.assert_array_equal(to_np(Ed), X - to_np(Md))
+    assert lib.conef_psgd_mq_batch_f32(items, len(specs), 3, 0.0, 1, 1, 0, 0, 0) == -1       # unknown mode
+    assert lib.conef_psgd_pqt_batch_f32(items, len(specs), 2, 0.9, 1, 1, 0) == -1            # mode 2 needs plans
+
+
 def test_products_with_sketch_on_a_plan(oracle):
     """P = (M + alpha unsketch) Q and the residual sketch after M = P Q^T, on row-list plans: the
     sketch must come out bit for bit (same terms, same order as the serial definition)."""
