@@ -10,6 +10,7 @@
 // error-feedback add (before the first product) and the residual (after the last) are fused into
 // the passes that touch M anyway.  Sums that cross workgroups meet through a caller-provided
 // workspace in a fixed order: no atomics, results do not change from run to run.
+#include <type_traits>
 #include <vector>
 
 #include "conef_device.h"
@@ -99,7 +100,11 @@ psgd_mq_body(float* __restrict__ x, const float* __restrict__ err, const float* 
 
     if (FAST) {
         const int m4 = m >> 2;
-        constexpr int U = (RB * RP <= 16) ? 4 : 2;      // column quads in flight per thread
+        constexpr int UMAX = (RB * RP <= 16) ? 4 : 2;   // column quads in flight per thread, at most
+        // narrow matrices do not have that many quads per thread: fewer in flight rather than
+        // clamped duplicates of the last quad
+        auto sweep = [&](auto u_tag) {
+        constexpr int U = decltype(u_tag)::value;
         for (int j0 = threadIdx.x; j0 < m4; j0 += U * 256) {
             float xv[U][RB][4];
             float qf[U][4 * RP];                        // Q rows 4j..4j+3: 4*RP consecutive floats
@@ -156,6 +161,10 @@ psgd_mq_body(float* __restrict__ x, const float* __restrict__ err, const float* 
                         for (int c = 0; c < RP; ++c) acc[a][c] = fmaf(xv[u][a][k], qf[u][k * RP + c], acc[a][c]);
             }
         }
+        };
+        if (m4 <= 256) sweep(std::integral_constant<int, 1>());
+        else if (m4 <= 512 || UMAX == 2) sweep(std::integral_constant<int, 2>());
+        else sweep(std::integral_constant<int, UMAX>());
     } else {
         for (int k = threadIdx.x; k < m; k += 256) {
             float qk[RP];
