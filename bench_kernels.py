@@ -234,7 +234,7 @@ def main():
         kk = max(1, int(0.2 * numel))
         ws_bytes = lib.conef_topk_workspace_bytes(numel)
         nset = copies(4 * numel, hi=16)
-        timeit("topk_sparsify_f32 %d elements, keep 20%%" % numel, 7 * 4 * numel,
+        timeit("topk_sparsify_f32 %d elements, keep 20%%" % numel, 8 * numel,
                lambda numel=numel, ws_bytes=ws_bytes, nset=nset: [(torch.randn(numel, device=dev),
                                                                    torch.empty(ws_bytes, dtype=torch.uint8, device=dev))
                                                                   for _ in range(nset)],

@@ -5,80 +5,132 @@
 // positions and so leaves ties open; here ties on the threshold magnitude keep the lowest flat
 // indices, which makes the result a function of the input alone.
 //
-// Selection is a most-significant-digit radix select on the magnitude bits (a non-negative
-// float orders like its bit pattern): four 8-bit histogram passes narrow the k-th largest key,
-// then one counting pass and one filtering pass resolve ties in index order.  Nothing returns to
-// the host between passes; the running (prefix, remaining) pair lives in the workspace.
+// Selection is a most-significant-digit radix select on the 31 magnitude bits (a non-negative
+// float orders like its bit pattern) in three histogram passes of 11, 11 and 9 bits.  Choosing the
+// digit that holds the k-th largest key is not a launch of its own: every workgroup of the next
+// pass does it from the finished histogram before it starts (2048 counters, one suffix scan).
+// If more keys equal the threshold than may be kept, two counting passes and an ordered filter
+// resolve the ties in index order; otherwise those two launches return at once and the filter
+// keeps every key at or above the threshold.  Nothing returns to the host between passes.
 #include "conef_device.h"
 
 namespace {
 
-constexpr int kBins = 256;
+constexpr int kPasses = 3;
+constexpr int kDigitBits[kPasses] = {11, 11, 9};
+constexpr int kDigitShift[kPasses] = {20, 9, 0};
+constexpr int kBins = 2048;          // bins of the widest digit
 constexpr int kFilterChunk = 1024;   // elements per workgroup iteration in the ordered passes
 
 struct TopkState {
-    uint32_t prefix;      // selected high digits so far
-    uint32_t remaining;   // how many keys to take among those matching the prefix
-    uint32_t hist[4][kBins];
+    uint32_t k;
+    uint32_t prefix[kPasses];       // prefix[p]: selected digits of passes 0..p, written by pass p + 1
+    uint32_t remaining[kPasses];    // how many keys to take among those matching prefix[p]
+    uint32_t ties[kPasses];         // keys that match prefix[p] exactly in their high digits
+    uint32_t pad[6];
+    uint32_t hist[kPasses][kBins];
 };
 
 __device__ __forceinline__ uint32_t mag_key(float v) { return __float_as_uint(v) & 0x7fffffffu; }
 
 __global__ void topk_init_kernel(TopkState* st, uint32_t k)
 {
-    for (int i = threadIdx.x; i < 4 * kBins; i += blockDim.x) (&st->hist[0][0])[i] = 0u;
-    if (threadIdx.x == 0) {
-        st->prefix = 0u;
-        st->remaining = k;
+    for (int i = threadIdx.x; i < kPasses * kBins; i += blockDim.x) (&st->hist[0][0])[i] = 0u;
+    if (threadIdx.x == 0) st->k = k;
+}
+
+// What pass `p` selected, from its finished histogram: the digit holding the k-th largest key
+// among those matching the earlier digits.  Every thread of a 256-thread workgroup returns the
+// same (prefix, remaining, ties); workgroup 0 also leaves them in the state for the next kernel.
+__device__ __forceinline__ void topk_resolve(TopkState* st, int p, uint32_t* prefix, uint32_t* remaining, uint32_t* ties)
+{
+    __shared__ uint32_t wave_sum[4];
+    __shared__ uint32_t picked[3];
+    const uint32_t before_prefix = p == 0 ? 0u : st->prefix[p - 1];
+    const uint32_t before_remaining = p == 0 ? st->k : st->remaining[p - 1];
+    const int bins = 1 << kDigitBits[p], per = bins / 256;          // 8, 8, 2 bins per thread
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    uint32_t cnt[8];
+    uint32_t mine = 0;
+    for (int b = 0; b < per; ++b) {
+        cnt[b] = st->hist[p][threadIdx.x * per + b];
+        mine += cnt[b];
     }
+    // suffix sums over threads: keys in digits above mine
+    uint32_t incl = mine;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        uint32_t t = __shfl_down(incl, off, 64);
+        if (lane + off < 64) incl += t;
+    }
+    if (lane == 0) wave_sum[wave] = incl;
+    __syncthreads();
+    uint32_t above = incl - mine;
+    for (int wv = wave + 1; wv < 4; ++wv) above += wave_sum[wv];
+    // exactly one (thread, bin) satisfies above < remaining <= above + count
+    for (int b = per - 1; b >= 0; --b) {
+        if (above < before_remaining && before_remaining <= above + cnt[b]) {
+            picked[0] = (before_prefix << kDigitBits[p]) | (uint32_t)(threadIdx.x * per + b);
+            picked[1] = before_remaining - above;
+            picked[2] = cnt[b];
+        }
+        above += cnt[b];
+    }
+    __syncthreads();
+    *prefix = picked[0];
+    *remaining = picked[1];
+    *ties = picked[2];
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        st->prefix[p] = picked[0];
+        st->remaining[p] = picked[1];
+        st->ties[p] = picked[2];
+    }
+    __syncthreads();
 }
 
 __global__ void __launch_bounds__(256)
 topk_hist_kernel(const float* __restrict__ x, int64_t numel, TopkState* st, int pass)
 {
     __shared__ uint32_t bins[kBins];
-    bins[threadIdx.x] = 0u;
+    uint32_t prefix = 0, remaining = 0, ties = 0;
+    if (pass > 0) topk_resolve(st, pass - 1, &prefix, &remaining, &ties);
+    const int nb = 1 << kDigitBits[pass];
+    for (int i = threadIdx.x; i < nb; i += 256) bins[i] = 0u;
     __syncthreads();
-    const int shift = 24 - 8 * pass;
-    const uint32_t prefix = st->prefix;
+    const int shift = kDigitShift[pass], hi = shift + kDigitBits[pass];
+    const uint32_t mask = (uint32_t)nb - 1u;
+    const int64_t quads = numel >> 2;
+    const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
     int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < numel; i += stride) {
+    if (vec) {
+        for (int64_t q = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; q < quads; q += stride) {
+            float4 v = reinterpret_cast<const float4*>(x)[q];
+            uint32_t key[4] = {mag_key(v.x), mag_key(v.y), mag_key(v.z), mag_key(v.w)};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (pass == 0 || (key[e] >> hi) == prefix) atomicAdd(&bins[(key[e] >> shift) & mask], 1u);
+        }
+    }
+    for (int64_t i = (vec ? quads * 4 : 0) + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < numel; i += stride) {
         uint32_t key = mag_key(x[i]);
-        bool match = pass == 0 || (key >> (shift + 8)) == prefix;
-        if (match) atomicAdd(&bins[(key >> shift) & 0xffu], 1u);
+        if (pass == 0 || (key >> hi) == prefix) atomicAdd(&bins[(key >> shift) & mask], 1u);
     }
     __syncthreads();
-    uint32_t c = bins[threadIdx.x];
-    if (c) atomicAdd(&st->hist[pass][threadIdx.x], c);
-}
-
-// one workgroup: pick the digit that holds the k-th largest key among those matching the prefix
-__global__ void __launch_bounds__(256)
-topk_select_kernel(TopkState* st, int pass)
-{
-    __shared__ uint32_t cnt[kBins];
-    cnt[threadIdx.x] = st->hist[pass][threadIdx.x];
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t remaining = st->remaining;
-        uint32_t above = 0;
-        int d = kBins - 1;
-        for (; d > 0; --d) {
-            if (above + cnt[d] >= remaining) break;
-            above += cnt[d];
-        }
-        st->prefix = (st->prefix << 8) | (uint32_t)d;
-        st->remaining = remaining - above;
+    for (int i = threadIdx.x; i < nb; i += 256) {
+        uint32_t c = bins[i];
+        if (c) atomicAdd(&st->hist[pass][i], c);
     }
 }
 
 // per-chunk count of keys equal to the threshold
 __global__ void __launch_bounds__(256)
-topk_count_ties_kernel(const float* __restrict__ x, int64_t numel, const TopkState* st, uint32_t* chunk_ties,
+topk_count_ties_kernel(const float* __restrict__ x, int64_t numel, TopkState* st, uint32_t* chunk_ties,
                        int64_t chunks)
 {
     __shared__ uint32_t total;
-    const uint32_t thr = st->prefix;
+    uint32_t thr, keep_ties, ties;
+    topk_resolve(st, kPasses - 1, &thr, &keep_ties, &ties);
+    if (ties == keep_ties) return;          // every key equal to the threshold is kept: no order needed
     for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
         if (threadIdx.x == 0) total = 0u;
         __syncthreads();
@@ -96,9 +148,10 @@ topk_count_ties_kernel(const float* __restrict__ x, int64_t numel, const TopkSta
 
 // one workgroup: exclusive prefix sum of the per-chunk tie counts, in place
 __global__ void __launch_bounds__(1024)
-topk_scan_kernel(uint32_t* chunk_ties, int64_t chunks)
+topk_scan_kernel(const TopkState* st, uint32_t* chunk_ties, int64_t chunks)
 {
     __shared__ uint32_t part[1024];
+    if (st->ties[kPasses - 1] == st->remaining[kPasses - 1]) return;
     int64_t per = (chunks + 1023) / 1024;
     int64_t lo = (int64_t)threadIdx.x * per;
     int64_t hi = lo + per < chunks ? lo + per : chunks;
@@ -129,9 +182,26 @@ topk_filter_kernel(float* __restrict__ x, int64_t numel, const TopkState* st, co
                    int64_t chunks)
 {
     __shared__ uint32_t wave_ties[4];
-    const uint32_t thr = st->prefix;
-    const uint32_t keep_ties = st->remaining;
+    const uint32_t thr = st->prefix[kPasses - 1];
+    const uint32_t keep_ties = st->remaining[kPasses - 1];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (st->ties[kPasses - 1] == keep_ties) {
+        // no ties to break: keep every key at or above the threshold, 16-byte accesses
+        const int64_t quads = numel >> 2;
+        const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+        const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+        if (vec) {
+            for (int64_t q = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; q < quads; q += stride) {
+                float4 v = reinterpret_cast<float4*>(x)[q];
+                bool k0 = mag_key(v.x) >= thr, k1 = mag_key(v.y) >= thr, k2 = mag_key(v.z) >= thr, k3 = mag_key(v.w) >= thr;
+                if (!(k0 && k1 && k2 && k3))
+                    reinterpret_cast<float4*>(x)[q] = make_float4(k0 ? v.x : 0.f, k1 ? v.y : 0.f, k2 ? v.z : 0.f, k3 ? v.w : 0.f);
+            }
+        }
+        for (int64_t i = (vec ? quads * 4 : 0) + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < numel; i += stride)
+            if (mag_key(x[i]) < thr) x[i] = 0.f;
+        return;
+    }
     for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
         int64_t base = c * kFilterChunk + (int64_t)threadIdx.x * 4;
         float v[4];
@@ -189,18 +259,16 @@ int conef_topk_sparsify_f32(float* x, int64_t numel, int64_t k, void* workspace,
     hipStream_t s = (hipStream_t)stream;
     TopkState* st = (TopkState*)workspace;
     uint32_t* chunk_ties = (uint32_t*)((char*)workspace + sizeof(TopkState));
-    int64_t g = (numel + 255) / 256 / 8;
+    int64_t g = (numel + 255) / 256 / 16;        // four 16-byte loads per thread and pass, at least
     if (g < 1) g = 1;
-    if (g > 2048) g = 2048;
+    if (g > 1024) g = 1024;
     hipLaunchKernelGGL(topk_init_kernel, dim3(1), dim3(256), 0, s, st, (uint32_t)k);
-    for (int pass = 0; pass < 4; ++pass) {
+    for (int pass = 0; pass < kPasses; ++pass)
         hipLaunchKernelGGL(topk_hist_kernel, dim3((unsigned)g), dim3(256), 0, s, x, numel, st, pass);
-        hipLaunchKernelGGL(topk_select_kernel, dim3(1), dim3(256), 0, s, st, pass);
-    }
     int64_t chunks = topk_chunks(numel);
     int64_t cg = chunks < 4096 ? chunks : 4096;
     hipLaunchKernelGGL(topk_count_ties_kernel, dim3((unsigned)cg), dim3(256), 0, s, x, numel, st, chunk_ties, chunks);
-    hipLaunchKernelGGL(topk_scan_kernel, dim3(1), dim3(1024), 0, s, chunk_ties, chunks);
+    hipLaunchKernelGGL(topk_scan_kernel, dim3(1), dim3(1024), 0, s, st, chunk_ties, chunks);
     hipLaunchKernelGGL(topk_filter_kernel, dim3((unsigned)cg), dim3(256), 0, s, x, numel, st, chunk_ties, chunks);
     return (int)hipGetLastError();
 }
