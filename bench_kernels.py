@@ -222,7 +222,8 @@ def main():
                                                                              s[4].data_ptr(), n, m, r, w, 0.9, A, B,
                                                                              stream), "pqt conef"), flops=fl)
 
-    for rows, r in [(5760, 4), (640, 4), (4096, 8), (1024, 8), (30522, 8), (4096, 32), (576, 2)]:
+    for rows, r in [(5760, 4), (640, 4), (4096, 8), (1024, 8), (30522, 8), (4096, 32), (576, 2), (1024, 32), (512, 32),
+                    (30522, 32), (1024, 16), (4096, 16), (2048, 32), (2048, 16), (256, 32), (64, 32)]:
         ws = torch.empty(lib.conef_psgd_workspace_bytes(rows, 1, r), dtype=torch.uint8, device=dev)
         timeit("gram_schmidt_f32 [%d,%d]" % (rows, r), 8 * rows * r,
                lambda rows=rows, r=r: [(torch.randn(rows, r, device=dev),) for _ in range(8)],

@@ -17,6 +17,7 @@
 #include "conef_sketch_core.h"
 #include "conef_plan.h"
 #include "conef_psgd_mfma.h"
+#include "conef_gs_lanes.h"
 #include "conef_hip.h"      // ConefPsgdItem, and a check of this file's definitions against the public header
 
 extern "C" int conef_cs_query_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
@@ -1190,6 +1191,8 @@ inline int64_t gs_sums_floats(int64_t rows, int r)
 {
     int64_t steps = 2 * (int64_t)kGsMaxWorkgroups * rank_bound(r);
     int64_t grid = (int64_t)(sizeof(GsGridWs) + 3) / 4;
+    int64_t lanes = (int64_t)(sizeof(GslWs) + 3) / 4;
+    if (lanes > grid) grid = lanes;
     return steps > grid ? steps : grid;
 }
 
@@ -1231,6 +1234,92 @@ inline int gs_launch_reg_batch(const GsBatch& batch, int count, int r, int slots
 #undef CONEF_GSR
 #undef CONEF_GSR_GO
     return (int)hipGetLastError();
+}
+
+// Kernels of conef_gs_lanes.h: which one a matrix takes.  kind 0: none (rank not 8, 16 or 32, the
+// matrix narrower than its rank bound, or larger than 128 workgroups hold); kind 1: one workgroup,
+// a wave per two columns (rank 32 up to 2048 rows) or per column (rank 16 up to 1024 rows), rpt
+// rows a lane; kind 2: wgs workgroups of the column-per-lane kernel, rpt rows a thread, launched
+// cooperatively.  Other matrices that fit one workgroup's registers (32768 elements) stay with
+// the row-per-thread kernel, which is faster there.
+struct GslChoice {
+    int kind, rpt, wgs;
+};
+
+inline GslChoice gsl_choose(int64_t rows, int r)
+{
+    GslChoice ch = {0, 0, 0};
+    if (r != rank_bound(r) || r < 8) return ch;
+    if ((r == 32 && rows <= 2048) || (r == 16 && rows <= 1024)) {
+        ch.kind = 1;
+        ch.rpt = rows <= 256 ? 4 : rows <= 512 ? 8 : rows <= 1024 ? 16 : 32;
+        ch.wgs = 1;
+        return ch;
+    }
+    const int64_t elements = rows * r;
+    if (elements <= (int64_t)kGsRegThreads * kGsRegFloats) return ch;      // the row-per-thread kernel, one workgroup
+    static const int kRpt[4] = {4, 8, 16, 64};
+    for (int k = 0; k < (r == 8 ? 3 : 4); ++k) {
+        const int64_t per = (int64_t)kGslThreads * kRpt[k];
+        const int64_t wgs = (elements + per - 1) / per;
+        if (wgs <= kGslMaxWgs) {
+            ch.kind = 2;
+            ch.rpt = kRpt[k];
+            ch.wgs = (int)wgs;
+            return ch;
+        }
+    }
+    return ch;
+}
+
+template <int RP, int RPT, int CW>
+inline hipError_t gsw_go(const GswBatch& batch, int count, float eps, hipStream_t s)
+{
+    constexpr int kLds = gsw_lds_floats<RP, RPT>() * 4;
+    static const hipError_t attr =
+        kLds > 48 * 1024 ? hipFuncSetAttribute((const void*)gsw_kernel<RP, RPT, CW>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLds)
+                         : hipSuccess;
+    if (attr != hipSuccess) return attr;
+    hipLaunchKernelGGL((gsw_kernel<RP, RPT, CW>), dim3((unsigned)count), dim3(64 * RP / CW), kLds, s, batch, eps);
+    return hipGetLastError();
+}
+
+// kind 1: `count` matrices of rank r, all of class rpt, one workgroup each
+inline int gsw_launch(const GswBatch& batch, int count, int r, int rpt, float eps, hipStream_t s)
+{
+    hipError_t e = hipErrorInvalidValue;
+    if (r == 32) {
+        e = rpt == 4 ? gsw_go<32, 4, 2>(batch, count, eps, s) : rpt == 8 ? gsw_go<32, 8, 2>(batch, count, eps, s)
+          : rpt == 16 ? gsw_go<32, 16, 2>(batch, count, eps, s) : gsw_go<32, 32, 2>(batch, count, eps, s);
+    } else if (r == 16) {
+        e = rpt == 4 ? gsw_go<16, 4, 1>(batch, count, eps, s) : rpt == 8 ? gsw_go<16, 8, 1>(batch, count, eps, s)
+                                                                          : gsw_go<16, 16, 1>(batch, count, eps, s);
+    }
+    if (e != hipSuccess) (void)hipGetLastError();
+    return (int)e;
+}
+
+// kind 2: one batch of matrices of rank r and class rpt over wgs workgroups in all.  A cooperative
+// launch the runtime refuses comes back as an error for the caller to take the other kernels.
+inline int gsl_launch(const GslBatch& batch, int count, int r, int rpt, int wgs, float eps, void* workspace, hipStream_t s)
+{
+    GslWs* ws = (GslWs*)workspace;
+    const void* fn = nullptr;
+#define CONEF_GSL(RP)                                                                                     \
+    fn = rpt == 4 ? (const void*)gsl_kernel<RP, 4> : rpt == 8 ? (const void*)gsl_kernel<RP, 8>            \
+       : rpt == 16 ? (const void*)gsl_kernel<RP, 16> : (const void*)gsl_kernel<RP, 64>
+    if (r == 32) CONEF_GSL(32);
+    else if (r == 16) CONEF_GSL(16);
+    else if (r == 8 && rpt <= 16) fn = rpt == 4 ? (const void*)gsl_kernel<8, 4> : rpt == 8 ? (const void*)gsl_kernel<8, 8>
+                                                                                            : (const void*)gsl_kernel<8, 16>;
+#undef CONEF_GSL
+    if (!fn) return CONEF_ERR_INVALID;
+    hipLaunchKernelGGL(gsl_reset_kernel, dim3(8), dim3(1024), 0, s, ws, wgs);
+    void* args[] = {(void*)&batch, (void*)&count, (void*)&eps, (void*)&ws};
+    hipError_t e = hipLaunchCooperativeKernel(fn, dim3((unsigned)wgs), dim3(kGslThreads), args, 0, s);
+    if (e != hipSuccess) (void)hipGetLastError();
+    return (int)e;
 }
 
 inline bool psgd_args_ok(int64_t n, int64_t m, int32_t r)
@@ -1464,6 +1553,23 @@ int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* w
     if (rows < 1 || rows > 0x7fffffffLL || r < 1 || r > kMaxRank || !a) return CONEF_ERR_INVALID;
     hipStream_t s = (hipStream_t)stream;
     const int rp = rank_bound(r);
+    {
+        const GslChoice ch = gsl_choose(rows, r);
+        if (ch.kind == 1) {
+            GswBatch one;
+            one.a[0] = a;
+            one.rows[0] = (int)rows;
+            if (gsw_launch(one, 1, r, ch.rpt, eps, s) == CONEF_OK) return CONEF_OK;
+        } else if (ch.kind == 2 && workspace && workspace_bytes >= (int64_t)sizeof(GslWs) &&
+                   (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0) {
+            GslBatch one;
+            one.a[0] = a;
+            one.elements[0] = rows * r;
+            one.first[0] = 0;
+            one.first[1] = ch.wgs;
+            if (gsl_launch(one, 1, r, ch.rpt, ch.wgs, eps, workspace, s) == CONEF_OK) return CONEF_OK;
+        }
+    }
     if (gs_reg_class(a, rows, r) >= 0) {
         GsBatch one;
         one.a[0] = a;
@@ -1546,6 +1652,41 @@ int conef_gram_schmidt_batch_f32(float* const* mats, const int64_t* rows, const 
     std::vector<char> done((size_t)count, 0);
     for (int k = 0; k < count; ++k) {
         if (rows[k] < 1 || rows[k] > 0x7fffffffLL || ranks[k] < 1 || ranks[k] > kMaxRank || !mats[k]) return CONEF_ERR_INVALID;
+    }
+    // kernels of conef_gs_lanes.h: matrices of one rank and class share launches (up to 48 matrices
+    // of the one-workgroup kernel; up to 24 matrices and 128 workgroups of the other)
+    const bool ws_ok = workspace && workspace_bytes >= (int64_t)sizeof(GslWs) && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0;
+    for (int k = 0; k < count; ++k) {
+        if (done[(size_t)k]) continue;
+        const GslChoice ck = gsl_choose(rows[k], ranks[k]);
+        if (ck.kind == 0 || (ck.kind == 2 && !ws_ok)) continue;
+        GslBatch grid;
+        GswBatch single;
+        std::vector<int> members;
+        int nb = 0, wgs = 0;
+        const int cap = ck.kind == 1 ? kGswBatchMax : kGslMaxItems;
+        for (int j = k; j < count && nb < cap; ++j) {
+            if (done[(size_t)j] || ranks[j] != ranks[k]) continue;
+            const GslChoice cj = gsl_choose(rows[j], ranks[j]);
+            if (cj.kind != ck.kind || cj.rpt != ck.rpt) continue;
+            if (ck.kind == 2 && wgs + cj.wgs > kGslMaxWgs) continue;
+            if (ck.kind == 1) {
+                single.a[nb] = mats[j];
+                single.rows[nb] = (int)rows[j];
+            } else {
+                grid.a[nb] = mats[j];
+                grid.elements[nb] = rows[j] * ranks[j];
+                grid.first[nb] = wgs;
+            }
+            wgs += cj.wgs;
+            ++nb;
+            members.push_back(j);
+        }
+        if (ck.kind == 2) grid.first[nb] = wgs;
+        const int rc = ck.kind == 1 ? gsw_launch(single, nb, ranks[k], ck.rpt, eps, s)
+                                    : gsl_launch(grid, nb, ranks[k], ck.rpt, wgs, eps, workspace, s);
+        if (rc != CONEF_OK) break;      // the other kernels below take what is left
+        for (int j : members) done[(size_t)j] = 1;
     }
     for (int k = 0; k < count; ++k) {
         if (done[(size_t)k]) continue;

@@ -144,7 +144,11 @@ def test_gram_schmidt_parity(oracle):
                          (300, 3, 1e-8), (33278, 4, 0.0), (2000, 13, 0.0), (30522, 8, 0.0), (70001, 3, 1e-8),
                          (64, 32, 0.0), (1, 1, 0.0), (1024, 32, 0.0), (1000, 32, 1e-8), (2048, 16, 0.0), (2047, 9, 0.0),
                          (8192, 4, 0.0), (8200, 4, 0.0), (32768, 1, 0.0), (16384, 2, 0.0), (4500, 8, 0.0), (255, 5, 0.0),
-                         (257, 7, 0.0)]:
+                         (257, 7, 0.0),
+                         # one column per lane at ranks 8, 16, 32: one workgroup up to 65536 elements,
+                         # several (cooperative launch) above, the multi-launch kernel past 128 workgroups
+                         (512, 32, 0.0), (2048, 32, 0.0), (4096, 16, 1e-8), (30522, 32, 0.0), (30522, 16, 0.0),
+                         (70000, 8, 0.0), (100, 16, 0.0), (270000, 32, 0.0), (65, 32, 0.0)]:
         g = torch.Generator().manual_seed(rows + r)
         a = torch.randn(rows, r, generator=g)
         want = a.numpy().copy()
@@ -165,7 +169,8 @@ def test_gram_schmidt_batch_parity(oracle):
     from conef_amd import _lib
     lib = _lib.load()
     shapes = [(640, 4), (5760, 4), (27, 4), (1440, 4), (30522, 4), (1024, 8), (4096, 8), (64, 2), (4096, 32), (33, 4),
-              (300, 3), (1, 1)] + [(100 + 7 * k, 4) for k in range(60)]
+              (300, 3), (1, 1), (1024, 32), (1024, 32), (512, 32), (4096, 32), (4096, 32), (30522, 32), (2048, 16), (1000, 32),
+              (30522, 8), (40000, 8)] + [(100 + 7 * k, 4) for k in range(60)]
     gen = torch.Generator().manual_seed(9)
     host = [torch.randn(rows, r, generator=gen) for rows, r in shapes]
     arena = torch.zeros(sum(h.numel() for h in host) + 8, device="cuda")
