@@ -100,7 +100,7 @@ class _RoundPlan:
     arenas.  Built on the first step of a bucket and reused while the bucket keeps its buffer
     and layout, so that a step costs a handful of foreign calls however many tensors it has."""
     __slots__ = ("key", "shapes", "work", "passthrough", "before", "after", "total_ps", "total_qs", "arena_key", "ps",
-                 "qs", "gs_p", "gs_q", "items", "count", "sketches", "fused_sketch", "residual_offsets")
+                 "qs", "gs_p", "gs_q", "items", "count", "sketches", "fused_sketch", "batched_update", "residual_offsets")
 
 
 def _gs_table(matrices):
@@ -139,6 +139,7 @@ def _build_round(state, grads, shapes, key, error_mode):
     plan.arena_key = None
     plan.sketches = []
     plan.fused_sketch = False
+    plan.batched_update = False
     plan.residual_offsets = []
     off = 0
     for _, n, m, _ in plan.work:
@@ -239,8 +240,8 @@ def run_round(state, bucket, error_mode):
                 it.w = cs.range
                 it.plan_host, it.plan_dev = (sk_plan.host_ptr, sk_plan.device.data_ptr()) if sk_plan is not None else (None, None)
                 plan.sketches.append((cs, sk_plan))
-            plan.fused_sketch = (state.matrix_approximation_rank <= 8 and
-                                 all(p is not None and p.in_place for _, p in plan.sketches))
+            plan.batched_update = all(p is not None and p.in_place for _, p in plan.sketches)
+            plan.fused_sketch = state.matrix_approximation_rank <= 8 and plan.batched_update
         for cnt, (cs, _) in enumerate(plan.sketches):
             items[cnt].cs = cs.cs.data_ptr()
     elif error_mode == "conef_v2":
@@ -293,9 +294,9 @@ def run_round(state, bucket, error_mode):
     elif error_mode == "conef" and plan.fused_sketch:
         mode3 = 2
     elif error_mode in ("conef", "conef_v2"):
-        # The residual goes out dense and every sketch is updated in a launch of its own: ranks
-        # above 8 (the low-rank product belongs on the matrix cores), sketches whose plan is not a
-        # row list, and the re-viewed sketches of C2CS_hook_v2.
+        # The residual goes out dense and the sketches are updated from it afterwards: ranks above
+        # 8 (the low-rank product belongs on the matrix cores), sketches whose plan is not a row
+        # list, and the re-viewed sketches of C2CS_hook_v2.
         mode3 = 1
         residual = _scratch_f32(device, stream, max(plan.residual_offsets[-1], 1))
         for cnt in range(count):
@@ -309,6 +310,10 @@ def run_round(state, bucket, error_mode):
         topk_ws = None
         for cnt in range(count):
             topk_ws = topk_sparsify(errs[cnt], state.topk_ratio, topk_ws)
+    elif residual is not None and error_mode == "conef" and plan.batched_update:
+        # every sketch of the bucket from its matrix's residual, in one launch
+        rc = lib.conef_psgd_sketch_update_batch_f32(items, count, float(state.beta), HASH_A, HASH_B, stream)
+        _lib.check(rc, "conef_psgd_sketch_update_batch_f32")
     elif residual is not None:
         for cnt, (matrix, n, m, rank) in enumerate(work):
             res = residual[plan.residual_offsets[cnt]: plan.residual_offsets[cnt + 1]]

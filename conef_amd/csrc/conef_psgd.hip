@@ -396,6 +396,139 @@ psgd_sum_partials_batch_kernel(PsgdBatch<SumItem> b)
     psgd_sum_partials_body(it.partial, it.out, it.count, it.slabs, local);
 }
 
+// ------------------------------------------- matrix-core products, batched ----
+// The MFMA kernels of conef_psgd_mfma.h over the matrices of a bucket: workgroup `local` of an
+// item is workgroup (local % its first grid dimension, local / it) of the single-matrix launch.
+struct MfmaMqItem {
+    float* x;
+    const float* err;
+    const float* q;
+    float* out;
+    int64_t n;
+    int m, r, cols_per_split, row_tiles;
+    ConefMod mod;       // of width 1: the batched kernel never unsketches
+};
+
+template <int MODE>
+__global__ void __launch_bounds__(kMfmaThreads)
+psgd_mfma_mq_batch_kernel(PsgdBatch<MfmaMqItem> b)
+{
+    static_assert(MODE == 0 || MODE == 1, "the sketch query of a batch runs as a launch of its own");
+    int local;
+    const MfmaMqItem& it = b.item[psgd_batch_locate(b, &local)];
+    const ConefSeeds hs = {0, 0, 0, 0};
+    psgd_mfma_mq_body<MODE>(it.x, it.err, nullptr, nullptr, it.q, it.out, it.n, it.m, it.r, it.cols_per_split, it.mod, 0.f,
+                            hs, local % it.row_tiles, local / it.row_tiles);
+}
+
+struct MfmaMtpItem {
+    const float* x;
+    const float* p;
+    float* out;
+    int64_t n;
+    int m, r, rows_per_slab, col_tiles;
+};
+
+template <int V>
+__global__ void __launch_bounds__(kMfmaThreads)
+psgd_mfma_mtp_batch_kernel(PsgdBatch<MfmaMtpItem> b)
+{
+    int local;
+    const MfmaMtpItem& it = b.item[psgd_batch_locate(b, &local)];
+    psgd_mfma_mtp_body<V>(it.x, it.p, it.out, it.n, it.m, it.r, it.rows_per_slab, local % it.col_tiles, local / it.col_tiles);
+}
+
+struct MfmaPqtItem {
+    float* x;
+    float* err;
+    const float* p;
+    const float* q;
+    int64_t n;
+    int m, rows_per_slab, col_wgs;
+};
+
+template <int R, int MODE>
+__global__ void __launch_bounds__(kMfmaThreads)
+psgd_mfma_pqt_batch_kernel(PsgdBatch<MfmaPqtItem> b)
+{
+    int local;
+    const MfmaPqtItem& it = b.item[psgd_batch_locate(b, &local)];
+    psgd_mfma_pqt_body<R, MODE>(it.x, it.err, it.p, it.q, it.n, it.m, it.rows_per_slab, local % it.col_wgs,
+                                local / it.col_wgs);
+}
+
+// X += alpha * unsketch(cs) over the matrices of a bucket (DenseCS.query, CountSketch.py:51-66):
+// a thread owns a column quad of a group of rows, its (bucket, sign) words from the plan's table
+// or hashed, once for the group.  VEC: m % 4 == 0 and 16-byte aligned x (and table).
+struct QueryItem {
+    float* x;
+    const float* cs;
+    const uint32_t* pktab;
+    int64_t n;
+    int m, rows_per_block, col_blocks;
+    ConefMod mod;
+};
+
+template <bool VEC>
+__global__ void __launch_bounds__(256)
+psgd_cs_query_batch_kernel(PsgdBatch<QueryItem> b, float alpha, ConefSeeds hs)
+{
+    int local;
+    const QueryItem& it = b.item[psgd_batch_locate(b, &local)];
+    const int bx = local % it.col_blocks, by = local / it.col_blocks;
+    const int c0 = (bx * 256 + (int)threadIdx.x) * 4;
+    if (c0 >= it.m) return;
+    uint32_t pk[4];
+    if (VEC && it.pktab) {
+        const uint4 t = *reinterpret_cast<const uint4*>(it.pktab + c0);
+        pk[0] = t.x; pk[1] = t.y; pk[2] = t.z; pk[3] = t.w;
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            pk[k] = c0 + k < it.m ? (it.pktab ? it.pktab[c0 + k] : conef_bucket_sign(c0 + k, it.mod, hs.a, hs.b, hs.sa, hs.sb))
+                                  : 0u;
+    }
+    const int64_t r0 = (int64_t)by * it.rows_per_block;
+    const int64_t r1 = r0 + it.rows_per_block < it.n ? r0 + it.rows_per_block : it.n;
+    const int w = (int)it.mod.w;
+    for (int64_t r = r0; r < r1; ++r) {
+        const float* row = it.cs + r * w;
+        float* xr = it.x + r * it.m + c0;
+        if (VEC) {
+            float4 v = *reinterpret_cast<const float4*>(xr);
+            v.x = __fadd_rn(v.x, conef_query_term(row[pk[0] & 0x7fffffffu], pk[0], alpha));
+            v.y = __fadd_rn(v.y, conef_query_term(row[pk[1] & 0x7fffffffu], pk[1], alpha));
+            v.z = __fadd_rn(v.z, conef_query_term(row[pk[2] & 0x7fffffffu], pk[2], alpha));
+            v.w = __fadd_rn(v.w, conef_query_term(row[pk[3] & 0x7fffffffu], pk[3], alpha));
+            *reinterpret_cast<float4*>(xr) = v;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (c0 + k < it.m) xr[k] = __fadd_rn(xr[k], conef_query_term(row[pk[k] & 0x7fffffffu], pk[k], alpha));
+        }
+    }
+}
+
+// DenseCS.update(vec, beta) (CountSketch.py:27-48) of the sketches of a bucket's matrices on
+// row-list plans, vec = the item's dense residual.
+struct RowlistVecItem {
+    ConefListVec front;
+    ConefRowlistView plan;
+    const float* cs_in;
+    float* cs_out;
+    int64_t n;
+    int d, w, rb;
+};
+
+__global__ void __launch_bounds__(kConefRowlistThreads)
+psgd_rowlist_vec_batch_kernel(PsgdBatch<RowlistVecItem> b, double one_minus_beta)
+{
+    int local;
+    const RowlistVecItem& it = b.item[psgd_batch_locate(b, &local)];
+    conef_rowlist_body<float, ConefListVec>(it.front, it.plan, it.cs_in, it.cs_out, it.n, it.d, it.w, it.rb, one_minus_beta,
+                                            local);
+}
+
 // ------------------------------------------------------------ M = P Q^T ----
 // MODE 0: write M.  MODE 1: also write the dense residual E = X - M (X = what M held on entry).
 // A thread owns a column quad (its 4 x r slice of Q stays in registers), the workgroup walks a slab
@@ -1750,6 +1883,65 @@ inline const uint32_t* item_pktab(const ConefPsgdItem& it)
     return (hp && it.plan_dev) ? (const uint32_t*)((const char*)it.plan_dev + hp->off_pk) : nullptr;
 }
 
+// Matrix-core items of a batch run side by side, so each needs its own region for the partial
+// tiles of its column splits (P = X Q) and row slabs (Q = X^T P); the two are never alive at once.
+// offs[k]: where item k's region starts, in floats, -1 for ranks below 16.
+inline int64_t mfma_batch_layout(const ConefPsgdItem* items, int count, std::vector<int64_t>* offs)
+{
+    int64_t off = 0;
+    for (int k = 0; k < count; ++k) {
+        int64_t at = -1;
+        if (rank_bound(items[k].r) >= 16) {
+            const int64_t n = items[k].n, m = items[k].m;
+            const int r = items[k].r;
+            MfmaMqShape q = mfma_mq_shape(n, m);
+            int64_t need = q.splits > 1 ? (int64_t)q.splits * n * r : 0;
+            for (int v = 4; v >= 1; v >>= 1) {
+                MfmaMtpShape t = mfma_mtp_shape(n, m, r, v);
+                int64_t b = t.slabs > 1 ? (int64_t)t.slabs * m * r : 0;
+                if (b > need) need = b;
+            }
+            at = off;
+            off += (need + 63) / 64 * 64;
+        }
+        if (offs) offs->push_back(at);
+    }
+    return off;
+}
+
+// bytes at the front of a batch workspace that matrix-core items launched one by one share
+inline int64_t batch_single_bytes(const ConefPsgdItem* items, int count)
+{
+    int64_t single = 0;
+    for (int k = 0; k < count; ++k)
+        if (rank_bound(items[k].r) >= 16) {
+            int64_t b = conef_psgd_workspace_bytes(items[k].n, items[k].m, items[k].r);
+            if (b > single) single = b;
+        }
+    return single;
+}
+
+struct MtpPlan;
+inline int64_t mtp_batch_layout(const ConefPsgdItem* items, int count, std::vector<MtpPlan>* plans);
+
+// where the matrix-core partial regions start inside a batch workspace; nullptr when it is too small
+inline float* mfma_partial_base(const ConefPsgdItem* items, int count, void* workspace, int64_t workspace_bytes,
+                                std::vector<int64_t>* offs)
+{
+    const int64_t floats = mfma_batch_layout(items, count, offs);
+    const int64_t front = batch_single_bytes(items, count) + conef_align256(4 * mtp_batch_layout(items, count, nullptr));
+    if (floats > 0 && (!workspace || workspace_bytes < front + 4 * floats)) return nullptr;
+    return (float*)((char*)workspace + front);
+}
+
+inline int rows_per_query_block(int64_t n, int64_t col_blocks)
+{
+    int64_t rpb = (n * col_blocks + 1023) / 1024;       // about a thousand workgroups a matrix, eight rows at least
+    if (rpb < 8) rpb = 8;
+    if (rpb > n) rpb = n;
+    return (int)(rpb < 1 ? 1 : rpb);
+}
+
 // rows per workgroup of the streaming P = X Q kernel inside a batch: four amortise the Q traffic
 // once the batch as a whole has workgroups to spare
 inline int mq_rows_per_wg(int64_t total_rows) { return total_rows / 4 >= 256 ? 4 : 1; }
@@ -1773,6 +1965,68 @@ int mq_batch(const ConefPsgdItem* items, int count, float alpha, int32_t a, int3
         auto alone = [&](const ConefPsgdItem& it) {
             return rank_bound(it.r) >= 16 || (MODE == 2 && (size_t)4 * it.w * 4 + 4 * 4 * 8 * 4 > 64 * 1024);
         };
+        // ranks on the matrix cores whose shapes allow the 16-byte paths share launches: the sketch
+        // query first when there is one, then the plain (or error-adding) product, then the sums
+        // of the column splits
+        auto mfma_ok = [&](const ConefPsgdItem& it) {
+            return rank_bound(it.r) >= 16 && it.m % 4 == 0 && aligned16(it.x) && (MODE != 1 || aligned16(it.err)) &&
+                   (MODE != 2 || !item_pktab(it) || aligned16(item_pktab(it)));
+        };
+        if (mfma_ok(lead)) {
+            std::vector<int64_t> offs;
+            float* partials = mfma_partial_base(items, count, workspace, workspace_bytes, &offs);
+            std::vector<QueryItem> queries;
+            std::vector<MfmaMqItem> table;
+            std::vector<SumItem> sums;
+            std::vector<int> qblocks, blocks, sum_blocks;
+            for (int j = k; j < count; ++j) {
+                if (done[(size_t)j] || !mfma_ok(items[j])) continue;
+                const ConefPsgdItem& it = items[j];
+                MfmaMqShape g = mfma_mq_shape(it.n, it.m);
+                if (g.splits > 1 && !partials) {
+                    g.splits = 1;
+                    g.cols_per_split = (int)((it.m + 127) / 128 * 128);
+                }
+                float* out = g.splits > 1 ? partials + offs[(size_t)j] : it.p;
+                if (MODE == 2) {
+                    const int64_t col_blocks = (it.m + 1023) / 1024;
+                    const int rpb = rows_per_query_block(it.n, col_blocks);
+                    QueryItem qi = {it.x, it.cs, item_pktab(it), it.n, (int)it.m, rpb, (int)col_blocks, conef_make_mod(it.w)};
+                    queries.push_back(qi);
+                    qblocks.push_back((int)(col_blocks * ((it.n + rpb - 1) / rpb)));
+                }
+                MfmaMqItem t = {it.x, MODE == 1 ? it.err : nullptr, it.q, out, it.n, (int)it.m, it.r, g.cols_per_split,
+                                g.row_tiles, conef_make_mod(1)};
+                table.push_back(t);
+                blocks.push_back(g.row_tiles * g.splits);
+                if (g.splits > 1) {
+                    const int64_t cnt = it.n * it.r;
+                    SumItem si = {out, it.p, cnt, g.splits};
+                    sums.push_back(si);
+                    sum_blocks.push_back((int)((cnt + 255) / 256));
+                }
+                done[(size_t)j] = 1;
+            }
+            int rc = CONEF_OK;
+            if (MODE == 2)
+                rc = run_batches(queries, qblocks, [&](const PsgdBatch<QueryItem>& bt, int grid) {
+                    hipLaunchKernelGGL(psgd_cs_query_batch_kernel<true>, dim3((unsigned)grid), dim3(256), 0, s, bt, alpha, hs);
+                });
+            if (rc != CONEF_OK) return rc;
+            const size_t lds = (size_t)kMfmaWaves * 16 * 64 * 4;
+            rc = run_batches(table, blocks, [&](const PsgdBatch<MfmaMqItem>& bt, int grid) {
+                hipLaunchKernelGGL((psgd_mfma_mq_batch_kernel<(MODE == 1 ? 1 : 0)>), dim3((unsigned)grid), dim3(kMfmaThreads),
+                                   lds, s, bt);
+            });
+            if (rc != CONEF_OK) return rc;
+            if (!sums.empty()) {
+                rc = run_batches(sums, sum_blocks, [&](const PsgdBatch<SumItem>& bt, int grid) {
+                    hipLaunchKernelGGL(psgd_sum_partials_batch_kernel, dim3((unsigned)grid), dim3(256), 0, s, bt);
+                });
+                if (rc != CONEF_OK) return rc;
+            }
+            continue;
+        }
         if (alone(lead)) {
             int rc = launch_mq<MODE>(lead.x, lead.err, lead.cs, item_pktab(lead), lead.q, lead.p, lead.n, lead.m, lead.r,
                                      MODE == 2 ? lead.w : 1, alpha, hs, workspace, workspace_bytes, s);
@@ -1851,17 +2105,46 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
 {
     std::vector<MtpPlan> plans;
     const int64_t floats = mtp_batch_layout(items, count, &plans);
-    int64_t single = 0;       // the matrix-core items run one by one and share the front of the workspace
-    for (int k = 0; k < count; ++k)
-        if (rank_bound(items[k].r) >= 16) {
-            int64_t b = conef_psgd_workspace_bytes(items[k].n, items[k].m, items[k].r);
-            if (b > single) single = b;
-        }
+    // matrix-core items that have to run one by one share the front of the workspace
+    const int64_t single = batch_single_bytes(items, count);
     if ((floats > 0 || single > 0) && (!workspace || workspace_bytes < floats * 4 + single)) return CONEF_ERR_INVALID;
     float* partial_base = (float*)((char*)workspace + single);
+    std::vector<int64_t> mfma_offs;
+    float* mfma_partials = mfma_partial_base(items, count, workspace, workspace_bytes, &mfma_offs);
     std::vector<char> done((size_t)count, 0);
     std::vector<SumItem> sums;
     std::vector<int> sum_blocks;
+    // matrix-core items: one launch per vector width (4, 2 or 1 floats a lane, by the alignment of x)
+    for (int v = 4; v >= 1 && mfma_partials; v >>= 1) {
+        std::vector<MfmaMtpItem> table;
+        std::vector<int> blocks;
+        for (int k = 0; k < count; ++k) {
+            const ConefPsgdItem& it = items[k];
+            if (done[(size_t)k] || rank_bound(it.r) < 16) continue;
+            const uintptr_t xa = reinterpret_cast<uintptr_t>(it.x);
+            const int vmax = (it.m % 4 == 0 && (xa & 15u) == 0) ? 4 : (it.m % 2 == 0 && (xa & 7u) == 0) ? 2 : 1;
+            MfmaMtpShape t = mfma_mtp_shape(it.n, it.m, it.r, vmax);
+            if (t.v != v) continue;
+            float* out = t.slabs > 1 ? mfma_partials + mfma_offs[(size_t)k] : it.q;
+            MfmaMtpItem mi = {it.x, it.p, out, it.n, (int)it.m, it.r, t.rows_per_slab, t.col_tiles};
+            table.push_back(mi);
+            blocks.push_back(t.col_tiles * t.slabs);
+            if (t.slabs > 1) {
+                const int64_t cnt = it.m * it.r;
+                SumItem si = {out, it.q, cnt, t.slabs};
+                sums.push_back(si);
+                sum_blocks.push_back((int)((cnt + 255) / 256));
+            }
+            done[(size_t)k] = 1;
+        }
+        if (table.empty()) continue;
+        int rc = run_batches(table, blocks, [&](const PsgdBatch<MfmaMtpItem>& bt, int grid) {
+            if (v == 4) hipLaunchKernelGGL(psgd_mfma_mtp_batch_kernel<4>, dim3((unsigned)grid), dim3(kMfmaThreads), 0, s, bt);
+            else if (v == 2) hipLaunchKernelGGL(psgd_mfma_mtp_batch_kernel<2>, dim3((unsigned)grid), dim3(kMfmaThreads), 0, s, bt);
+            else hipLaunchKernelGGL(psgd_mfma_mtp_batch_kernel<1>, dim3((unsigned)grid), dim3(kMfmaThreads), 0, s, bt);
+        });
+        if (rc != CONEF_OK) return rc;
+    }
     for (int k = 0; k < count; ++k) {
         if (done[(size_t)k]) continue;
         const ConefPsgdItem& lead = items[k];
@@ -1975,6 +2258,34 @@ int pqt_batch(const ConefPsgdItem* items, int count, int mode, float beta, int32
         if (done[(size_t)k]) continue;
         const ConefPsgdItem& lead = items[k];
         const int rp = rank_bound(lead.r);
+        if (mode != 2 && (lead.r == 16 || lead.r == 32) && aligned16(lead.p) && aligned16(lead.q)) {
+            // matrix-core items of one rank share a launch
+            std::vector<MfmaPqtItem> table;
+            std::vector<int> blocks;
+            for (int j = k; j < count; ++j) {
+                const ConefPsgdItem& it = items[j];
+                if (done[(size_t)j] || it.r != lead.r || !aligned16(it.p) || !aligned16(it.q)) continue;
+                int64_t col_wgs = (it.m + 32 * kMfmaWaves - 1) / (32 * kMfmaWaves);
+                int64_t slabs = (1024 + col_wgs - 1) / col_wgs;
+                int64_t rps = ((it.n + slabs - 1) / slabs + 31) / 32 * 32;
+                slabs = (it.n + rps - 1) / rps;
+                MfmaPqtItem t = {it.x, mode == 1 ? it.err : nullptr, it.p, it.q, it.n, (int)it.m, (int)rps, (int)col_wgs};
+                table.push_back(t);
+                blocks.push_back((int)(col_wgs * slabs));
+                done[(size_t)j] = 1;
+            }
+            int rc = run_batches(table, blocks, [&](const PsgdBatch<MfmaPqtItem>& bt, int grid) {
+                if (lead.r == 32) {
+                    if (mode == 1) hipLaunchKernelGGL((psgd_mfma_pqt_batch_kernel<32, 1>), dim3((unsigned)grid), dim3(kMfmaThreads), 0, s, bt);
+                    else hipLaunchKernelGGL((psgd_mfma_pqt_batch_kernel<32, 0>), dim3((unsigned)grid), dim3(kMfmaThreads), 0, s, bt);
+                } else {
+                    if (mode == 1) hipLaunchKernelGGL((psgd_mfma_pqt_batch_kernel<16, 1>), dim3((unsigned)grid), dim3(kMfmaThreads), 0, s, bt);
+                    else hipLaunchKernelGGL((psgd_mfma_pqt_batch_kernel<16, 0>), dim3((unsigned)grid), dim3(kMfmaThreads), 0, s, bt);
+                }
+            });
+            if (rc != CONEF_OK) return rc;
+            continue;
+        }
         if (rp >= 16 || mode == 2) {
             if (mode == 2 && rp < 16) {
                 // residual sketch on row-list plans: items of one rank class share launches
@@ -2072,7 +2383,8 @@ int64_t conef_psgd_batch_workspace_bytes(const ConefPsgdItem* items, int32_t cou
         int64_t b = conef_psgd_workspace_bytes(items[k].n, items[k].m, items[k].r);
         if (b > single) single = b;
     }
-    return conef_align256(single) + conef_align256(4 * mtp_batch_layout(items, count, nullptr));
+    return conef_align256(single) + conef_align256(4 * mtp_batch_layout(items, count, nullptr)) +
+           conef_align256(4 * mfma_batch_layout(items, count, nullptr));
 }
 
 int conef_psgd_mq_batch_f32(const ConefPsgdItem* items, int32_t count, int32_t mode, float alpha, int32_t a, int32_t b,
@@ -2108,6 +2420,42 @@ int conef_psgd_pqt_batch_f32(const ConefPsgdItem* items, int32_t count, int32_t 
     for (int k = 0; k < count; ++k)
         if (!item_ok(items[k]) || (mode == 1 && !items[k].err)) return CONEF_ERR_INVALID;
     return pqt_batch(items, count, mode, beta, a, b, (hipStream_t)stream);
+}
+
+// cs = update(cs, err, beta) in place for every item (DenseCS.update, CountSketch.py:27-48, with
+// vec = the item's dense [n,m] residual at err): the sketches of a bucket in one launch.  Every
+// item needs a row-list plan built for (n, m, w, a, b).
+int conef_psgd_sketch_update_batch_f32(const ConefPsgdItem* items, int32_t count, float beta, int32_t a, int32_t b,
+                                       void* stream)
+{
+    if (count < 0 || (count > 0 && !items)) return CONEF_ERR_INVALID;
+    std::vector<RowlistVecItem> table;
+    std::vector<int> blocks;
+    size_t lds = 0;
+    for (int k = 0; k < count; ++k) {
+        const ConefPsgdItem& it = items[k];
+        const ConefPlanHeader* hp = (const ConefPlanHeader*)it.plan_host;
+        if (!psgd_args_ok(it.n, it.m, it.r) || !it.err || !it.cs || !it.plan_dev ||
+            !conef_plan_matches(hp, it.n, it.m, it.w, a, b) || hp->kind != kConefPlanRowlist)
+            return CONEF_ERR_INVALID;
+        ConefRowlistShape shape;
+        if (!conef_rowlist_shape(it.n, it.m, it.w, ConefListVec::kNeedsCells, &shape, count)) return CONEF_ERR_INVALID;
+        RowlistVecItem t = {{it.err, aligned16(it.err) && it.m % 4 == 0}, conef_rowlist_view(hp, it.plan_dev), it.cs, it.cs,
+                            it.n, (int)it.m, it.w, shape.rb};
+        table.push_back(t);
+        blocks.push_back((int)shape.tiles);
+        if (shape.lds > lds) lds = shape.lds;
+    }
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)psgd_rowlist_vec_batch_kernel,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    const double omb = 1. - (double)beta;
+    hipStream_t s = (hipStream_t)stream;
+    return run_batches(table, blocks, [&](const PsgdBatch<RowlistVecItem>& bt, int grid) {
+        hipLaunchKernelGGL(psgd_rowlist_vec_batch_kernel, dim3((unsigned)grid), dim3(kConefRowlistThreads), lds, s, bt, omb);
+    });
 }
 
 // dense error feedback on the parts of a bucket that are not compressed: x += e; e = 0

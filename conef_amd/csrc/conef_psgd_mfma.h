@@ -38,17 +38,17 @@ constexpr int kMfmaThreads = 64 * kMfmaWaves;
 // more than one column split the tile goes to a partial buffer [split][n][r] that a second kernel
 // adds up in split order.  Requires m % 4 == 0 and 16-byte aligned x (err, pktab).
 template <int MODE>
-__global__ void __launch_bounds__(kMfmaThreads)
-psgd_mfma_mq_kernel(float* __restrict__ x, const float* __restrict__ err, const float* __restrict__ cs,
-                    const uint32_t* __restrict__ pktab, const float* __restrict__ q, float* __restrict__ out, int64_t n,
-                    int m, int r, int cols_per_split, ConefMod mod, float alpha, ConefSeeds hs)
+__device__ __forceinline__ void
+psgd_mfma_mq_body(float* __restrict__ x, const float* __restrict__ err, const float* __restrict__ cs,
+                  const uint32_t* __restrict__ pktab, const float* __restrict__ q, float* __restrict__ out, int64_t n,
+                  int m, int r, int cols_per_split, ConefMod mod, float alpha, ConefSeeds hs, int bx, int by)
 {
     extern __shared__ float mfma_lds[];
     float* red = mfma_lds;                              // [kMfmaWaves][16][64]
     float* cells = mfma_lds + kMfmaWaves * 16 * 64;     // [32][w], MODE 2 only
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int lrow = lane & 31, half = lane >> 5;
-    const int64_t row0 = (int64_t)blockIdx.x * 32;
+    const int64_t row0 = (int64_t)bx * 32;
     const int64_t row = row0 + lrow < n ? row0 + lrow : n - 1;     // clamped for loads, stores are guarded
     const bool row_ok = row0 + lrow < n;
     const int w = (int)mod.w;
@@ -60,7 +60,7 @@ psgd_mfma_mq_kernel(float* __restrict__ x, const float* __restrict__ err, const 
         }
         __syncthreads();
     }
-    const int c_begin = blockIdx.y * cols_per_split;
+    const int c_begin = by * cols_per_split;
     const int c_end = c_begin + cols_per_split < m ? c_begin + cols_per_split : m;
     const bool rank_ok = lrow < r;
     conef_f16v acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -142,7 +142,7 @@ psgd_mfma_mq_kernel(float* __restrict__ x, const float* __restrict__ err, const 
 #pragma unroll
     for (int v = 0; v < 16; ++v) red[(wave * 16 + v) * 64 + lane] = acc[v];
     __syncthreads();
-    float* dst = out + (int64_t)blockIdx.y * n * r;
+    float* dst = out + (int64_t)by * n * r;
     for (int e = threadIdx.x; e < 16 * 64; e += kMfmaThreads) {
         const int v = e >> 6, l = e & 63;
         float s = (red[e] + red[16 * 64 + e]) + (red[2 * 16 * 64 + e] + red[3 * 16 * 64 + e]);
@@ -150,6 +150,16 @@ psgd_mfma_mq_kernel(float* __restrict__ x, const float* __restrict__ err, const 
         const int j = l & 31;
         if (i < n && j < r) dst[i * r + j] = s;
     }
+}
+
+template <int MODE>
+__global__ void __launch_bounds__(kMfmaThreads)
+psgd_mfma_mq_kernel(float* __restrict__ x, const float* __restrict__ err, const float* __restrict__ cs,
+                    const uint32_t* __restrict__ pktab, const float* __restrict__ q, float* __restrict__ out, int64_t n,
+                    int m, int r, int cols_per_split, ConefMod mod, float alpha, ConefSeeds hs)
+{
+    psgd_mfma_mq_body<MODE>(x, err, cs, pktab, q, out, n, m, r, cols_per_split, mod, alpha, hs, (int)blockIdx.x,
+                            (int)blockIdx.y);
 }
 
 // -------------------------------------------------------------- Q = X^T P ----
@@ -160,18 +170,18 @@ psgd_mfma_mq_kernel(float* __restrict__ x, const float* __restrict__ err, const 
 // rows of the slab, meet in LDS, and the slab's tile is stored (one slab) or left as a partial.
 // Requires m % V == 0 and V*4-byte aligned x.
 template <int V>
-__global__ void __launch_bounds__(kMfmaThreads)
-psgd_mfma_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, float* __restrict__ out, int64_t n, int m,
-                     int r, int rows_per_slab)
+__device__ __forceinline__ void
+psgd_mfma_mtp_body(const float* __restrict__ x, const float* __restrict__ p, float* __restrict__ out, int64_t n, int m,
+                   int r, int rows_per_slab, int bx, int by)
 {
     __shared__ float red[kMfmaWaves][16][64];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int lq = lane & 31, half = lane >> 5;
-    const int c0 = blockIdx.x * 32 * V;
+    const int c0 = bx * 32 * V;
     const int c = c0 + V * lq;
     const bool col_ok = c < m;
     const int cc = col_ok ? c : 0;
-    const int64_t i0 = (int64_t)blockIdx.y * rows_per_slab;
+    const int64_t i0 = (int64_t)by * rows_per_slab;
     const int64_t i1 = i0 + rows_per_slab < n ? i0 + rows_per_slab : n;
     const bool rank_ok = lq < r;
     conef_f16v acc[V];
@@ -228,7 +238,7 @@ psgd_mfma_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, f
             ib = nb;
         }
     }
-    float* dst = out + (int64_t)blockIdx.y * m * r;
+    float* dst = out + (int64_t)by * m * r;
 #pragma unroll
     for (int t = 0; t < V; ++t) {
         if (t) __syncthreads();
@@ -246,6 +256,14 @@ psgd_mfma_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, f
     }
 }
 
+template <int V>
+__global__ void __launch_bounds__(kMfmaThreads)
+psgd_mfma_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, float* __restrict__ out, int64_t n, int m,
+                     int r, int rows_per_slab)
+{
+    psgd_mfma_mtp_body<V>(x, p, out, n, m, r, rows_per_slab, (int)blockIdx.x, (int)blockIdx.y);
+}
+
 // ------------------------------------------------------------ M = P Q^T ----
 // D[i][c] = sum_k P[i][k] Q[c][k] with K = R (16 or 32): R/2 steps per 32x32 tile.  Lane
 // (t = l % 32, half) supplies k = half * R/2 + s at step s for both operands, so its slice of a
@@ -253,15 +271,15 @@ psgd_mfma_mtp_kernel(const float* __restrict__ x, const float* __restrict__ p, f
 // 32 columns in registers and walks the row tiles of its slab; a half-wave stores 128 contiguous
 // bytes of a row of M.  MODE 1 also writes the residual E = X - M (X = what M held on entry).
 template <int R, int MODE>
-__global__ void __launch_bounds__(kMfmaThreads)
-psgd_mfma_pqt_kernel(float* __restrict__ x, float* __restrict__ err, const float* __restrict__ p,
-                     const float* __restrict__ q, int64_t n, int m, int rows_per_slab)
+__device__ __forceinline__ void
+psgd_mfma_pqt_body(float* __restrict__ x, float* __restrict__ err, const float* __restrict__ p,
+                   const float* __restrict__ q, int64_t n, int m, int rows_per_slab, int bx, int by)
 {
     constexpr int KS = R / 2;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int lt = lane & 31, half = lane >> 5;
-    const int c = (blockIdx.x * kMfmaWaves + wave) * 32 + lt;
-    if ((blockIdx.x * kMfmaWaves + wave) * 32 >= m) return;        // whole wave past the edge (no barriers below)
+    const int c = (bx * kMfmaWaves + wave) * 32 + lt;
+    if ((bx * kMfmaWaves + wave) * 32 >= m) return;        // whole wave past the edge (no barriers below)
     const bool col_ok = c < m;
     float qb[KS];
     {
@@ -272,7 +290,7 @@ psgd_mfma_pqt_kernel(float* __restrict__ x, float* __restrict__ err, const float
             qb[s] = t.x; qb[s + 1] = t.y; qb[s + 2] = t.z; qb[s + 3] = t.w;
         }
     }
-    const int64_t i0 = (int64_t)blockIdx.y * rows_per_slab;
+    const int64_t i0 = (int64_t)by * rows_per_slab;
     const int64_t i1 = i0 + rows_per_slab < n ? i0 + rows_per_slab : n;
     for (int64_t ib = i0; ib < i1; ib += 32) {
         float pa[KS], xv[16];
@@ -304,4 +322,12 @@ psgd_mfma_pqt_kernel(float* __restrict__ x, float* __restrict__ err, const float
             }
         }
     }
+}
+
+template <int R, int MODE>
+__global__ void __launch_bounds__(kMfmaThreads)
+psgd_mfma_pqt_kernel(float* __restrict__ x, float* __restrict__ err, const float* __restrict__ p,
+                     const float* __restrict__ q, int64_t n, int m, int rows_per_slab)
+{
+    psgd_mfma_pqt_body<R, MODE>(x, err, p, q, n, m, rows_per_slab, (int)blockIdx.x, (int)blockIdx.y);
 }

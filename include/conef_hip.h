@@ -275,6 +275,13 @@ int conef_psgd_mtp_batch_f32(const ConefPsgdItem* items, int32_t count, void* wo
 int conef_psgd_pqt_batch_f32(const ConefPsgdItem* items, int32_t count, int32_t mode, float beta, int32_t a, int32_t b,
                              void* stream);
 
+/* cs = update(cs, err, beta) in place for every item, err the item's dense [n,m] residual
+ * (DenseCS.update, compressors/CountSketch.py:27-48, once per matrix in the reference's hook,
+ * powerSGD_hook.py:564): the sketches of a bucket in one launch.  Every item needs a row-list
+ * plan for (n, m, w, a, b). */
+int conef_psgd_sketch_update_batch_f32(const ConefPsgdItem* items, int32_t count, float beta, int32_t a, int32_t b,
+                                       void* stream);
+
 /* Dense error feedback on a stretch of the bucket that is not compressed: x += err; err = 0
  * (the copy-minus-result of powerSGD_hook.py:558 is exactly zero there). */
 int conef_ef_passthrough_f32(float* x, float* err, int64_t count, void* stream);

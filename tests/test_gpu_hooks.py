@@ -244,7 +244,10 @@ def test_batch_products_parity(oracle):
     lib = _lib.load()
     rng = np.random.RandomState(4)
     specs = [(64, 576, 2, 0), (640, 1440, 4, 0), (1024, 1024, 8, 0), (13, 29, 3, 0), (300, 4096, 32, 0), (37, 4096, 8, 2),
-             (2049, 260, 4, 0), (16, 27, 2, 0), (5000, 64, 1, 0), (128, 128, 16, 0)] + [(96 + k, 200, 4, 0) for k in range(30)]
+             (2049, 260, 4, 0), (16, 27, 2, 0), (5000, 64, 1, 0), (128, 128, 16, 0),
+             # matrix-core items share launches when m % 4 == 0 and the matrix is 16-byte aligned
+             (1024, 1024, 32, 0), (1000, 516, 32, 0), (4096, 1024, 32, 0), (33, 4096, 16, 0), (100, 130, 32, 0),
+             (2049, 1000, 20, 0), (77, 128, 16, 1), (1024, 4096, 32, 0)] + [(96 + k, 200, 4, 0) for k in range(30)]
     for mode in (0, 1):
         items = (_lib.PsgdItem * len(specs))()
         keep, host = [], []
@@ -319,6 +322,64 @@ def test_products_with_sketch_on_a_plan(oracle):
         assert_close(low, oracle.pqt(P, Q), what="PQt %s" % ((n, m, r),))
         ocs.update(MQ - low, 0.9)         # the residual against the low-rank product the GPU wrote
         np.testing.assert_array_equal(to_np(cs.cs), ocs.cs)
+
+
+def test_batch_sketched_products_on_matrix_cores(oracle):
+    """Ranks 16 and 32 in a batch with count-sketch error: the query of all matrices in one launch
+    (bucket and sign from the plan's table, or hashed where a matrix has no plan), the products on
+    the matrix cores, the dense residual, and all sketches updated from it in one launch - sketches
+    bit for bit."""
+    from conef_amd import _lib
+    from conef_amd.compressors.CountSketch import DenseCS
+    lib = _lib.load()
+    rng = np.random.RandomState(12)
+    specs = [(1024, 1024, 32, 0.1), (256, 1024, 32, 0.1), (1024, 256, 16, 0.2), (300, 4096, 32, 0.05), (64, 128, 16, 0.5),
+             (2048, 512, 32, 0.1)]
+    count = len(specs)
+    items = (_lib.PsgdItem * count)()
+    keep, host = [], []
+    for k, (n, m, r, ss) in enumerate(specs):
+        M = rng.randn(n, m).astype(np.float32)
+        Q = rng.randn(m, r).astype(np.float32)
+        cs, ocs = DenseCS(n, m, ss), oracle.DenseCS(n, m, ss)
+        ocs.cs[:] = rng.randn(n, cs.range).astype(np.float32)
+        cs.cs.copy_(torch.from_numpy(ocs.cs))
+        plan = cs.plan()
+        assert plan is not None and plan.in_place
+        Md, Qd = torch.from_numpy(M).cuda(), torch.from_numpy(Q).cuda()
+        Pd, Rd = torch.empty(n, r, device="cuda"), torch.empty(n, m, device="cuda")
+        it = items[k]
+        it.x, it.cs, it.p, it.q, it.n, it.m, it.r, it.w = Md.data_ptr(), cs.cs.data_ptr(), Pd.data_ptr(), Qd.data_ptr(), n, m, r, cs.range
+        if k != 1:                      # one matrix without a plan: its query hashes
+            it.plan_host, it.plan_dev = plan.host_ptr, plan.device.data_ptr()
+        keep.append((Md, Qd, Pd, Rd, cs, plan))
+        host.append((M, Q, ocs))
+    a, b = keep[0][4].a, keep[0][4].b
+    ws = torch.empty(lib.conef_psgd_batch_workspace_bytes(items, count), dtype=torch.uint8, device="cuda")
+    assert lib.conef_psgd_mq_batch_f32(items, count, 2, 0.1, a, b, ws.data_ptr(), ws.numel(), 0) == 0
+    xs = []
+    for (Md, Qd, Pd, Rd, cs, plan), (M, Q, ocs), spec in zip(keep, host, specs):
+        X = M.copy()
+        ocs.query(X, 0.1)
+        np.testing.assert_array_equal(to_np(Md), X)
+        assert_close(Pd, oracle.mq(X, Q), what="batch MQ + sketch %s" % (spec,))
+        xs.append(X)
+    assert lib.conef_psgd_mtp_batch_f32(items, count, ws.data_ptr(), ws.numel(), 0) == 0
+    for (Md, Qd, Pd, Rd, cs, plan), X, spec in zip(keep, xs, specs):
+        assert_close(Qd, oracle.mtp(X, to_np(Pd)), what="batch MtP %s" % (spec,))
+    for k, (Md, Qd, Pd, Rd, cs, plan) in enumerate(keep):
+        items[k].err = Rd.data_ptr()
+        items[k].plan_host, items[k].plan_dev = plan.host_ptr, plan.device.data_ptr()
+    assert lib.conef_psgd_pqt_batch_f32(items, count, 1, 0.0, a, b, 0) == 0
+    assert lib.conef_psgd_sketch_update_batch_f32(items, count, 0.9, a, b, 0) == 0
+    for (Md, Qd, Pd, Rd, cs, plan), (M, Q, ocs), X, spec in zip(keep, host, xs, specs):
+        low = to_np(Md)
+        assert_close(low, oracle.pqt(to_np(Pd), to_np(Qd)), what="batch PQt %s" % (spec,))
+        np.testing.assert_array_equal(to_np(Rd), X - low)
+        ocs.update(X - low, 0.9)
+        np.testing.assert_array_equal(to_np(cs.cs), ocs.cs)
+    items[0].plan_dev = None
+    assert lib.conef_psgd_sketch_update_batch_f32(items, count, 0.9, a, b, 0) == -1      # every item needs its plan
 
 
 def psgd_check_factory(st, ost, mode):
