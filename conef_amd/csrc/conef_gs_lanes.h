@@ -242,25 +242,17 @@ __device__ __forceinline__ void gsw_publish_column(float (&col)[RPT], float* pb,
     }
 }
 
-// Matrix batch.a[blockIdx.x]: [rows, RP] row-major, rows <= 64 RPT, in place.
+// The workgroup's rows of a row-major [rows, RP] matrix into registers and back: v[cc][t] is row
+// lane + 64 t of column col0 + cc.  Coalesced dwords to an LDS tile (row stride RP + 1), columns
+// out of the tile; rows past the end read as zero.  All threads of the workgroup call these.
 template <int RP, int RPT, int CW>
-__global__ void __launch_bounds__(64 * RP / CW)
-gsw_kernel(GswBatch batch, float eps)
+__device__ __forceinline__ void gsw_load_columns(const float* __restrict__ a, int rows, float* tile, float (&v)[CW][RPT],
+                                                 int tid, int lane, int col0)
 {
     constexpr int T = 64 * RP / CW, LD = RP + 1;
-    constexpr int PS = RPT + 4;      // a lane's slice of the pivot column: 16-byte accesses of 16 lanes then cover all banks once
     constexpr int CAP = 64 * RPT, TR = CAP < kGswTileRows ? CAP : kGswTileRows, NCH = CAP / TR, SPC = TR / 64;
     constexpr int JN = TR * RP / T, JU = JN % 16 == 0 ? 16 : JN % 8 == 0 ? 8 : 4;      // tile elements per thread, loads in flight
     static_assert(RPT % 4 == 0 && CAP % TR == 0 && RP % CW == 0 && JN % JU == 0, "wave-owns-columns layout");
-    extern __shared__ __attribute__((aligned(16))) float gsw_lds[];
-    float* piv = gsw_lds;                       // [2][64][PS]: the normalised pivot column, lane-major
-    float* tile = gsw_lds + 2 * 64 * PS;        // [TR][LD]
-    float* __restrict__ a = batch.a[blockIdx.x];
-    const int rows = batch.rows[blockIdx.x];
-    const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int col0 = w * CW;
-
-    float v[CW][RPT];
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
         const int r0 = k * TR;
@@ -286,7 +278,7 @@ gsw_kernel(GswBatch batch, float eps)
 #pragma unroll
             for (int t = 0; t < SPC; ++t) {
 #pragma unroll
-                for (int cc = 0; cc < CW; ++cc) v[cc][k * SPC + t] = tile[(lane + 64 * t) * LD + col0 + cc];   // rows past the end: zero fill
+                for (int cc = 0; cc < CW; ++cc) v[cc][k * SPC + t] = tile[(lane + 64 * t) * LD + col0 + cc];
             }
             __syncthreads();
         } else {
@@ -297,6 +289,54 @@ gsw_kernel(GswBatch batch, float eps)
             }
         }
     }
+}
+
+template <int RP, int RPT, int CW>
+__device__ __forceinline__ void gsw_store_columns(float* __restrict__ a, int rows, float* tile, const float (&v)[CW][RPT],
+                                                  int tid, int lane, int col0)
+{
+    constexpr int T = 64 * RP / CW, LD = RP + 1;
+    constexpr int CAP = 64 * RPT, TR = CAP < kGswTileRows ? CAP : kGswTileRows, NCH = CAP / TR, SPC = TR / 64;
+    constexpr int JN = TR * RP / T;
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const int r0 = k * TR;
+        if (r0 < rows) {
+            if (k > 0) __syncthreads();
+#pragma unroll
+            for (int t = 0; t < SPC; ++t) {
+#pragma unroll
+                for (int cc = 0; cc < CW; ++cc) tile[(lane + 64 * t) * LD + col0 + cc] = v[cc][k * SPC + t];
+            }
+            __syncthreads();
+            const int n = (rows - r0 < TR ? rows - r0 : TR) * RP;
+            float* dst = a + (int64_t)r0 * RP;
+#pragma unroll 8
+            for (int j = 0; j < JN; ++j) {
+                const int e = tid + T * j;
+                const int row = e / RP, c = e - row * RP;
+                if (e < n) dst[e] = tile[row * LD + c];
+            }
+        }
+    }
+}
+
+// Matrix batch.a[blockIdx.x]: [rows, RP] row-major, rows <= 64 RPT, in place.
+template <int RP, int RPT, int CW>
+__global__ void __launch_bounds__(64 * RP / CW)
+gsw_kernel(GswBatch batch, float eps)
+{
+    constexpr int PS = RPT + 4;      // a lane's slice of the pivot column: 16-byte accesses of 16 lanes then cover all banks once
+    extern __shared__ __attribute__((aligned(16))) float gsw_lds[];
+    float* piv = gsw_lds;                       // [2][64][PS]: the normalised pivot column, lane-major
+    float* tile = gsw_lds + 2 * 64 * PS;        // [TR][RP + 1]
+    float* __restrict__ a = batch.a[blockIdx.x];
+    const int rows = batch.rows[blockIdx.x];
+    const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col0 = w * CW;
+
+    float v[CW][RPT];
+    gsw_load_columns<RP, RPT, CW>(a, rows, tile, v, tid, lane, col0);
 
     // Normalises this wave's column i and publishes it: a lane's slice of the column is RPT words,
     // written and read 16 bytes at a time.
@@ -304,17 +344,10 @@ gsw_kernel(GswBatch batch, float eps)
         float* pb = piv + (i & 1) * (64 * PS) + lane * PS;
         if constexpr (CW == 1) {
             gsw_publish_column<RPT>(v[0], pb, eps);
-        } else if constexpr (CW == 2) {
+        } else {
+            static_assert(CW == 2, "columns per wave");
             if (i % 2 == 0) gsw_publish_column<RPT>(v[0], pb, eps);
             else gsw_publish_column<RPT>(v[1], pb, eps);
-        } else {
-            static_assert(CW == 4, "columns per wave");
-            switch (i % 4) {
-                case 0: gsw_publish_column<RPT>(v[0], pb, eps); break;
-                case 1: gsw_publish_column<RPT>(v[1], pb, eps); break;
-                case 2: gsw_publish_column<RPT>(v[2], pb, eps); break;
-                default: gsw_publish_column<RPT>(v[3], pb, eps); break;
-            }
         }
     };
 
@@ -369,26 +402,5 @@ gsw_kernel(GswBatch batch, float eps)
         }
         __syncthreads();
     }
-
-#pragma unroll
-    for (int k = 0; k < NCH; ++k) {
-        const int r0 = k * TR;
-        if (r0 < rows) {
-            if (k > 0) __syncthreads();
-#pragma unroll
-            for (int t = 0; t < SPC; ++t) {
-#pragma unroll
-                for (int cc = 0; cc < CW; ++cc) tile[(lane + 64 * t) * LD + col0 + cc] = v[cc][k * SPC + t];
-            }
-            __syncthreads();
-            const int n = (rows - r0 < TR ? rows - r0 : TR) * RP;
-            float* dst = a + (int64_t)r0 * RP;
-#pragma unroll 8
-            for (int j = 0; j < JN; ++j) {
-                const int e = tid + T * j;
-                const int row = e / RP, c = e - row * RP;
-                if (e < n) dst[e] = tile[row * LD + c];
-            }
-        }
-    }
+    gsw_store_columns<RP, RPT, CW>(a, rows, tile, v, tid, lane, col0);
 }

@@ -1299,7 +1299,9 @@ struct MfmaMtpShape {
     int v, col_tiles, slabs, rows_per_slab;
 };
 
-inline MfmaMtpShape mfma_mtp_shape(int64_t n, int64_t m, int r, int vmax)
+// want_wgs: workgroups the matrix should bring (512 alone; its share of them inside a batch, where
+// wider lanes then win: fewer, fuller workgroups per matrix)
+inline MfmaMtpShape mfma_mtp_shape(int64_t n, int64_t m, int r, int vmax, int64_t want_wgs = 512)
 {
     MfmaMtpShape g = {1, 0, 1, 0};
     int64_t slabs_most = n / (4 * (int64_t)r);
@@ -1307,12 +1309,12 @@ inline MfmaMtpShape mfma_mtp_shape(int64_t n, int64_t m, int r, int vmax)
     if (slabs_most > (n + 7) / 8) slabs_most = (n + 7) / 8;
     for (int v = vmax; v >= 1; v >>= 1) {
         int64_t tiles = (m + 32 * v - 1) / (32 * v);
-        int64_t want = (512 + tiles - 1) / tiles;
+        int64_t want = (want_wgs + tiles - 1) / tiles;
         int64_t slabs = want < slabs_most ? want : slabs_most;
         g.v = v;
         g.col_tiles = (int)tiles;
         g.slabs = (int)slabs;
-        if (tiles * slabs >= 512 || v == 1) break;
+        if (tiles * slabs >= want_wgs || v == 1) break;
     }
     int64_t rps = ((n + g.slabs - 1) / g.slabs + 7) / 8 * 8;
     g.rows_per_slab = (int)rps;
@@ -2114,7 +2116,11 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
     std::vector<char> done((size_t)count, 0);
     std::vector<SumItem> sums;
     std::vector<int> sum_blocks;
-    // matrix-core items: one launch per vector width (4, 2 or 1 floats a lane, by the alignment of x)
+    // matrix-core items: one launch per vector width (4, 2 or 1 floats a lane, by the alignment of x
+    // and by how many workgroups the matrix has to bring to a launch it shares)
+    int mfma_items = 0;
+    for (int k = 0; k < count; ++k) mfma_items += rank_bound(items[k].r) >= 16;
+    const int64_t want_wgs = mfma_items > 0 && 768 / mfma_items > 96 ? 768 / mfma_items : 96;
     for (int v = 4; v >= 1 && mfma_partials; v >>= 1) {
         std::vector<MfmaMtpItem> table;
         std::vector<int> blocks;
@@ -2123,7 +2129,7 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
             if (done[(size_t)k] || rank_bound(it.r) < 16) continue;
             const uintptr_t xa = reinterpret_cast<uintptr_t>(it.x);
             const int vmax = (it.m % 4 == 0 && (xa & 15u) == 0) ? 4 : (it.m % 2 == 0 && (xa & 7u) == 0) ? 2 : 1;
-            MfmaMtpShape t = mfma_mtp_shape(it.n, it.m, it.r, vmax);
+            MfmaMtpShape t = mfma_mtp_shape(it.n, it.m, it.r, vmax, want_wgs < 512 ? want_wgs : 512);
             if (t.v != v) continue;
             float* out = t.slabs > 1 ? mfma_partials + mfma_offs[(size_t)k] : it.q;
             MfmaMtpItem mi = {it.x, it.p, out, it.n, (int)it.m, it.r, t.rows_per_slab, t.col_tiles};
