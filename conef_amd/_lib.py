@@ -72,6 +72,8 @@ SIGNATURES = {
                                                _I32, _I32, _P],
     "conef_topk_workspace_bytes": [_I64],
     "conef_topk_sparsify_f32": [_P, _I64, _I64, _P, _I64, _P],
+    "conef_topk_batch_workspace_bytes": [_P, _I32],
+    "conef_topk_sparsify_batch_f32": [_P, _P, _P, _I32, _P, _I64, _P],
 }
 
 class PsgdItem(ctypes.Structure):
@@ -80,8 +82,8 @@ class PsgdItem(ctypes.Structure):
                 ("n", _I64), ("m", _I64), ("r", _I32), ("w", _I32)]
 
 
-_RETURNS_I64 = ("conef_topk_workspace_bytes", "conef_plan_bytes", "conef_plan_workspace_bytes",
-                "conef_psgd_workspace_bytes", "conef_psgd_batch_workspace_bytes")
+_RETURNS_I64 = ("conef_topk_workspace_bytes", "conef_topk_batch_workspace_bytes", "conef_plan_bytes",
+                "conef_plan_workspace_bytes", "conef_psgd_workspace_bytes", "conef_psgd_batch_workspace_bytes")
 
 _handle = None
 

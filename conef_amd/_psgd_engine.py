@@ -94,13 +94,40 @@ def topk_sparsify(err, topk_ratio, workspace=None):
     return workspace
 
 
+def topk_sparsify_all(tensors, topk_ratio, table=None):
+    """``topk_sparsify`` of every tensor of a list (one stream, one device) with each pass a
+    single launch over all of them.  ``table`` is what an earlier call over the same tensors
+    returned: the host arrays and the workspace are reused while the tensors stay where they are."""
+    import ctypes
+    count = len(tensors)
+    if count == 0:
+        return table
+    key = tuple(t.data_ptr() for t in tensors)
+    lib = _lib.load()
+    if table is None or table[0] != key:
+        for t in tensors:
+            _lib.require_device_f32(t, "err")
+        ptrs = (ctypes.c_void_p * count)(*key)
+        numels = (ctypes.c_int64 * count)(*[t.numel() for t in tensors])
+        ks = (ctypes.c_int64 * count)(*[max(1, int(0.5 * topk_ratio * t.numel())) for t in tensors])
+        ws = torch.empty(lib.conef_topk_batch_workspace_bytes(numels, count), dtype=torch.uint8, device=tensors[0].device)
+        table = (key, ptrs, numels, ks, ws, topk_ratio)
+    elif table[5] != topk_ratio:
+        return topk_sparsify_all(tensors, topk_ratio, None)
+    _, ptrs, numels, ks, ws, _ = table
+    rc = lib.conef_topk_sparsify_batch_f32(ptrs, numels, ks, count, ws.data_ptr(), ws.numel(), _lib.stream_ptr(tensors[0]))
+    _lib.check(rc, "conef_topk_sparsify_batch_f32")
+    return table
+
+
 class _RoundPlan:
     """What a bucket's round needs that does not change from step to step: which tensors are
     compressed, the table of matrices the batch entry points read, the views into the P / Q
     arenas.  Built on the first step of a bucket and reused while the bucket keeps its buffer
     and layout, so that a step costs a handful of foreign calls however many tensors it has."""
     __slots__ = ("key", "shapes", "work", "passthrough", "before", "after", "total_ps", "total_qs", "arena_key", "ps",
-                 "qs", "gs_p", "gs_q", "items", "count", "sketches", "fused_sketch", "batched_update", "residual_offsets")
+                 "qs", "gs_p", "gs_q", "items", "count", "sketches", "fused_sketch", "batched_update", "residual_offsets",
+                 "topk_table")
 
 
 def _gs_table(matrices):
@@ -140,6 +167,7 @@ def _build_round(state, grads, shapes, key, error_mode):
     plan.sketches = []
     plan.fused_sketch = False
     plan.batched_update = False
+    plan.topk_table = None
     plan.residual_offsets = []
     off = 0
     for _, n, m, _ in plan.work:
@@ -307,9 +335,7 @@ def run_round(state, bucket, error_mode):
                                       stream)
     _lib.check(rc, "conef_psgd_pqt_batch_f32")
     if error_mode == "topk":
-        topk_ws = None
-        for cnt in range(count):
-            topk_ws = topk_sparsify(errs[cnt], state.topk_ratio, topk_ws)
+        plan.topk_table = topk_sparsify_all([errs[cnt] for cnt in range(count)], state.topk_ratio, plan.topk_table)
     elif residual is not None and error_mode == "conef" and plan.batched_update:
         # every sketch of the bucket from its matrix's residual, in one launch
         rc = lib.conef_psgd_sketch_update_batch_f32(items, count, float(state.beta), HASH_A, HASH_B, stream)

@@ -33,16 +33,52 @@ struct TopkState {
 
 __device__ __forceinline__ uint32_t mag_key(float v) { return __float_as_uint(v) & 0x7fffffffu; }
 
-__global__ void topk_init_kernel(TopkState* st, uint32_t k)
+// Several tensors per launch (the dense errors of a bucket's matrices, each with its own k and its
+// own state): the table travels by value, a workgroup finds its tensor from the running workgroup
+// count of the pass (`first_h` for the histogram passes, `first_c` for the chunked ones) and then
+// does what it would do in a launch of its own.
+constexpr int kTopkBatchMax = 24;
+
+struct TopkItem {
+    float* x;
+    int64_t numel, chunks;
+    TopkState* st;
+    uint32_t* chunk_ties;
+    uint32_t k;
+};
+
+struct TopkBatch {
+    TopkItem item[kTopkBatchMax];
+    int first_h[kTopkBatchMax + 1];
+    int first_c[kTopkBatchMax + 1];
+    int count;
+};
+
+__device__ __forceinline__ int topk_locate(const int* first, int count, int* local, int* width)
+{
+    int i = 0;
+    while (i + 1 < count && (int)blockIdx.x >= first[i + 1]) ++i;
+    *local = (int)blockIdx.x - first[i];
+    *width = first[i + 1] - first[i];
+    return i;
+}
+
+__device__ __forceinline__ void topk_init_body(TopkState* st, uint32_t k)
 {
     for (int i = threadIdx.x; i < kPasses * kBins; i += blockDim.x) (&st->hist[0][0])[i] = 0u;
     if (threadIdx.x == 0) st->k = k;
 }
 
+__global__ void topk_init_kernel(TopkState* st, uint32_t k) { topk_init_body(st, k); }
+
+__global__ void topk_init_batch_kernel(TopkBatch b) { topk_init_body(b.item[blockIdx.x].st, b.item[blockIdx.x].k); }
+
 // What pass `p` selected, from its finished histogram: the digit holding the k-th largest key
 // among those matching the earlier digits.  Every thread of a 256-thread workgroup returns the
-// same (prefix, remaining, ties); workgroup 0 also leaves them in the state for the next kernel.
-__device__ __forceinline__ void topk_resolve(TopkState* st, int p, uint32_t* prefix, uint32_t* remaining, uint32_t* ties)
+// same (prefix, remaining, ties); workgroup 0 (bx) of the tensor also leaves them in the state for
+// the next kernel.
+__device__ __forceinline__ void topk_resolve(TopkState* st, int p, uint32_t* prefix, uint32_t* remaining, uint32_t* ties,
+                                             int bx)
 {
     __shared__ uint32_t wave_sum[4];
     __shared__ uint32_t picked[3];
@@ -80,7 +116,7 @@ __device__ __forceinline__ void topk_resolve(TopkState* st, int p, uint32_t* pre
     *prefix = picked[0];
     *remaining = picked[1];
     *ties = picked[2];
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (bx == 0 && threadIdx.x == 0) {
         st->prefix[p] = picked[0];
         st->remaining[p] = picked[1];
         st->ties[p] = picked[2];
@@ -88,12 +124,12 @@ __device__ __forceinline__ void topk_resolve(TopkState* st, int p, uint32_t* pre
     __syncthreads();
 }
 
-__global__ void __launch_bounds__(256)
-topk_hist_kernel(const float* __restrict__ x, int64_t numel, TopkState* st, int pass)
+__device__ __forceinline__ void
+topk_hist_body(const float* __restrict__ x, int64_t numel, TopkState* st, int pass, int bx, int gx)
 {
     __shared__ uint32_t bins[kBins];
     uint32_t prefix = 0, remaining = 0, ties = 0;
-    if (pass > 0) topk_resolve(st, pass - 1, &prefix, &remaining, &ties);
+    if (pass > 0) topk_resolve(st, pass - 1, &prefix, &remaining, &ties, bx);
     const int nb = 1 << kDigitBits[pass];
     for (int i = threadIdx.x; i < nb; i += 256) bins[i] = 0u;
     __syncthreads();
@@ -101,9 +137,9 @@ topk_hist_kernel(const float* __restrict__ x, int64_t numel, TopkState* st, int 
     const uint32_t mask = (uint32_t)nb - 1u;
     const int64_t quads = numel >> 2;
     const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
-    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    int64_t stride = (int64_t)gx * blockDim.x;
     if (vec) {
-        for (int64_t q = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; q < quads; q += stride) {
+        for (int64_t q = bx * (int64_t)blockDim.x + threadIdx.x; q < quads; q += stride) {
             float4 v = reinterpret_cast<const float4*>(x)[q];
             uint32_t key[4] = {mag_key(v.x), mag_key(v.y), mag_key(v.z), mag_key(v.w)};
 #pragma unroll
@@ -111,7 +147,7 @@ topk_hist_kernel(const float* __restrict__ x, int64_t numel, TopkState* st, int 
                 if (pass == 0 || (key[e] >> hi) == prefix) atomicAdd(&bins[(key[e] >> shift) & mask], 1u);
         }
     }
-    for (int64_t i = (vec ? quads * 4 : 0) + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < numel; i += stride) {
+    for (int64_t i = (vec ? quads * 4 : 0) + bx * (int64_t)blockDim.x + threadIdx.x; i < numel; i += stride) {
         uint32_t key = mag_key(x[i]);
         if (pass == 0 || (key >> hi) == prefix) atomicAdd(&bins[(key >> shift) & mask], 1u);
     }
@@ -122,16 +158,30 @@ topk_hist_kernel(const float* __restrict__ x, int64_t numel, TopkState* st, int 
     }
 }
 
-// per-chunk count of keys equal to the threshold
 __global__ void __launch_bounds__(256)
-topk_count_ties_kernel(const float* __restrict__ x, int64_t numel, TopkState* st, uint32_t* chunk_ties,
-                       int64_t chunks)
+topk_hist_kernel(const float* __restrict__ x, int64_t numel, TopkState* st, int pass)
+{
+    topk_hist_body(x, numel, st, pass, (int)blockIdx.x, (int)gridDim.x);
+}
+
+__global__ void __launch_bounds__(256)
+topk_hist_batch_kernel(TopkBatch b, int pass)
+{
+    int local, width;
+    const TopkItem& it = b.item[topk_locate(b.first_h, b.count, &local, &width)];
+    topk_hist_body(it.x, it.numel, it.st, pass, local, width);
+}
+
+// per-chunk count of keys equal to the threshold
+__device__ __forceinline__ void
+topk_count_ties_body(const float* __restrict__ x, int64_t numel, TopkState* st, uint32_t* chunk_ties, int64_t chunks,
+                     int bx, int gx)
 {
     __shared__ uint32_t total;
     uint32_t thr, keep_ties, ties;
-    topk_resolve(st, kPasses - 1, &thr, &keep_ties, &ties);
+    topk_resolve(st, kPasses - 1, &thr, &keep_ties, &ties, bx);
     if (ties == keep_ties) return;          // every key equal to the threshold is kept: no order needed
-    for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+    for (int64_t c = bx; c < chunks; c += gx) {
         if (threadIdx.x == 0) total = 0u;
         __syncthreads();
         uint32_t mine = 0;
@@ -146,9 +196,23 @@ topk_count_ties_kernel(const float* __restrict__ x, int64_t numel, TopkState* st
     }
 }
 
+__global__ void __launch_bounds__(256)
+topk_count_ties_kernel(const float* __restrict__ x, int64_t numel, TopkState* st, uint32_t* chunk_ties,
+                       int64_t chunks)
+{
+    topk_count_ties_body(x, numel, st, chunk_ties, chunks, (int)blockIdx.x, (int)gridDim.x);
+}
+
+__global__ void __launch_bounds__(256)
+topk_count_ties_batch_kernel(TopkBatch b)
+{
+    int local, width;
+    const TopkItem& it = b.item[topk_locate(b.first_c, b.count, &local, &width)];
+    topk_count_ties_body(it.x, it.numel, it.st, it.chunk_ties, it.chunks, local, width);
+}
+
 // one workgroup: exclusive prefix sum of the per-chunk tie counts, in place
-__global__ void __launch_bounds__(1024)
-topk_scan_kernel(const TopkState* st, uint32_t* chunk_ties, int64_t chunks)
+__device__ __forceinline__ void topk_scan_body(const TopkState* st, uint32_t* chunk_ties, int64_t chunks)
 {
     __shared__ uint32_t part[1024];
     if (st->ties[kPasses - 1] == st->remaining[kPasses - 1]) return;
@@ -176,10 +240,23 @@ topk_scan_kernel(const TopkState* st, uint32_t* chunk_ties, int64_t chunks)
     }
 }
 
+__global__ void __launch_bounds__(1024)
+topk_scan_kernel(const TopkState* st, uint32_t* chunk_ties, int64_t chunks)
+{
+    topk_scan_body(st, chunk_ties, chunks);
+}
+
+__global__ void __launch_bounds__(1024)
+topk_scan_batch_kernel(TopkBatch b)
+{
+    const TopkItem& it = b.item[blockIdx.x];
+    topk_scan_body(it.st, it.chunk_ties, it.chunks);
+}
+
 // keep key > threshold, keep the first `remaining` keys == threshold in index order, zero the rest
-__global__ void __launch_bounds__(256)
-topk_filter_kernel(float* __restrict__ x, int64_t numel, const TopkState* st, const uint32_t* chunk_ties,
-                   int64_t chunks)
+__device__ __forceinline__ void
+topk_filter_body(float* __restrict__ x, int64_t numel, const TopkState* st, const uint32_t* chunk_ties, int64_t chunks,
+                 int bx, int gx)
 {
     __shared__ uint32_t wave_ties[4];
     const uint32_t thr = st->prefix[kPasses - 1];
@@ -189,20 +266,20 @@ topk_filter_kernel(float* __restrict__ x, int64_t numel, const TopkState* st, co
         // no ties to break: keep every key at or above the threshold, 16-byte accesses
         const int64_t quads = numel >> 2;
         const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
-        const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+        const int64_t stride = (int64_t)gx * blockDim.x;
         if (vec) {
-            for (int64_t q = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; q < quads; q += stride) {
+            for (int64_t q = bx * (int64_t)blockDim.x + threadIdx.x; q < quads; q += stride) {
                 float4 v = reinterpret_cast<float4*>(x)[q];
                 bool k0 = mag_key(v.x) >= thr, k1 = mag_key(v.y) >= thr, k2 = mag_key(v.z) >= thr, k3 = mag_key(v.w) >= thr;
                 if (!(k0 && k1 && k2 && k3))
                     reinterpret_cast<float4*>(x)[q] = make_float4(k0 ? v.x : 0.f, k1 ? v.y : 0.f, k2 ? v.z : 0.f, k3 ? v.w : 0.f);
             }
         }
-        for (int64_t i = (vec ? quads * 4 : 0) + blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < numel; i += stride)
+        for (int64_t i = (vec ? quads * 4 : 0) + bx * (int64_t)blockDim.x + threadIdx.x; i < numel; i += stride)
             if (mag_key(x[i]) < thr) x[i] = 0.f;
         return;
     }
-    for (int64_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+    for (int64_t c = bx; c < chunks; c += gx) {
         int64_t base = c * kFilterChunk + (int64_t)threadIdx.x * 4;
         float v[4];
         uint32_t mine = 0;
@@ -238,6 +315,21 @@ topk_filter_kernel(float* __restrict__ x, int64_t numel, const TopkState* st, co
     }
 }
 
+__global__ void __launch_bounds__(256)
+topk_filter_kernel(float* __restrict__ x, int64_t numel, const TopkState* st, const uint32_t* chunk_ties,
+                   int64_t chunks)
+{
+    topk_filter_body(x, numel, st, chunk_ties, chunks, (int)blockIdx.x, (int)gridDim.x);
+}
+
+__global__ void __launch_bounds__(256)
+topk_filter_batch_kernel(TopkBatch b)
+{
+    int local, width;
+    const TopkItem& it = b.item[topk_locate(b.first_c, b.count, &local, &width)];
+    topk_filter_body(it.x, it.numel, it.st, it.chunk_ties, it.chunks, local, width);
+}
+
 inline int64_t topk_chunks(int64_t numel) { return (numel + kFilterChunk - 1) / kFilterChunk; }
 
 }  // namespace
@@ -270,6 +362,69 @@ int conef_topk_sparsify_f32(float* x, int64_t numel, int64_t k, void* workspace,
     hipLaunchKernelGGL(topk_count_ties_kernel, dim3((unsigned)cg), dim3(256), 0, s, x, numel, st, chunk_ties, chunks);
     hipLaunchKernelGGL(topk_scan_kernel, dim3(1), dim3(1024), 0, s, st, chunk_ties, chunks);
     hipLaunchKernelGGL(topk_filter_kernel, dim3((unsigned)cg), dim3(256), 0, s, x, numel, st, chunk_ties, chunks);
+    return (int)hipGetLastError();
+}
+
+// The same for `count` tensors, every pass one launch over all of them (in runs of 24): tensor i
+// is xs[i] with numels[i] elements and keeps ks[i]; tensors with ks[i] >= numels[i] are left as
+// they are.  xs / numels / ks are host arrays, read before the call returns.
+int64_t conef_topk_batch_workspace_bytes(const int64_t* numels, int32_t count)
+{
+    if (count < 0 || (count > 0 && !numels)) return -1;
+    int64_t total = 0;
+    for (int i = 0; i < count; ++i) {
+        if (numels[i] < 0) return -1;
+        total += (conef_topk_workspace_bytes(numels[i]) + 255) / 256 * 256;
+    }
+    return total > 256 ? total : 256;
+}
+
+int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const int64_t* ks, int32_t count,
+                                  void* workspace, int64_t workspace_bytes, void* stream)
+{
+    if (count < 0 || (count > 0 && (!xs || !numels || !ks))) return CONEF_ERR_INVALID;
+    for (int i = 0; i < count; ++i)
+        if (numels[i] < 1 || ks[i] < 1 || !xs[i] || numels[i] > 0xffffffffLL) return CONEF_ERR_INVALID;
+    if (count > 0 && (!workspace || workspace_bytes < conef_topk_batch_workspace_bytes(numels, count) ||
+                      (reinterpret_cast<uintptr_t>(workspace) & 15u) != 0))
+        return CONEF_ERR_INVALID;
+    hipStream_t s = (hipStream_t)stream;
+    char* ws = (char*)workspace;
+    int i = 0;
+    while (i < count) {
+        TopkBatch b;
+        int nb = 0, wh = 0, wc = 0;
+        for (; i < count && nb < kTopkBatchMax; ++i) {
+            char* mine = ws;
+            ws += (conef_topk_workspace_bytes(numels[i]) + 255) / 256 * 256;
+            if (ks[i] >= numels[i]) continue;
+            TopkItem& it = b.item[nb];
+            it.x = xs[i];
+            it.numel = numels[i];
+            it.chunks = topk_chunks(numels[i]);
+            it.st = (TopkState*)mine;
+            it.chunk_ties = (uint32_t*)(mine + sizeof(TopkState));
+            it.k = (uint32_t)ks[i];
+            int64_t g = (numels[i] + 255) / 256 / 16;
+            if (g < 1) g = 1;
+            if (g > 1024) g = 1024;
+            b.first_h[nb] = wh;
+            b.first_c[nb] = wc;
+            wh += (int)g;
+            wc += (int)(it.chunks < 4096 ? it.chunks : 4096);
+            ++nb;
+        }
+        if (nb == 0) continue;
+        b.first_h[nb] = wh;
+        b.first_c[nb] = wc;
+        b.count = nb;
+        hipLaunchKernelGGL(topk_init_batch_kernel, dim3((unsigned)nb), dim3(256), 0, s, b);
+        for (int pass = 0; pass < kPasses; ++pass)
+            hipLaunchKernelGGL(topk_hist_batch_kernel, dim3((unsigned)wh), dim3(256), 0, s, b, pass);
+        hipLaunchKernelGGL(topk_count_ties_batch_kernel, dim3((unsigned)wc), dim3(256), 0, s, b);
+        hipLaunchKernelGGL(topk_scan_batch_kernel, dim3((unsigned)nb), dim3(1024), 0, s, b);
+        hipLaunchKernelGGL(topk_filter_batch_kernel, dim3((unsigned)wc), dim3(256), 0, s, b);
+    }
     return (int)hipGetLastError();
 }
 

@@ -297,6 +297,15 @@ int64_t conef_topk_workspace_bytes(int64_t numel);
 int conef_topk_sparsify_f32(float* x, int64_t numel, int64_t k, void* workspace, int64_t workspace_bytes,
                             void* stream);
 
+/* The same for `count` tensors with every pass one launch over all of them: tensor i is xs[i] with
+ * numels[i] elements and keeps ks[i].  Replaces the `_topk(...)` call inside the per-tensor loop of
+ * hpowerSGD_hook (hPowerSGD_hook.py:554) for all matrices of a bucket at once.  xs / numels / ks
+ * are host arrays, read before the call returns; the workspace (16-byte aligned) holds
+ * conef_topk_batch_workspace_bytes(numels, count) bytes. */
+int64_t conef_topk_batch_workspace_bytes(const int64_t* numels, int32_t count);
+int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const int64_t* ks, int32_t count,
+                                  void* workspace, int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -494,6 +494,37 @@ def test_topk_exact(oracle):
         np.testing.assert_array_equal(to_np(xd), want)
 
 
+def test_topk_batch_exact(oracle):
+    """Every pass one launch over all tensors: each tensor must come out as from a call of its own
+    (ties broken by index, tensors that keep everything untouched, unaligned starts, more tensors
+    than one launch table holds)."""
+    from conef_amd._psgd_engine import topk_sparsify_all
+    gen = torch.Generator().manual_seed(5)
+    sizes = [11, 1025, 1_048_576, 100_000, 7, 4_194_304, 3, 65_537] + [300 + 17 * k for k in range(30)]
+    host = [torch.randn(n, generator=gen) for n in sizes]
+    host[3] = torch.tensor([1.0, -1.0, 1.0, 0.5, 0.0, 0.0, -1.0, 2.0] * 12_500)        # ties on the threshold
+    for ratio in (0.4, 0.01, 2.0):
+        arena = torch.zeros(sum(sizes) + 8, device="cuda")
+        dev, off = [], 0
+        for h in host:                       # back to back: most starts are not 16-byte aligned
+            dev.append(arena[off:off + h.numel()])
+            dev[-1].copy_(h)
+            off += h.numel()
+        table = topk_sparsify_all(dev, ratio)
+        for h, d in zip(host, dev):
+            want = h.numpy().copy()
+            oracle.topk_sparsify(want, ratio)
+            np.testing.assert_array_equal(to_np(d), want)
+        assert float(arena[off:].abs().max()) == 0.0
+        # the cached table serves a second round over the same tensors
+        for h, d in zip(host, dev):
+            d.copy_(h)
+        assert topk_sparsify_all(dev, ratio, table) is table
+        want = host[2].numpy().copy()
+        oracle.topk_sparsify(want, ratio)
+        np.testing.assert_array_equal(to_np(dev[2]), want)
+
+
 def test_powersgd_state_errors_and_warmup():
     from conef_amd.powerSGD_hook import PowerSGDState, _should_compress, powerSGD_hook
     with pytest.raises(ValueError, match="Expect `start_powerSGD_iter` > 1"):
