@@ -124,44 +124,63 @@ __device__ __forceinline__ void topk_resolve(TopkState* st, int p, uint32_t* pre
     __syncthreads();
 }
 
+// REP copies of every bin, copy = lane % REP, laid out [bin][copy]: the keys of a gradient crowd
+// into a few dozen bins of the first digit (one exponent and three mantissa bits), and lanes of a
+// wave that meet in a bin then add to different LDS banks instead of queueing on one address.
+template <int REP>
 __device__ __forceinline__ void
 topk_hist_body(const float* __restrict__ x, int64_t numel, TopkState* st, int pass, int bx, int gx)
 {
-    __shared__ uint32_t bins[kBins];
+    __shared__ uint32_t bins[kBins * REP];
     uint32_t prefix = 0, remaining = 0, ties = 0;
     if (pass > 0) topk_resolve(st, pass - 1, &prefix, &remaining, &ties, bx);
     const int nb = 1 << kDigitBits[pass];
-    for (int i = threadIdx.x; i < nb; i += 256) bins[i] = 0u;
+    for (int i = threadIdx.x; i < nb * REP; i += 256) bins[i] = 0u;
     __syncthreads();
     const int shift = kDigitShift[pass], hi = shift + kDigitBits[pass];
     const uint32_t mask = (uint32_t)nb - 1u;
+    const int copy = (int)(threadIdx.x & (REP - 1));
     const int64_t quads = numel >> 2;
     const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
-    int64_t stride = (int64_t)gx * blockDim.x;
+    const int64_t stride = (int64_t)gx * blockDim.x;
     if (vec) {
-        for (int64_t q = bx * (int64_t)blockDim.x + threadIdx.x; q < quads; q += stride) {
-            float4 v = reinterpret_cast<const float4*>(x)[q];
-            uint32_t key[4] = {mag_key(v.x), mag_key(v.y), mag_key(v.z), mag_key(v.w)};
+        // four 16-byte loads in flight per thread
+        for (int64_t q0 = bx * (int64_t)blockDim.x + threadIdx.x; q0 < quads; q0 += 4 * stride) {
+            float4 v[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (pass == 0 || (key[e] >> hi) == prefix) atomicAdd(&bins[(key[e] >> shift) & mask], 1u);
+            for (int u = 0; u < 4; ++u) {
+                const int64_t q = q0 + u * stride;
+                v[u] = reinterpret_cast<const float4*>(x)[q < quads ? q : q0];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (q0 + u * stride >= quads) break;
+                const uint32_t key[4] = {mag_key(v[u].x), mag_key(v[u].y), mag_key(v[u].z), mag_key(v[u].w)};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (pass == 0 || (key[e] >> hi) == prefix) atomicAdd(&bins[((key[e] >> shift) & mask) * REP + copy], 1u);
+            }
         }
     }
     for (int64_t i = (vec ? quads * 4 : 0) + bx * (int64_t)blockDim.x + threadIdx.x; i < numel; i += stride) {
         uint32_t key = mag_key(x[i]);
-        if (pass == 0 || (key >> hi) == prefix) atomicAdd(&bins[(key >> shift) & mask], 1u);
+        if (pass == 0 || (key >> hi) == prefix) atomicAdd(&bins[((key >> shift) & mask) * REP + copy], 1u);
     }
     __syncthreads();
     for (int i = threadIdx.x; i < nb; i += 256) {
-        uint32_t c = bins[i];
+        uint32_t c = 0;
+#pragma unroll
+        for (int k = 0; k < REP; ++k) c += bins[i * REP + k];
         if (c) atomicAdd(&st->hist[pass][i], c);
     }
 }
 
+// pass 0 counts every key (replicated bins), the later passes only the few that match the prefix
 __global__ void __launch_bounds__(256)
 topk_hist_kernel(const float* __restrict__ x, int64_t numel, TopkState* st, int pass)
 {
-    topk_hist_body(x, numel, st, pass, (int)blockIdx.x, (int)gridDim.x);
+    if (pass == 0) topk_hist_body<4>(x, numel, st, 0, (int)blockIdx.x, (int)gridDim.x);
+    else topk_hist_body<1>(x, numel, st, pass, (int)blockIdx.x, (int)gridDim.x);
 }
 
 __global__ void __launch_bounds__(256)
@@ -169,7 +188,8 @@ topk_hist_batch_kernel(TopkBatch b, int pass)
 {
     int local, width;
     const TopkItem& it = b.item[topk_locate(b.first_h, b.count, &local, &width)];
-    topk_hist_body(it.x, it.numel, it.st, pass, local, width);
+    if (pass == 0) topk_hist_body<4>(it.x, it.numel, it.st, 0, local, width);
+    else topk_hist_body<1>(it.x, it.numel, it.st, pass, local, width);
 }
 
 // per-chunk count of keys equal to the threshold
@@ -332,6 +352,15 @@ topk_filter_batch_kernel(TopkBatch b)
 
 inline int64_t topk_chunks(int64_t numel) { return (numel + kFilterChunk - 1) / kFilterChunk; }
 
+// Workgroups of a histogram pass: every workgroup ends with one global atomic per bin it touched,
+// all workgroups on the same few dozen counters, so fewer workgroups with longer loops (16 quads a
+// thread) beat many short ones.
+inline int64_t topk_hist_groups(int64_t numel)
+{
+    int64_t g = (numel + 255) / 256 / 64;
+    return g < 1 ? 1 : g > 512 ? 512 : g;
+}
+
 }  // namespace
 
 extern "C" {
@@ -351,9 +380,7 @@ int conef_topk_sparsify_f32(float* x, int64_t numel, int64_t k, void* workspace,
     hipStream_t s = (hipStream_t)stream;
     TopkState* st = (TopkState*)workspace;
     uint32_t* chunk_ties = (uint32_t*)((char*)workspace + sizeof(TopkState));
-    int64_t g = (numel + 255) / 256 / 16;        // four 16-byte loads per thread and pass, at least
-    if (g < 1) g = 1;
-    if (g > 1024) g = 1024;
+    const int64_t g = topk_hist_groups(numel);
     hipLaunchKernelGGL(topk_init_kernel, dim3(1), dim3(256), 0, s, st, (uint32_t)k);
     for (int pass = 0; pass < kPasses; ++pass)
         hipLaunchKernelGGL(topk_hist_kernel, dim3((unsigned)g), dim3(256), 0, s, x, numel, st, pass);
@@ -405,9 +432,7 @@ int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const
             it.st = (TopkState*)mine;
             it.chunk_ties = (uint32_t*)(mine + sizeof(TopkState));
             it.k = (uint32_t)ks[i];
-            int64_t g = (numels[i] + 255) / 256 / 16;
-            if (g < 1) g = 1;
-            if (g > 1024) g = 1024;
+            const int64_t g = topk_hist_groups(numels[i]);
             b.first_h[nb] = wh;
             b.first_c[nb] = wc;
             wh += (int)g;
