@@ -101,7 +101,9 @@ psgd_mq_body(float* __restrict__ x, const float* __restrict__ err, const float* 
 
     if (FAST) {
         const int m4 = m >> 2;
-        constexpr int UMAX = (RB * RP <= 16) ? 4 : 2;   // column quads in flight per thread, at most
+        // column quads in flight per thread, at most: registers for more of them cost more in
+        // resident waves than the extra loads in flight bring
+        constexpr int UMAX = (RB * RP <= 16) ? 2 : 1;
         // narrow matrices do not have that many quads per thread: fewer in flight rather than
         // clamped duplicates of the last quad
         auto sweep = [&](auto u_tag) {
@@ -163,8 +165,7 @@ psgd_mq_body(float* __restrict__ x, const float* __restrict__ err, const float* 
             }
         }
         };
-        if (m4 <= 256) sweep(std::integral_constant<int, 1>());
-        else if (m4 <= 512 || UMAX == 2) sweep(std::integral_constant<int, 2>());
+        if (m4 <= 256 || UMAX == 1) sweep(std::integral_constant<int, 1>());
         else sweep(std::integral_constant<int, UMAX>());
     } else {
         for (int k = threadIdx.x; k < m; k += 256) {
