@@ -23,6 +23,7 @@ A, B = 994443, 609478
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--filter", default="")
+    ap.add_argument("--hook-streams", type=int, default=2, help="side streams of the 'N streams' hook-step lines")
     ap.add_argument("--iters", type=int, default=200)
     ap.add_argument("--json", action="store_true")
     args = ap.parse_args()
@@ -302,9 +303,12 @@ def hook_steps(args, results):
         bert += [(hh, hh), (hh,)] * 4 + [(hh,), (hh,), (ff, hh), (ff,), (hh, ff), (hh,), (hh,), (hh,)]
     bert += [(hh, hh), (hh,), (hh, hh), (hh,), (hh,), (hh,), (vv,), (2, hh), (2,)]
 
-    def psgd(rank, ss):
+    ns = max(1, args.hook_streams)
+
+    def psgd(rank, ss, streams=1):
         return lambda: (PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2,
-                                      use_error_compression=True, sketch_size=ss, beta=0.9), powerSGD_hook)
+                                      use_error_compression=True, sketch_size=ss, beta=0.9, hook_streams=streams),
+                        powerSGD_hook)
 
     cases = [
         ("hook cfg1 ResNet-20, PowerSGD r=2 + sketch 50%", resnet20, psgd(2, 0.5)),
@@ -323,6 +327,12 @@ def hook_steps(args, results):
         ("hook cfg5 BERT-large, hPowerSGD r=8 + top-k error", bert,
          lambda: (hPowerSGDState(None, matrix_approximation_rank=8, start_powerSGD_iter=2, use_error_compression=True,
                                  topk_ratio=0.4), hpowerSGD_hook)),
+        # the same steps with the buckets spread over side streams (hook_streams, not in the reference)
+        ("hook cfg5 BERT-large, PowerSGD r=8 + sketch 10%%, %d streams" % ns, bert, psgd(8, 0.1, ns)),
+        ("hook cfg5 BERT-large, PowerSGD r=32 + sketch 10%%, %d streams" % ns, bert, psgd(32, 0.1, ns)),
+        ("hook cfg5 BERT-large, hPowerSGD r=8 + top-k error, %d streams" % ns, bert,
+         lambda: (hPowerSGDState(None, matrix_approximation_rank=8, start_powerSGD_iter=2, use_error_compression=True,
+                                 topk_ratio=0.4, hook_streams=ns), hpowerSGD_hook)),
     ]
     dev = torch.device("cuda", 0)
     for name, shapes, make in cases:
@@ -335,8 +345,11 @@ def hook_steps(args, results):
         grads = [torch.randn(sum(numel(s) for s in b), device=dev) * 1e-3 for b in buckets]
 
         def step():
-            for i, (b, g) in enumerate(zip(buckets, grads)):
-                hook(state, FakeGradBucket(g, b, index=i, is_last=i == len(buckets) - 1)).wait()
+            # as the reducer does: every bucket's hook as its gradients are ready, the waits at the end
+            futs = [hook(state, FakeGradBucket(g, b, index=i, is_last=i == len(buckets) - 1))
+                    for i, (b, g) in enumerate(zip(buckets, grads))]
+            for f in futs:
+                f.wait()
 
         for _ in range(3):
             step()

@@ -177,10 +177,40 @@ def _build_round(state, grads, shapes, key, error_mode):
     return plan
 
 
+_SIDE_STREAMS = {}
+
+
+def _side_stream(device, bucket_index, count):
+    """Side stream ``bucket_index % count`` of ``device`` (default priority), created on first use.
+    A bucket keeps its stream from step to step, so its state is only ever touched in order."""
+    pool = _SIDE_STREAMS.get((device, count))
+    if pool is None:
+        pool = [torch.cuda.Stream(device=device) for _ in range(count)]
+        _SIDE_STREAMS[(device, count)] = pool
+    return pool[bucket_index % count]
+
+
 def run_round(state, bucket, error_mode):
     """One hook call.  error_mode: None | 'ef' (dense, whole bucket) | 'conef' (count sketch per
     matrix) | 'conef_v2' (count sketch over the [m,n] re-view of each matrix's memory,
-    powerSGD_hook.py:918-920,1074-1076) | 'topk' (dense per matrix, magnitude-sparsified)."""
+    powerSGD_hook.py:918-920,1074-1076) | 'topk' (dense per matrix, magnitude-sparsified).
+
+    With ``state.hook_streams`` > 1 the round is enqueued on one of that many side streams: the
+    side stream first waits for the stream the hook was called on (the gradients are ready there),
+    and the returned Future carries the side stream's completion event, which is what DDP (or any
+    caller of ``wait()``) orders its own stream after."""
+    streams = int(getattr(state, "hook_streams", 1) or 1)
+    input_tensor = _bucket.buffer(bucket)
+    if streams <= 1 or not input_tensor.is_cuda or state.iter < state.start_powerSGD_iter:
+        return _run_round(state, bucket, error_mode)
+    side = _side_stream(input_tensor.device, _bucket.index(bucket), streams)
+    side.wait_stream(torch.cuda.current_stream(input_tensor.device))
+    input_tensor.record_stream(side)
+    with torch.cuda.stream(side):
+        return _run_round(state, bucket, error_mode)
+
+
+def _run_round(state, bucket, error_mode):
     group, world_size = _bucket.group_and_size(state.process_group)
     input_tensor = _bucket.buffer(bucket)
 

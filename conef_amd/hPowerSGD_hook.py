@@ -46,6 +46,7 @@ class hPowerSGDState(Checkpointable):
         "compression_stats_logging_frequency",
         "next_stats_report",
         "round_cache",
+        "hook_streams",
     ]
 
     def __init__(
@@ -61,6 +62,7 @@ class hPowerSGDState(Checkpointable):
         orthogonalization_epsilon=0,
         random_seed=0,
         compression_stats_logging_frequency=10_000,
+        hook_streams=1,
     ):
         if (use_error_feedback or warm_start) and start_powerSGD_iter <= 1:
             raise ValueError(
@@ -84,6 +86,10 @@ class hPowerSGDState(Checkpointable):
         self.compression_stats_logging_frequency = max(1, compression_stats_logging_frequency)
         self.next_stats_report = 0
         self.round_cache = {}            # per-bucket launch tables of the engine, rebuilt when a bucket changes
+        # Not in the reference: with hook_streams > 1 bucket i runs on side stream i % hook_streams
+        # of its device (the Future orders the consumer after it), so the Gram-Schmidt chains of
+        # one bucket, which keep a handful of CUs busy, overlap the streaming passes of the next.
+        self.hook_streams = hook_streams
         self.use_error_compression = use_error_compression
         self.topk_ratio = topk_ratio
 

@@ -54,6 +54,7 @@ class PowerSGDState(Checkpointable):
         "next_stats_report",
         "round_cache",
         "batched_square_dict",
+        "hook_streams",
     ]
 
     def __init__(
@@ -70,6 +71,7 @@ class PowerSGDState(Checkpointable):
         orthogonalization_epsilon=0,
         random_seed=0,
         compression_stats_logging_frequency=10_000,
+        hook_streams=1,
     ):
         logging.info(
             "PowerSGD config: matrix_approximation_rank = {}; start_powerSGD_iter = {}; "
@@ -99,6 +101,10 @@ class PowerSGDState(Checkpointable):
         self.compression_stats_logging_frequency = max(1, compression_stats_logging_frequency)
         self.next_stats_report = 0
         self.round_cache = {}            # per-bucket launch tables of the engine, rebuilt when a bucket changes
+        # Not in the reference: with hook_streams > 1 bucket i runs on side stream i % hook_streams
+        # of its device (the Future orders the consumer after it), so the Gram-Schmidt chains of
+        # one bucket, which keep a handful of CUs busy, overlap the streaming passes of the next.
+        self.hook_streams = hook_streams
         self.use_error_compression = use_error_compression
         self.beta = beta
         self.sketch_size = sketch_size

@@ -53,9 +53,11 @@ def recording(hook, calls):
     return recorded_hook
 
 
-@pytest.mark.parametrize("name", ["conef_randomblock", "ef_randomblock", "unbiased_randomblock", "conef_powersgd",
-                                  "ef_powersgd", "hefsgd_powersgd"])
-def test_hook_under_ddp(process_group, oracle, name):
+@pytest.mark.parametrize("name,streams", [("conef_randomblock", 1), ("ef_randomblock", 1), ("unbiased_randomblock", 1),
+                                          ("conef_powersgd", 1), ("ef_powersgd", 1), ("hefsgd_powersgd", 1),
+                                          # the PowerSGD rounds of a step spread over side streams
+                                          ("conef_powersgd", 3), ("hefsgd_powersgd", 2)])
+def test_hook_under_ddp(process_group, oracle, name, streams):
     from torch.nn.parallel import DistributedDataParallel as DDP
 
     from conef_amd.get_comm_hooks import make_state
@@ -63,6 +65,8 @@ def test_hook_under_ddp(process_group, oracle, name):
     # a small bucket cap so that the model spans several buckets
     ddp = DDP(copy.deepcopy(model), device_ids=[0], bucket_cap_mb=0.25)
     state, hook = make_state(Namespace(grad_reducer=name, **ARGS))
+    if streams > 1:
+        state.hook_streams = streams
     calls_log = []
     ddp.register_comm_hook(state, recording(hook, calls_log))
 

@@ -525,6 +525,46 @@ def test_topk_batch_exact(oracle):
         np.testing.assert_array_equal(to_np(dev[2]), want)
 
 
+@pytest.mark.parametrize("mode", ["conef", "ef", "topk"])
+def test_powersgd_rounds_on_side_streams(mode):
+    """hook_streams > 1: the buckets of a step run on side streams and only the Futures order the
+    caller after them.  Same kernels, same order per bucket: every result must equal the
+    single-stream run bit for bit, over several steps with the state carried along."""
+    from conef_amd.hPowerSGD_hook import hPowerSGDState, hpowerSGD_hook
+    from conef_amd.powerSGD_hook import PowerSGDState, powerSGD_hook
+    buckets = [[(1024, 256), (256,), (256, 1024)], [(640, 1440), (33, 40)], [(512, 512), (512,), (128, 2048)],
+               [(2048, 128), (300, 300)], [(96, 4096)]]
+
+    def run(streams):
+        if mode == "topk":
+            st = hPowerSGDState(None, matrix_approximation_rank=8, start_powerSGD_iter=2, use_error_compression=True,
+                                topk_ratio=0.4, hook_streams=streams)
+            hook = hpowerSGD_hook
+        else:
+            st = PowerSGDState(None, matrix_approximation_rank=8, start_powerSGD_iter=2, use_error_feedback=True,
+                               use_error_compression=mode == "conef", sketch_size=0.1, beta=0.9, hook_streams=streams)
+            hook = powerSGD_hook
+        st.iter = 2
+        outs = []
+        for step in range(4):
+            gen = torch.Generator().manual_seed(50 + step)
+            flats = [(torch.randn(numel_of(b), generator=gen) * 1e-3).cuda() for b in buckets]
+            futs = [hook(st, FakeGradBucket(f, b, index=i, is_last=i == len(buckets) - 1))
+                    for i, (f, b) in enumerate(zip(flats, buckets))]
+            outs.append([to_np(f.wait()) for f in futs])       # as the reducer does: all hooks first, then the waits
+        torch.cuda.synchronize()
+        keep = [to_np(st.p_memory_dict[i]) for i in range(len(buckets))] + [to_np(st.q_memory_dict[i]) for i in range(len(buckets))]
+        return outs, keep
+
+    one, state_one = run(1)
+    three, state_three = run(3)
+    for a, b in zip(one, three):
+        for x, y in zip(a, b):
+            np.testing.assert_array_equal(x, y)
+    for x, y in zip(state_one, state_three):
+        np.testing.assert_array_equal(x, y)
+
+
 def test_powersgd_state_errors_and_warmup():
     from conef_amd.powerSGD_hook import PowerSGDState, _should_compress, powerSGD_hook
     with pytest.raises(ValueError, match="Expect `start_powerSGD_iter` > 1"):
