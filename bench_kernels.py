@@ -344,10 +344,14 @@ def hook_steps(args, results):
         total = sum(numel(s) for s in shapes)
         grads = [torch.randn(sum(numel(s) for s in b), device=dev) * 1e-3 for b in buckets]
 
+        # bucket objects with their per-parameter views made once, as the reducer's are
+        fakes = [FakeGradBucket(g, b, index=i, is_last=i == len(buckets) - 1) for i, (b, g) in enumerate(zip(buckets, grads))]
+        for f in fakes:
+            f.gradients()
+
         def step():
             # as the reducer does: every bucket's hook as its gradients are ready, the waits at the end
-            futs = [hook(state, FakeGradBucket(g, b, index=i, is_last=i == len(buckets) - 1))
-                    for i, (b, g) in enumerate(zip(buckets, grads))]
+            futs = [hook(state, f) for f in fakes]
             for f in futs:
                 f.wait()
 

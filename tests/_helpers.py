@@ -10,17 +10,20 @@ class FakeGradBucket:
 
     def __init__(self, flat, shapes, index=0, is_last=True):
         self._flat, self._shapes, self._index, self._is_last = flat, list(shapes), index, is_last
+        self._views = None
 
     def buffer(self):
         return self._flat
 
     def gradients(self):
-        out, off = [], 0
-        for s in self._shapes:
-            c = int(np.prod(s))
-            out.append(self._flat[off:off + c].view(*s))
-            off += c
-        return out
+        if self._views is None:          # made once: the reducer's bucket hands its views over without Python work
+            out, off = [], 0
+            for s in self._shapes:
+                c = int(np.prod(s))
+                out.append(self._flat[off:off + c].view(*s))
+                off += c
+            self._views = out
+        return list(self._views)
 
     def index(self):
         return self._index
