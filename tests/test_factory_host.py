@@ -95,3 +95,10 @@ def test_hooks_register_directly():
         sig = inspect.signature(hook)
         assert sig.parameters["bucket"].annotation in (inspect._empty, dist.GradBucket), hook.__name__
         assert sig.return_annotation in (inspect._empty, torch.futures.Future[torch.Tensor]), hook.__name__
+
+
+def test_hook_streams_is_taken_from_the_namespace_when_present():
+    """Not a flag of the reference's drivers: one stream unless the namespace says otherwise."""
+    for name in ("ef_powersgd", "conef_powersgd", "hefsgd_powersgd"):
+        assert make(name)[0].hook_streams == 1
+        assert make(name, hook_streams=2)[0].hook_streams == 2
