@@ -126,17 +126,8 @@ class _RoundPlan:
     arenas.  Built on the first step of a bucket and reused while the bucket keeps its buffer
     and layout, so that a step costs a handful of foreign calls however many tensors it has."""
     __slots__ = ("key", "shapes", "work", "passthrough", "before", "after", "total_ps", "total_qs", "arena_key", "ps",
-                 "qs", "gs_p", "gs_q", "items", "count", "sketches", "fused_sketch", "batched_update", "residual_offsets",
+                 "qs", "items", "count", "sketches", "fused_sketch", "batched_update", "residual_offsets",
                  "topk_table")
-
-
-def _gs_table(matrices):
-    import ctypes
-    count = len(matrices)
-    ptrs = (ctypes.c_void_p * max(count, 1))(*[m.data_ptr() for m in matrices])
-    rows = (ctypes.c_int64 * max(count, 1))(*[m.shape[0] for m in matrices])
-    ranks = (ctypes.c_int32 * max(count, 1))(*[m.shape[1] for m in matrices])
-    return ptrs, rows, ranks, count
 
 
 def _build_round(state, grads, shapes, key, error_mode):
@@ -270,7 +261,6 @@ def _run_round(state, bucket, error_mode):
             items[cnt].p, items[cnt].q = plan.ps[-1].data_ptr(), plan.qs[-1].data_ptr()
             p_idx += n * rank
             q_idx += m * rank
-        plan.gs_p, plan.gs_q = _gs_table(plan.ps), _gs_table(plan.qs)
         plan.arena_key = (p_mem.data_ptr(), q_mem.data_ptr())
     qs = plan.qs
 
@@ -317,20 +307,11 @@ def _run_round(state, bucket, error_mode):
             host_q = [torch.randn(*q.shape, device="cpu", dtype=dtype) for q in qs]
         for q, hq in zip(qs, host_q):
             q.copy_(hq)
-    ptrs, rows, ranks, n_mats = plan.gs_q
-    _lib.check(lib.conef_gram_schmidt_batch_f32(ptrs, rows, ranks, n_mats, eps, ws_ptr, ws_len, stream),
-               "conef_gram_schmidt_batch_f32")
-
-    # pass 1: error add fused into P = M Q
     if error_mode == "conef_v2":
         # the sketch sees the same memory as m rows of n columns, so its rows are not the matrix
-        # rows: query as a pass of its own, then the plain product
+        # rows: query as a pass of its own (P = M Q then runs without a fused error add)
         for cnt, (matrix, n, m, rank) in enumerate(work):
             errs[cnt].query(matrix.view(m, n), alpha)
-    mode1 = {"ef": 1, "topk": 1, "conef": 2}.get(error_mode, 0)
-    rc = lib.conef_psgd_mq_batch_f32(items, count, mode1, float(alpha), HASH_A, HASH_B, ws_ptr, ws_len, stream)
-    _lib.check(rc, "conef_psgd_mq_batch_f32")
-
     if error_mode == "ef":
         # tensors that are not compressed: g += e, and their new error is exactly zero (:361,:558)
         for tensor in plan.passthrough:
@@ -339,13 +320,10 @@ def _run_round(state, bucket, error_mode):
             rc = lib.conef_ef_passthrough_f32(tensor.data_ptr(), dense_err.data_ptr() + 4 * off, cnt_el, stream)
             _lib.check(rc, "conef_ef_passthrough_f32")
 
-    # pass 2: orthogonalise all P side by side, then Q = M^T P
-    ptrs, rows, ranks, n_mats = plan.gs_p
-    _lib.check(lib.conef_gram_schmidt_batch_f32(ptrs, rows, ranks, n_mats, eps, ws_ptr, ws_len, stream),
-               "conef_gram_schmidt_batch_f32")
-    _lib.check(lib.conef_psgd_mtp_batch_f32(items, count, ws_ptr, ws_len, stream), "conef_psgd_mtp_batch_f32")
-
-    # pass 3: M = P Q^T with the residual fused
+    # The round itself, one foreign call: orthogonalise all Q side by side; pass 1, the error add
+    # fused into P = M Q; orthogonalise all P; pass 2, Q = M^T P; pass 3, M = P Q^T with the
+    # residual fused.
+    mode1 = {"ef": 1, "topk": 1, "conef": 2}.get(error_mode, 0)
     residual = None
     if error_mode in ("ef", "topk"):
         mode3 = 1
@@ -355,22 +333,19 @@ def _run_round(state, bucket, error_mode):
         # The residual goes out dense and the sketches are updated from it afterwards: ranks above
         # 8 (the low-rank product belongs on the matrix cores), sketches whose plan is not a row
         # list, and the re-viewed sketches of C2CS_hook_v2.
-        mode3 = 1
         residual = _scratch_f32(device, stream, max(plan.residual_offsets[-1], 1))
         for cnt in range(count):
             items[cnt].err = residual.data_ptr() + 4 * plan.residual_offsets[cnt]
+        # every sketch of the bucket from its matrix's residual in one more launch, when the plans allow
+        mode3 = 3 if error_mode == "conef" and plan.batched_update else 1
     else:
         mode3 = 0
-    rc = lib.conef_psgd_pqt_batch_f32(items, count, mode3, float(state.beta) if mode3 == 2 else 0.0, HASH_A, HASH_B,
-                                      stream)
-    _lib.check(rc, "conef_psgd_pqt_batch_f32")
+    rc = lib.conef_psgd_round_f32(items, count, mode1, mode3, float(alpha), float(state.beta) if mode3 in (2, 3) else 0.0,
+                                  eps, HASH_A, HASH_B, ws_ptr, ws_len, stream)
+    _lib.check(rc, "conef_psgd_round_f32")
     if error_mode == "topk":
         plan.topk_table = topk_sparsify_all([errs[cnt] for cnt in range(count)], state.topk_ratio, plan.topk_table)
-    elif residual is not None and error_mode == "conef" and plan.batched_update:
-        # every sketch of the bucket from its matrix's residual, in one launch
-        rc = lib.conef_psgd_sketch_update_batch_f32(items, count, float(state.beta), HASH_A, HASH_B, stream)
-        _lib.check(rc, "conef_psgd_sketch_update_batch_f32")
-    elif residual is not None:
+    elif residual is not None and mode3 != 3:
         for cnt, (matrix, n, m, rank) in enumerate(work):
             res = residual[plan.residual_offsets[cnt]: plan.residual_offsets[cnt + 1]]
             errs[cnt].update(res.view(n, m) if error_mode == "conef" else res.view(m, n), state.beta)

@@ -2465,6 +2465,45 @@ int conef_psgd_sketch_update_batch_f32(const ConefPsgdItem* items, int32_t count
     });
 }
 
+// One PowerSGD round over the matrices of a bucket in a single call (powerSGD_hook.py:473-564 at
+// world size 1): orthogonalise every Q, P = X Q with the error added first (mq_mode as in
+// conef_psgd_mq_batch_f32), orthogonalise every P, Q = X^T P, X = P Q^T with the new error
+// (pqt_mode 0, 1, 2 as in conef_psgd_pqt_batch_f32; 3 = mode 1 followed by
+// conef_psgd_sketch_update_batch_f32 on the residuals).  The same launches as the separate calls,
+// in the same order; what it saves is the caller's trips through its foreign-function interface.
+int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, float alpha,
+                         float beta, float eps, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
+                         void* stream)
+{
+    if (count < 0 || (count > 0 && !items) || pqt_mode < 0 || pqt_mode > 3) return CONEF_ERR_INVALID;
+    if (count == 0) return CONEF_OK;
+    std::vector<float*> mats((size_t)count);
+    std::vector<int64_t> rows((size_t)count);
+    std::vector<int32_t> ranks((size_t)count);
+    for (int k = 0; k < count; ++k) {
+        if (!item_ok(items[k])) return CONEF_ERR_INVALID;
+        mats[(size_t)k] = items[k].q;
+        rows[(size_t)k] = items[k].m;
+        ranks[(size_t)k] = items[k].r;
+    }
+    int rc = conef_gram_schmidt_batch_f32(mats.data(), rows.data(), ranks.data(), count, eps, workspace, workspace_bytes, stream);
+    if (rc != CONEF_OK) return rc;
+    rc = conef_psgd_mq_batch_f32(items, count, mq_mode, alpha, a, b, workspace, workspace_bytes, stream);
+    if (rc != CONEF_OK) return rc;
+    for (int k = 0; k < count; ++k) {
+        mats[(size_t)k] = items[k].p;
+        rows[(size_t)k] = items[k].n;
+    }
+    rc = conef_gram_schmidt_batch_f32(mats.data(), rows.data(), ranks.data(), count, eps, workspace, workspace_bytes, stream);
+    if (rc != CONEF_OK) return rc;
+    rc = conef_psgd_mtp_batch_f32(items, count, workspace, workspace_bytes, stream);
+    if (rc != CONEF_OK) return rc;
+    rc = conef_psgd_pqt_batch_f32(items, count, pqt_mode == 3 ? 1 : pqt_mode, pqt_mode == 2 ? beta : 0.f, a, b, stream);
+    if (rc != CONEF_OK) return rc;
+    if (pqt_mode == 3) rc = conef_psgd_sketch_update_batch_f32(items, count, beta, a, b, stream);
+    return rc;
+}
+
 // dense error feedback on the parts of a bucket that are not compressed: x += e; e = 0
 // (powerSGD_hook.py:361 and :558, where copy - result is exactly zero for untouched tensors)
 int conef_ef_passthrough_f32(float* x, float* err, int64_t count, void* stream);

@@ -282,6 +282,15 @@ int conef_psgd_pqt_batch_f32(const ConefPsgdItem* items, int32_t count, int32_t 
 int conef_psgd_sketch_update_batch_f32(const ConefPsgdItem* items, int32_t count, float beta, int32_t a, int32_t b,
                                        void* stream);
 
+/* One PowerSGD round over the matrices of a bucket in a single call: Gram-Schmidt of every Q,
+ * conef_psgd_mq_batch_f32 (mq_mode), Gram-Schmidt of every P, conef_psgd_mtp_batch_f32,
+ * conef_psgd_pqt_batch_f32 (pqt_mode 0..2; 3 = mode 1, then conef_psgd_sketch_update_batch_f32 on the
+ * residuals it wrote to err).  Replaces powerSGD_hook.py:473-564 at world size 1 (the all-reduces in
+ * between are the identity there).  Same launches as the separate calls, in the same order. */
+int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, float alpha,
+                         float beta, float eps, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
+                         void* stream);
+
 /* Dense error feedback on a stretch of the bucket that is not compressed: x += err; err = 0
  * (the copy-minus-result of powerSGD_hook.py:558 is exactly zero there). */
 int conef_ef_passthrough_f32(float* x, float* err, int64_t count, void* stream);
