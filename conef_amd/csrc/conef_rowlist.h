@@ -52,6 +52,8 @@ inline bool conef_rowlist_shape(int64_t n, int64_t d, int32_t w, bool cells, Con
 {
     if (d < 1 || d > kConefRowlistMaxCols || n < 1 || w < 1) return false;
     int64_t rb = 8192 / d;
+    // tiles to spare: half-height ones, twice as many resident per CU (a quarter was slower again)
+    if (rb >= 2 && n / rb >= 2048) rb = (rb + 1) / 2;
     if (rb > n * companions / 1024) rb = n * companions / 1024;
     if (rb > 16) rb = 16;
     if (rb < 1) rb = 1;
