@@ -9,9 +9,11 @@
 // float orders like its bit pattern) in three histogram passes of 11, 11 and 9 bits.  Choosing the
 // digit that holds the k-th largest key is not a launch of its own: every workgroup of the next
 // pass does it from the finished histogram before it starts (2048 counters, one suffix scan).
-// If more keys equal the threshold than may be kept, two counting passes and an ordered filter
-// resolve the ties in index order; otherwise those two launches return at once and the filter
-// keeps every key at or above the threshold.  Nothing returns to the host between passes.
+// The filter keeps every key at or above the threshold.  If more keys equal the threshold than may
+// be kept (and the threshold is not zero, where it makes no difference which zeros stay), one
+// workgroup of the filter launch then walks the tensor in index order and clears the ties past the
+// first `remaining` of them: exact, slow, and only ever needed for inputs with repeated
+// magnitudes right at the threshold.  Nothing returns to the host between passes.
 #include "conef_device.h"
 
 namespace {
@@ -35,15 +37,14 @@ __device__ __forceinline__ uint32_t mag_key(float v) { return __float_as_uint(v)
 
 // Several tensors per launch (the dense errors of a bucket's matrices, each with its own k and its
 // own state): the table travels by value, a workgroup finds its tensor from the running workgroup
-// count of the pass (`first_h` for the histogram passes, `first_c` for the chunked ones) and then
+// count of the pass (`first_h` for the histogram passes, `first_c` for the filter) and then
 // does what it would do in a launch of its own.
 constexpr int kTopkBatchMax = 24;
 
 struct TopkItem {
     float* x;
-    int64_t numel, chunks;
+    int64_t numel;
     TopkState* st;
-    uint32_t* chunk_ties;
     uint32_t k;
 };
 
@@ -192,123 +193,29 @@ topk_hist_batch_kernel(TopkBatch b, int pass)
     else topk_hist_body<1>(it.x, it.numel, it.st, pass, local, width);
 }
 
-// per-chunk count of keys equal to the threshold
-__device__ __forceinline__ void
-topk_count_ties_body(const float* __restrict__ x, int64_t numel, TopkState* st, uint32_t* chunk_ties, int64_t chunks,
-                     int bx, int gx)
-{
-    __shared__ uint32_t total;
-    uint32_t thr, keep_ties, ties;
-    topk_resolve(st, kPasses - 1, &thr, &keep_ties, &ties, bx);
-    if (ties == keep_ties) return;          // every key equal to the threshold is kept: no order needed
-    for (int64_t c = bx; c < chunks; c += gx) {
-        if (threadIdx.x == 0) total = 0u;
-        __syncthreads();
-        uint32_t mine = 0;
-        int64_t base = c * kFilterChunk + (int64_t)threadIdx.x * 4;
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-            if (base + k < numel && mag_key(x[base + k]) == thr) ++mine;
-        if (mine) atomicAdd(&total, mine);
-        __syncthreads();
-        if (threadIdx.x == 0) chunk_ties[c] = total;
-        __syncthreads();
-    }
-}
-
-__global__ void __launch_bounds__(256)
-topk_count_ties_kernel(const float* __restrict__ x, int64_t numel, TopkState* st, uint32_t* chunk_ties,
-                       int64_t chunks)
-{
-    topk_count_ties_body(x, numel, st, chunk_ties, chunks, (int)blockIdx.x, (int)gridDim.x);
-}
-
-__global__ void __launch_bounds__(256)
-topk_count_ties_batch_kernel(TopkBatch b)
-{
-    int local, width;
-    const TopkItem& it = b.item[topk_locate(b.first_c, b.count, &local, &width)];
-    topk_count_ties_body(it.x, it.numel, it.st, it.chunk_ties, it.chunks, local, width);
-}
-
-// one workgroup: exclusive prefix sum of the per-chunk tie counts, in place
-__device__ __forceinline__ void topk_scan_body(const TopkState* st, uint32_t* chunk_ties, int64_t chunks)
-{
-    __shared__ uint32_t part[1024];
-    if (st->ties[kPasses - 1] == st->remaining[kPasses - 1]) return;
-    int64_t per = (chunks + 1023) / 1024;
-    int64_t lo = (int64_t)threadIdx.x * per;
-    int64_t hi = lo + per < chunks ? lo + per : chunks;
-    uint32_t s = 0;
-    for (int64_t i = lo; i < hi; ++i) s += chunk_ties[i];
-    part[threadIdx.x] = s;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t run = 0;
-        for (int t = 0; t < 1024; ++t) {
-            uint32_t v = part[t];
-            part[t] = run;
-            run += v;
-        }
-    }
-    __syncthreads();
-    uint32_t run = part[threadIdx.x];
-    for (int64_t i = lo; i < hi; ++i) {
-        uint32_t v = chunk_ties[i];
-        chunk_ties[i] = run;
-        run += v;
-    }
-}
-
-__global__ void __launch_bounds__(1024)
-topk_scan_kernel(const TopkState* st, uint32_t* chunk_ties, int64_t chunks)
-{
-    topk_scan_body(st, chunk_ties, chunks);
-}
-
-__global__ void __launch_bounds__(1024)
-topk_scan_batch_kernel(TopkBatch b)
-{
-    const TopkItem& it = b.item[blockIdx.x];
-    topk_scan_body(it.st, it.chunk_ties, it.chunks);
-}
-
-// keep key > threshold, keep the first `remaining` keys == threshold in index order, zero the rest
-__device__ __forceinline__ void
-topk_filter_body(float* __restrict__ x, int64_t numel, const TopkState* st, const uint32_t* chunk_ties, int64_t chunks,
-                 int bx, int gx)
+// keys equal to the threshold, in index order: the first `keep_ties` stay, the rest are cleared.
+// One workgroup of 256 threads, 1024 elements a round; once the quota is used up the rounds need
+// no scan any more.
+__device__ __forceinline__ void topk_order_ties(float* __restrict__ x, int64_t numel, uint32_t thr, uint32_t keep_ties)
 {
     __shared__ uint32_t wave_ties[4];
-    const uint32_t thr = st->prefix[kPasses - 1];
-    const uint32_t keep_ties = st->remaining[kPasses - 1];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    if (st->ties[kPasses - 1] == keep_ties) {
-        // no ties to break: keep every key at or above the threshold, 16-byte accesses
-        const int64_t quads = numel >> 2;
-        const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
-        const int64_t stride = (int64_t)gx * blockDim.x;
-        if (vec) {
-            for (int64_t q = bx * (int64_t)blockDim.x + threadIdx.x; q < quads; q += stride) {
-                float4 v = reinterpret_cast<float4*>(x)[q];
-                bool k0 = mag_key(v.x) >= thr, k1 = mag_key(v.y) >= thr, k2 = mag_key(v.z) >= thr, k3 = mag_key(v.w) >= thr;
-                if (!(k0 && k1 && k2 && k3))
-                    reinterpret_cast<float4*>(x)[q] = make_float4(k0 ? v.x : 0.f, k1 ? v.y : 0.f, k2 ? v.z : 0.f, k3 ? v.w : 0.f);
-            }
-        }
-        for (int64_t i = (vec ? quads * 4 : 0) + bx * (int64_t)blockDim.x + threadIdx.x; i < numel; i += stride)
-            if (mag_key(x[i]) < thr) x[i] = 0.f;
-        return;
-    }
-    for (int64_t c = bx; c < chunks; c += gx) {
-        int64_t base = c * kFilterChunk + (int64_t)threadIdx.x * 4;
-        float v[4];
+    uint32_t running = 0;                       // ties seen in earlier rounds: the same in every thread
+    for (int64_t base0 = 0; base0 < numel; base0 += kFilterChunk) {
+        const int64_t base = base0 + (int64_t)threadIdx.x * 4;
+        bool tie[4];
         uint32_t mine = 0;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            v[k] = base + k < numel ? x[base + k] : 0.f;
-            if (base + k < numel && mag_key(v[k]) == thr) ++mine;
+            tie[k] = base + k < numel && mag_key(x[base + k]) == thr;
+            mine += tie[k];
         }
-        // exclusive rank of this thread's first tie inside the chunk: scan over lanes, then waves
+        if (running >= keep_ties) {             // uniform: nothing more may stay
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (tie[k]) x[base + k] = 0.f;
+            continue;
+        }
         uint32_t incl = mine;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
@@ -317,29 +224,48 @@ topk_filter_body(float* __restrict__ x, int64_t numel, const TopkState* st, cons
         }
         if (lane == 63) wave_ties[wave] = incl;
         __syncthreads();
-        uint32_t rank = chunk_ties[c] + incl - mine;
+        uint32_t rank = running + incl - mine;
         for (int wv = 0; wv < wave; ++wv) rank += wave_ties[wv];
+        const uint32_t total = (wave_ties[0] + wave_ties[1]) + (wave_ties[2] + wave_ties[3]);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            if (base + k < numel) {
-                uint32_t key = mag_key(v[k]);
-                bool keep = key > thr;
-                if (key == thr) {
-                    keep = rank < keep_ties;
-                    ++rank;
-                }
-                if (!keep) x[base + k] = 0.f;
+        for (int k = 0; k < 4; ++k)
+            if (tie[k]) {
+                if (rank >= keep_ties) x[base + k] = 0.f;
+                ++rank;
             }
-        }
+        running += total;
         __syncthreads();
     }
 }
 
-__global__ void __launch_bounds__(256)
-topk_filter_kernel(float* __restrict__ x, int64_t numel, const TopkState* st, const uint32_t* chunk_ties,
-                   int64_t chunks)
+// keep key >= threshold, zero the rest; workgroup 0 of the tensor then settles surplus ties
+__device__ __forceinline__ void
+topk_filter_body(float* __restrict__ x, int64_t numel, TopkState* st, int bx, int gx)
 {
-    topk_filter_body(x, numel, st, chunk_ties, chunks, (int)blockIdx.x, (int)gridDim.x);
+    uint32_t thr, keep_ties, ties;
+    topk_resolve(st, kPasses - 1, &thr, &keep_ties, &ties, bx);
+    const int64_t quads = numel >> 2;
+    const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+    const int64_t stride = (int64_t)gx * blockDim.x;
+    if (vec) {
+        for (int64_t q = bx * (int64_t)blockDim.x + threadIdx.x; q < quads; q += stride) {
+            float4 v = reinterpret_cast<float4*>(x)[q];
+            bool k0 = mag_key(v.x) >= thr, k1 = mag_key(v.y) >= thr, k2 = mag_key(v.z) >= thr, k3 = mag_key(v.w) >= thr;
+            if (!(k0 && k1 && k2 && k3))
+                reinterpret_cast<float4*>(x)[q] = make_float4(k0 ? v.x : 0.f, k1 ? v.y : 0.f, k2 ? v.z : 0.f, k3 ? v.w : 0.f);
+        }
+    }
+    for (int64_t i = (vec ? quads * 4 : 0) + bx * (int64_t)blockDim.x + threadIdx.x; i < numel; i += stride)
+        if (mag_key(x[i]) < thr) x[i] = 0.f;
+    // The pass above never touches a key equal to the threshold, so the tie walk may run beside
+    // the other workgroups' share of it.  A zero threshold has only zeros for ties.
+    if (bx == 0 && ties != keep_ties && thr != 0u) topk_order_ties(x, numel, thr, keep_ties);
+}
+
+__global__ void __launch_bounds__(256)
+topk_filter_kernel(float* __restrict__ x, int64_t numel, TopkState* st)
+{
+    topk_filter_body(x, numel, st, (int)blockIdx.x, (int)gridDim.x);
 }
 
 __global__ void __launch_bounds__(256)
@@ -347,7 +273,7 @@ topk_filter_batch_kernel(TopkBatch b)
 {
     int local, width;
     const TopkItem& it = b.item[topk_locate(b.first_c, b.count, &local, &width)];
-    topk_filter_body(it.x, it.numel, it.st, it.chunk_ties, it.chunks, local, width);
+    topk_filter_body(it.x, it.numel, it.st, local, width);
 }
 
 inline int64_t topk_chunks(int64_t numel) { return (numel + kFilterChunk - 1) / kFilterChunk; }
@@ -368,7 +294,7 @@ extern "C" {
 int64_t conef_topk_workspace_bytes(int64_t numel)
 {
     if (numel < 0) return -1;
-    return (int64_t)sizeof(TopkState) + (int64_t)sizeof(uint32_t) * (topk_chunks(numel) + 1);
+    return ((int64_t)sizeof(TopkState) + 255) / 256 * 256;      // the selection state; nothing grows with numel
 }
 
 int conef_topk_sparsify_f32(float* x, int64_t numel, int64_t k, void* workspace, int64_t workspace_bytes,
@@ -379,16 +305,13 @@ int conef_topk_sparsify_f32(float* x, int64_t numel, int64_t k, void* workspace,
     if (!workspace || workspace_bytes < conef_topk_workspace_bytes(numel)) return CONEF_ERR_INVALID;
     hipStream_t s = (hipStream_t)stream;
     TopkState* st = (TopkState*)workspace;
-    uint32_t* chunk_ties = (uint32_t*)((char*)workspace + sizeof(TopkState));
     const int64_t g = topk_hist_groups(numel);
     hipLaunchKernelGGL(topk_init_kernel, dim3(1), dim3(256), 0, s, st, (uint32_t)k);
     for (int pass = 0; pass < kPasses; ++pass)
         hipLaunchKernelGGL(topk_hist_kernel, dim3((unsigned)g), dim3(256), 0, s, x, numel, st, pass);
     int64_t chunks = topk_chunks(numel);
     int64_t cg = chunks < 4096 ? chunks : 4096;
-    hipLaunchKernelGGL(topk_count_ties_kernel, dim3((unsigned)cg), dim3(256), 0, s, x, numel, st, chunk_ties, chunks);
-    hipLaunchKernelGGL(topk_scan_kernel, dim3(1), dim3(1024), 0, s, st, chunk_ties, chunks);
-    hipLaunchKernelGGL(topk_filter_kernel, dim3((unsigned)cg), dim3(256), 0, s, x, numel, st, chunk_ties, chunks);
+    hipLaunchKernelGGL(topk_filter_kernel, dim3((unsigned)cg), dim3(256), 0, s, x, numel, st);
     return (int)hipGetLastError();
 }
 
@@ -428,15 +351,14 @@ int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const
             TopkItem& it = b.item[nb];
             it.x = xs[i];
             it.numel = numels[i];
-            it.chunks = topk_chunks(numels[i]);
             it.st = (TopkState*)mine;
-            it.chunk_ties = (uint32_t*)(mine + sizeof(TopkState));
             it.k = (uint32_t)ks[i];
+            const int64_t chunks = topk_chunks(numels[i]);
             const int64_t g = topk_hist_groups(numels[i]);
             b.first_h[nb] = wh;
             b.first_c[nb] = wc;
             wh += (int)g;
-            wc += (int)(it.chunks < 4096 ? it.chunks : 4096);
+            wc += (int)(chunks < 4096 ? chunks : 4096);
             ++nb;
         }
         if (nb == 0) continue;
@@ -446,8 +368,6 @@ int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const
         hipLaunchKernelGGL(topk_init_batch_kernel, dim3((unsigned)nb), dim3(256), 0, s, b);
         for (int pass = 0; pass < kPasses; ++pass)
             hipLaunchKernelGGL(topk_hist_batch_kernel, dim3((unsigned)wh), dim3(256), 0, s, b, pass);
-        hipLaunchKernelGGL(topk_count_ties_batch_kernel, dim3((unsigned)wc), dim3(256), 0, s, b);
-        hipLaunchKernelGGL(topk_scan_batch_kernel, dim3((unsigned)nb), dim3(1024), 0, s, b);
         hipLaunchKernelGGL(topk_filter_batch_kernel, dim3((unsigned)wc), dim3(256), 0, s, b);
     }
     return (int)hipGetLastError();
