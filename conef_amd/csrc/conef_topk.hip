@@ -10,10 +10,12 @@
 // digit that holds the k-th largest key is not a launch of its own: every workgroup of the next
 // pass does it from the finished histogram before it starts (2048 counters, one suffix scan).
 // The filter keeps every key at or above the threshold.  If more keys equal the threshold than may
-// be kept (and the threshold is not zero, where it makes no difference which zeros stay), one
-// workgroup of the filter launch then walks the tensor in index order and clears the ties past the
-// first `remaining` of them: exact, slow, and only ever needed for inputs with repeated
-// magnitudes right at the threshold.  Nothing returns to the host between passes.
+// be kept (two equal magnitudes at the threshold turn up in a few percent of million-element
+// gradients; at a zero threshold it makes no difference which zeros stay), the filter's workgroups
+// also note where those keys sit, and the workgroup that finishes last ranks the noted indices
+// and clears the ties past the first `remaining` of them.  More than 1024 such ties (a tensor of
+// repeated values) are settled by one workgroup walking the tensor in index order instead: exact,
+// slow, and of no practical concern.  Nothing returns to the host between passes.
 #include "conef_device.h"
 
 namespace {
@@ -22,22 +24,26 @@ constexpr int kPasses = 3;
 constexpr int kDigitBits[kPasses] = {11, 11, 9};
 constexpr int kDigitShift[kPasses] = {20, 9, 0};
 constexpr int kBins = 2048;          // bins of the widest digit
-constexpr int kFilterChunk = 1024;   // elements per workgroup iteration in the ordered passes
+constexpr int kFilterChunk = 1024;   // elements per workgroup iteration in the ordered walk
+constexpr int kTieMax = 1024;        // surplus ties up to this many are ranked from a list, more by a walk
 
 struct TopkState {
     uint32_t k;
     uint32_t prefix[kPasses];       // prefix[p]: selected digits of passes 0..p, written by pass p + 1
     uint32_t remaining[kPasses];    // how many keys to take among those matching prefix[p]
     uint32_t ties[kPasses];         // keys that match prefix[p] exactly in their high digits
-    uint32_t pad[6];
+    uint32_t done;                  // workgroups of the filter that have finished (surplus ties only)
+    uint32_t tie_count;             // indices recorded in tie_idx so far
+    uint32_t pad[4];
     uint32_t hist[kPasses][kBins];
+    uint32_t tie_idx[kTieMax];      // where the keys equal to the threshold sit, in no order
 };
 
 __device__ __forceinline__ uint32_t mag_key(float v) { return __float_as_uint(v) & 0x7fffffffu; }
 
 // Several tensors per launch (the dense errors of a bucket's matrices, each with its own k and its
 // own state): the table travels by value, a workgroup finds its tensor from the running workgroup
-// count of the pass (`first_h` for the histogram passes, `first_c` for the filter) and then
+// count (`first`, the same for every pass) and then
 // does what it would do in a launch of its own.
 constexpr int kTopkBatchMax = 24;
 
@@ -50,8 +56,7 @@ struct TopkItem {
 
 struct TopkBatch {
     TopkItem item[kTopkBatchMax];
-    int first_h[kTopkBatchMax + 1];
-    int first_c[kTopkBatchMax + 1];
+    int first[kTopkBatchMax + 1];
     int count;
 };
 
@@ -67,7 +72,11 @@ __device__ __forceinline__ int topk_locate(const int* first, int count, int* loc
 __device__ __forceinline__ void topk_init_body(TopkState* st, uint32_t k)
 {
     for (int i = threadIdx.x; i < kPasses * kBins; i += blockDim.x) (&st->hist[0][0])[i] = 0u;
-    if (threadIdx.x == 0) st->k = k;
+    if (threadIdx.x == 0) {
+        st->k = k;
+        st->done = 0u;
+        st->tie_count = 0u;
+    }
 }
 
 __global__ void topk_init_kernel(TopkState* st, uint32_t k) { topk_init_body(st, k); }
@@ -188,7 +197,7 @@ __global__ void __launch_bounds__(256)
 topk_hist_batch_kernel(TopkBatch b, int pass)
 {
     int local, width;
-    const TopkItem& it = b.item[topk_locate(b.first_h, b.count, &local, &width)];
+    const TopkItem& it = b.item[topk_locate(b.first, b.count, &local, &width)];
     if (pass == 0) topk_hist_body<4>(it.x, it.numel, it.st, 0, local, width);
     else topk_hist_body<1>(it.x, it.numel, it.st, pass, local, width);
 }
@@ -238,28 +247,66 @@ __device__ __forceinline__ void topk_order_ties(float* __restrict__ x, int64_t n
     }
 }
 
-// keep key >= threshold, zero the rest; workgroup 0 of the tensor then settles surplus ties
+// keep key >= threshold, zero the rest, settle surplus ties on the threshold by index
 __device__ __forceinline__ void
 topk_filter_body(float* __restrict__ x, int64_t numel, TopkState* st, int bx, int gx)
 {
+    __shared__ uint32_t ticket;
+    __shared__ uint32_t idx_l[kTieMax];
     uint32_t thr, keep_ties, ties;
     topk_resolve(st, kPasses - 1, &thr, &keep_ties, &ties, bx);
+    const bool surplus = ties != keep_ties && thr != 0u;      // a zero threshold has only zeros for ties
+    const bool listed = surplus && ties <= (uint32_t)kTieMax;
+    auto note = [&](int64_t i) {
+        const uint32_t slot = atomicAdd(&st->tie_count, 1u);
+        if (slot < (uint32_t)kTieMax) st->tie_idx[slot] = (uint32_t)i;
+    };
     const int64_t quads = numel >> 2;
     const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
     const int64_t stride = (int64_t)gx * blockDim.x;
     if (vec) {
         for (int64_t q = bx * (int64_t)blockDim.x + threadIdx.x; q < quads; q += stride) {
             float4 v = reinterpret_cast<float4*>(x)[q];
-            bool k0 = mag_key(v.x) >= thr, k1 = mag_key(v.y) >= thr, k2 = mag_key(v.z) >= thr, k3 = mag_key(v.w) >= thr;
+            const uint32_t key[4] = {mag_key(v.x), mag_key(v.y), mag_key(v.z), mag_key(v.w)};
+            bool k0 = key[0] >= thr, k1 = key[1] >= thr, k2 = key[2] >= thr, k3 = key[3] >= thr;
             if (!(k0 && k1 && k2 && k3))
                 reinterpret_cast<float4*>(x)[q] = make_float4(k0 ? v.x : 0.f, k1 ? v.y : 0.f, k2 ? v.z : 0.f, k3 ? v.w : 0.f);
+            if (listed) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (key[e] == thr) note(4 * q + e);
+            }
         }
     }
-    for (int64_t i = (vec ? quads * 4 : 0) + bx * (int64_t)blockDim.x + threadIdx.x; i < numel; i += stride)
-        if (mag_key(x[i]) < thr) x[i] = 0.f;
-    // The pass above never touches a key equal to the threshold, so the tie walk may run beside
-    // the other workgroups' share of it.  A zero threshold has only zeros for ties.
-    if (bx == 0 && ties != keep_ties && thr != 0u) topk_order_ties(x, numel, thr, keep_ties);
+    for (int64_t i = (vec ? quads * 4 : 0) + bx * (int64_t)blockDim.x + threadIdx.x; i < numel; i += stride) {
+        const uint32_t key = mag_key(x[i]);
+        if (key < thr) x[i] = 0.f;
+        else if (listed && key == thr) note(i);
+    }
+    if (!surplus) return;
+    if (!listed) {
+        // the pass above never touches a key equal to the threshold, so the walk may run beside
+        // the other workgroups' share of it
+        if (bx == 0) topk_order_ties(x, numel, thr, keep_ties);
+        return;
+    }
+    // the workgroup that finishes last sees every noted index
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) ticket = atomicAdd(&st->done, 1u);
+    __syncthreads();
+    if (ticket != (uint32_t)gx - 1u) return;
+    __threadfence();
+    const int n = (int)ties;
+    for (int j = threadIdx.x; j < n; j += blockDim.x)
+        idx_l[j] = __hip_atomic_load(&st->tie_idx[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    for (int j = threadIdx.x; j < n; j += blockDim.x) {
+        const uint32_t mine = idx_l[j];
+        uint32_t rank = 0;
+        for (int t = 0; t < n; ++t) rank += idx_l[t] < mine;
+        if (rank >= keep_ties) x[mine] = 0.f;
+    }
 }
 
 __global__ void __launch_bounds__(256)
@@ -272,14 +319,14 @@ __global__ void __launch_bounds__(256)
 topk_filter_batch_kernel(TopkBatch b)
 {
     int local, width;
-    const TopkItem& it = b.item[topk_locate(b.first_c, b.count, &local, &width)];
+    const TopkItem& it = b.item[topk_locate(b.first, b.count, &local, &width)];
     topk_filter_body(it.x, it.numel, it.st, local, width);
 }
 
-inline int64_t topk_chunks(int64_t numel) { return (numel + kFilterChunk - 1) / kFilterChunk; }
 
-// Workgroups of a histogram pass: every workgroup ends with one global atomic per bin it touched,
-// all workgroups on the same few dozen counters, so fewer workgroups with longer loops (16 quads a
+// Workgroups of a pass over a tensor.  A histogram workgroup ends with one global atomic per bin
+// it touched, all workgroups on the same few dozen counters, and a filter workgroup that has to
+// settle ties ends with one on a single counter: fewer workgroups with longer loops (16 quads a
 // thread) beat many short ones.
 inline int64_t topk_hist_groups(int64_t numel)
 {
@@ -309,9 +356,7 @@ int conef_topk_sparsify_f32(float* x, int64_t numel, int64_t k, void* workspace,
     hipLaunchKernelGGL(topk_init_kernel, dim3(1), dim3(256), 0, s, st, (uint32_t)k);
     for (int pass = 0; pass < kPasses; ++pass)
         hipLaunchKernelGGL(topk_hist_kernel, dim3((unsigned)g), dim3(256), 0, s, x, numel, st, pass);
-    int64_t chunks = topk_chunks(numel);
-    int64_t cg = chunks < 4096 ? chunks : 4096;
-    hipLaunchKernelGGL(topk_filter_kernel, dim3((unsigned)cg), dim3(256), 0, s, x, numel, st);
+    hipLaunchKernelGGL(topk_filter_kernel, dim3((unsigned)g), dim3(256), 0, s, x, numel, st);
     return (int)hipGetLastError();
 }
 
@@ -343,7 +388,7 @@ int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const
     int i = 0;
     while (i < count) {
         TopkBatch b;
-        int nb = 0, wh = 0, wc = 0;
+        int nb = 0, wgs = 0;
         for (; i < count && nb < kTopkBatchMax; ++i) {
             char* mine = ws;
             ws += (conef_topk_workspace_bytes(numels[i]) + 255) / 256 * 256;
@@ -353,22 +398,17 @@ int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const
             it.numel = numels[i];
             it.st = (TopkState*)mine;
             it.k = (uint32_t)ks[i];
-            const int64_t chunks = topk_chunks(numels[i]);
-            const int64_t g = topk_hist_groups(numels[i]);
-            b.first_h[nb] = wh;
-            b.first_c[nb] = wc;
-            wh += (int)g;
-            wc += (int)(chunks < 4096 ? chunks : 4096);
+            b.first[nb] = wgs;
+            wgs += (int)topk_hist_groups(numels[i]);
             ++nb;
         }
         if (nb == 0) continue;
-        b.first_h[nb] = wh;
-        b.first_c[nb] = wc;
+        b.first[nb] = wgs;
         b.count = nb;
         hipLaunchKernelGGL(topk_init_batch_kernel, dim3((unsigned)nb), dim3(256), 0, s, b);
         for (int pass = 0; pass < kPasses; ++pass)
-            hipLaunchKernelGGL(topk_hist_batch_kernel, dim3((unsigned)wh), dim3(256), 0, s, b, pass);
-        hipLaunchKernelGGL(topk_filter_batch_kernel, dim3((unsigned)wc), dim3(256), 0, s, b);
+            hipLaunchKernelGGL(topk_hist_batch_kernel, dim3((unsigned)wgs), dim3(256), 0, s, b, pass);
+        hipLaunchKernelGGL(topk_filter_batch_kernel, dim3((unsigned)wgs), dim3(256), 0, s, b);
     }
     return (int)hipGetLastError();
 }

@@ -484,6 +484,24 @@ def test_topk_exact(oracle):
         xd = x.cuda()
         _topk(xd, ratio)
         np.testing.assert_array_equal(to_np(xd), want)
+    # a few equal magnitudes right at the threshold of a large tensor (what real gradients show in a few
+    # percent of million-element matrices): the lowest indices among them stay
+    g = torch.Generator().manual_seed(11)
+    for numel, ratio, copies in [(1_000_003, 0.4, 5), (262_144, 0.1, 40), (50_000, 0.4, 1500)]:
+        x = torch.randn(numel, generator=g)
+        k = max(1, int(0.5 * ratio * numel))
+        kth = torch.topk(x.abs(), k).values[-1]
+        where = torch.randperm(numel, generator=g)[:copies]
+        sign = torch.where(torch.rand(copies, generator=g) < 0.5, -1.0, 1.0)
+        x[where] = kth * sign                      # now more keys equal the threshold than may be kept
+        want = x.numpy().copy()
+        oracle.topk_sparsify(want, ratio)
+        assert np.count_nonzero(want) == k
+        for off in (0, 1):
+            xd = torch.zeros(numel + off, device="cuda")[off:]
+            xd.copy_(x)
+            _topk(xd, ratio)
+            np.testing.assert_array_equal(to_np(xd), want)
     # ties, zeros and a threshold of zero
     x = torch.tensor([1.0, -1.0, 1.0, 0.5, 0.0, 0.0, -1.0, 2.0] * 300)
     for ratio in (0.25, 0.5, 1.0, 1.9):
