@@ -284,19 +284,19 @@ topk_filter_body(float* __restrict__ x, int64_t numel, TopkState* st, int bx, in
         else if (listed && key == thr) note(i);
     }
     if (!surplus) return;
-    if (!listed) {
-        // the pass above never touches a key equal to the threshold, so the walk may run beside
-        // the other workgroups' share of it
-        if (bx == 0) topk_order_ties(x, numel, thr, keep_ties);
-        return;
-    }
-    // the workgroup that finishes last sees every noted index
+    // The workgroup that finishes last sees every noted index, and nobody else's 16-byte stores
+    // (which rewrite a tie with its own value when a neighbour in the quad goes) can land after
+    // the zeros it writes.
     __threadfence();
     __syncthreads();
     if (threadIdx.x == 0) ticket = atomicAdd(&st->done, 1u);
     __syncthreads();
     if (ticket != (uint32_t)gx - 1u) return;
     __threadfence();
+    if (!listed) {
+        topk_order_ties(x, numel, thr, keep_ties);
+        return;
+    }
     const int n = (int)ties;
     for (int j = threadIdx.x; j < n; j += blockDim.x)
         idx_l[j] = __hip_atomic_load(&st->tie_idx[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
