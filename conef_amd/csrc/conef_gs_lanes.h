@@ -66,8 +66,8 @@ __device__ __forceinline__ float gsl_column_sum(float x)
 
 // Workgroup b of a matrix owns elements [1024 RPT b, 1024 RPT (b + 1)).  The launch must be
 // cooperative (all workgroups resident) and ws reset for its workgroups.  A workgroup that waits
-// about a second for another one's record gives up, tells the others, and the kernel ends with
-// the matrix unfinished.
+// about a second for another one's record gives up, tells the others, and every workgroup that
+// hears of it fills its share of the matrix with NaN before it ends.
 template <int RP, int RPT>
 __global__ void __launch_bounds__(kGslThreads)
 gsl_kernel(GslBatch batch, int count, float eps, GslWs* ws)
@@ -150,7 +150,15 @@ gsl_kernel(GslBatch batch, int count, float eps, GslWs* ws)
             part[c2 * kGslMaxWgs + g2] = __uint_as_float((unsigned)rec);
         }
         __syncthreads();
-        if (failed) return;
+        if (failed) {
+            // a half-orthogonalised matrix would pass for a result: leave one that cannot
+#pragma unroll
+            for (int t = 0; t < RPT; ++t) {
+                const int e = tid + T * t;
+                if (e < mine) a[e] = __builtin_nanf("");
+            }
+            return;
+        }
         if (tid < RP) {
             float s = 0.f;
             for (int g2 = 0; g2 < nwg; ++g2) s += part[tid * kGslMaxWgs + g2];      // same order in every workgroup

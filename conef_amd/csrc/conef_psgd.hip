@@ -1066,6 +1066,13 @@ gram_schmidt_grid_kernel(float* __restrict__ a, int64_t rows, int r, float eps, 
         }
     }
     gs_grid_steps<RP, RPT, 0>(v, red, part, tot_l, ws, r, nrt, eps, wave, lane);
+    if (tot_l[RP] == 0.f) {
+        // a wait ran out: a half-orthogonalised matrix would pass for a result, NaN cannot
+#pragma unroll
+        for (int t = 0; t < RPT; ++t)
+#pragma unroll
+            for (int c = 0; c < RP; ++c) v[t][c] = __builtin_nanf("");
+    }
 #pragma unroll
     for (int t = 0; t < RPT; ++t) {
         const int k = threadIdx.x + t * kGsRegThreads;

@@ -188,7 +188,10 @@ int conef_randblock_scatter_f32(float* x, const float* payload, int64_t numel, i
 
 /* In-place Gram-Schmidt of a row-major [rows, r] matrix: column by column, col /= ||col|| (+ eps
  * if eps != 0), then every later column loses its projection on col.
- * Replaces: _orthogonalize, powerSGD_hook.py:12-44 (about 4r torch kernels per matrix). */
+ * Replaces: _orthogonalize, powerSGD_hook.py:12-44 (about 4r torch kernels per matrix).
+ * Matrices spread over several workgroups exchange their sums through device memory inside one
+ * cooperative launch; should a workgroup ever wait about a second for another, the kernel ends
+ * and leaves NaN in the matrix instead of a half-orthogonalised one. */
 int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* workspace, int64_t workspace_bytes,
                            void* stream);
 
