@@ -30,8 +30,11 @@ __global__ void hash_table_kernel(int32_t* bucket, int32_t* sign, int64_t d, Con
 
 // ----------------------------------------------------------------- query ----
 // x[r,i] += (sign_i * cs[r,h_i]) * alpha.  Thread = 4 consecutive columns, loop over a group of
-// rows so the two hashes per column are paid once per row group.
-template <typename CsT, bool VEC>
+// rows so the two hashes per column are paid once per row group.  The rows are taken RB at a time
+// with every load of the batch (values and gathered cells) issued before the first is used: a
+// thread's stores and later loads retire through one in-order counter, so row-at-a-time code pays
+// a full memory round trip per row.
+template <typename CsT, bool VEC, int RB>
 __global__ void __launch_bounds__(256)
 cs_query_kernel(float* __restrict__ x, const CsT* __restrict__ cs, int64_t n, int64_t d, ConefMod mod,
                 float alpha, ConefSeeds hs, int rows_per_block)
@@ -44,17 +47,34 @@ cs_query_kernel(float* __restrict__ x, const CsT* __restrict__ cs, int64_t n, in
         pk[k] = (c0 + k < d) ? conef_bucket_sign((int32_t)(c0 + k), mod, hs.a, hs.b, hs.sa, hs.sb) : 0u;
     int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
     int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
-    for (int64_t r = r0; r < r1; ++r) {
-        const CsT* row = cs + r * (int64_t)mod.w;
-        float* xr = x + r * d + c0;
-        if (VEC) {
-            float4 v = *reinterpret_cast<const float4*>(xr);
-            v.x = __fadd_rn(v.x, conef_query_term(conef_ld(row + (pk[0] & 0x7fffffffu)), pk[0], alpha));
-            v.y = __fadd_rn(v.y, conef_query_term(conef_ld(row + (pk[1] & 0x7fffffffu)), pk[1], alpha));
-            v.z = __fadd_rn(v.z, conef_query_term(conef_ld(row + (pk[2] & 0x7fffffffu)), pk[2], alpha));
-            v.w = __fadd_rn(v.w, conef_query_term(conef_ld(row + (pk[3] & 0x7fffffffu)), pk[3], alpha));
-            *reinterpret_cast<float4*>(xr) = v;
-        } else {
+    if (VEC) {
+        for (int64_t r = r0; r < r1; r += RB) {
+            float4 v[RB];
+            float cell[RB][4];
+#pragma unroll
+            for (int u = 0; u < RB; ++u) {
+                const int64_t rr = r + u < r1 ? r + u : r1 - 1;     // clamped: the loads are unconditional
+                const CsT* row = cs + rr * (int64_t)mod.w;
+                v[u] = *reinterpret_cast<const float4*>(x + rr * d + c0);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) cell[u][k] = conef_ld(row + (pk[k] & 0x7fffffffu));
+            }
+#pragma unroll
+            for (int u = 0; u < RB; ++u) {
+                if (r + u < r1) {
+                    float4 o;
+                    o.x = __fadd_rn(v[u].x, conef_query_term(cell[u][0], pk[0], alpha));
+                    o.y = __fadd_rn(v[u].y, conef_query_term(cell[u][1], pk[1], alpha));
+                    o.z = __fadd_rn(v[u].z, conef_query_term(cell[u][2], pk[2], alpha));
+                    o.w = __fadd_rn(v[u].w, conef_query_term(cell[u][3], pk[3], alpha));
+                    *reinterpret_cast<float4*>(x + (r + u) * d + c0) = o;
+                }
+            }
+        }
+    } else {
+        for (int64_t r = r0; r < r1; ++r) {
+            const CsT* row = cs + r * (int64_t)mod.w;
+            float* xr = x + r * d + c0;
 #pragma unroll
             for (int k = 0; k < 4; ++k)
                 if (c0 + k < d)
@@ -204,12 +224,28 @@ int launch_query(float* x, const CsT* cs, int64_t n, int64_t d, int32_t w, float
     int rpb = rows_per_block_for(n, col_blocks);
     dim3 grid((unsigned)col_blocks, (unsigned)((n + rpb - 1) / rpb));
     bool vec = (d % 4 == 0) && aligned16(x);
-    if (vec)
-        hipLaunchKernelGGL((cs_query_kernel<CsT, true>), grid, dim3(256), 0, stream, x, cs, n, d,
-                           conef_make_mod(w), alpha, hs, rpb);
-    else
-        hipLaunchKernelGGL((cs_query_kernel<CsT, false>), grid, dim3(256), 0, stream, x, cs, n, d,
-                           conef_make_mod(w), alpha, hs, rpb);
+    ConefMod mod = conef_make_mod(w);
+    if (!vec) {
+        hipLaunchKernelGGL((cs_query_kernel<CsT, false, 1>), grid, dim3(256), 0, stream, x, cs, n, d, mod, alpha, hs, rpb);
+        return (int)hipGetLastError();
+    }
+    // Rows in flight per thread: the whole row group when it is small; four at a time when the
+    // launch has too few workgroups to hide a round trip per row behind other waves; one otherwise
+    // (more costs registers, and with them resident waves, on the shapes that have rows to spare).
+    const int64_t wgs = (int64_t)grid.x * grid.y;
+    switch (rpb <= 5 ? rpb : wgs <= 256 ? 4 : 1) {
+#define CONEF_QUERY_CASE(RB)                                                                                         \
+    case RB:                                                                                                         \
+        hipLaunchKernelGGL((cs_query_kernel<CsT, true, RB>), grid, dim3(256), 0, stream, x, cs, n, d, mod, alpha, hs, \
+                           rpb);                                                                                     \
+        break
+        CONEF_QUERY_CASE(1);
+        CONEF_QUERY_CASE(2);
+        CONEF_QUERY_CASE(3);
+        CONEF_QUERY_CASE(4);
+        CONEF_QUERY_CASE(5);
+#undef CONEF_QUERY_CASE
+    }
     return (int)hipGetLastError();
 }
 
