@@ -34,7 +34,7 @@ __global__ void hash_table_kernel(int32_t* bucket, int32_t* sign, int64_t d, Con
 // with every load of the batch (values and gathered cells) issued before the first is used: a
 // thread's stores and later loads retire through one in-order counter, so row-at-a-time code pays
 // a full memory round trip per row.
-template <typename CsT, bool VEC, int RB>
+template <typename CsT, int VW, int RB>
 __global__ void __launch_bounds__(256)
 cs_query_kernel(float* __restrict__ x, const CsT* __restrict__ cs, int64_t n, int64_t d, ConefMod mod,
                 float alpha, ConefSeeds hs, int rows_per_block)
@@ -47,7 +47,8 @@ cs_query_kernel(float* __restrict__ x, const CsT* __restrict__ cs, int64_t n, in
         pk[k] = (c0 + k < d) ? conef_bucket_sign((int32_t)(c0 + k), mod, hs.a, hs.b, hs.sa, hs.sb) : 0u;
     int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
     int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
-    if (VEC) {
+    // VW = 4: rows are 16-byte aligned, one float4 per row; VW = 2: 8-byte aligned, two float2
+    if (VW > 1 && c0 + 4 <= d) {
         for (int64_t r = r0; r < r1; r += RB) {
             float4 v[RB];
             float cell[RB][4];
@@ -55,7 +56,13 @@ cs_query_kernel(float* __restrict__ x, const CsT* __restrict__ cs, int64_t n, in
             for (int u = 0; u < RB; ++u) {
                 const int64_t rr = r + u < r1 ? r + u : r1 - 1;     // clamped: the loads are unconditional
                 const CsT* row = cs + rr * (int64_t)mod.w;
-                v[u] = *reinterpret_cast<const float4*>(x + rr * d + c0);
+                const float* xr = x + rr * d + c0;
+                if (VW == 4) {
+                    v[u] = *reinterpret_cast<const float4*>(xr);
+                } else {
+                    const float2 lo = *reinterpret_cast<const float2*>(xr), hi = *reinterpret_cast<const float2*>(xr + 2);
+                    v[u] = make_float4(lo.x, lo.y, hi.x, hi.y);
+                }
 #pragma unroll
                 for (int k = 0; k < 4; ++k) cell[u][k] = conef_ld(row + (pk[k] & 0x7fffffffu));
             }
@@ -67,7 +74,13 @@ cs_query_kernel(float* __restrict__ x, const CsT* __restrict__ cs, int64_t n, in
                     o.y = __fadd_rn(v[u].y, conef_query_term(cell[u][1], pk[1], alpha));
                     o.z = __fadd_rn(v[u].z, conef_query_term(cell[u][2], pk[2], alpha));
                     o.w = __fadd_rn(v[u].w, conef_query_term(cell[u][3], pk[3], alpha));
-                    *reinterpret_cast<float4*>(x + (r + u) * d + c0) = o;
+                    float* xo = x + (r + u) * d + c0;
+                    if (VW == 4) {
+                        *reinterpret_cast<float4*>(xo) = o;
+                    } else {
+                        *reinterpret_cast<float2*>(xo) = make_float2(o.x, o.y);
+                        *reinterpret_cast<float2*>(xo + 2) = make_float2(o.z, o.w);
+                    }
                 }
             }
         }
@@ -223,10 +236,10 @@ int launch_query(float* x, const CsT* cs, int64_t n, int64_t d, int32_t w, float
     int64_t col_blocks = (d + 1023) / 1024;
     int rpb = rows_per_block_for(n, col_blocks);
     dim3 grid((unsigned)col_blocks, (unsigned)((n + rpb - 1) / rpb));
-    bool vec = (d % 4 == 0) && aligned16(x);
+    const int vw = (d % 4 == 0 && aligned16(x)) ? 4 : (d % 2 == 0 && (reinterpret_cast<uintptr_t>(x) & 7u) == 0) ? 2 : 1;
     ConefMod mod = conef_make_mod(w);
-    if (!vec) {
-        hipLaunchKernelGGL((cs_query_kernel<CsT, false, 1>), grid, dim3(256), 0, stream, x, cs, n, d, mod, alpha, hs, rpb);
+    if (vw == 1) {
+        hipLaunchKernelGGL((cs_query_kernel<CsT, 1, 1>), grid, dim3(256), 0, stream, x, cs, n, d, mod, alpha, hs, rpb);
         return (int)hipGetLastError();
     }
     // Rows in flight per thread: the whole row group when it is small; four at a time when the
@@ -234,10 +247,14 @@ int launch_query(float* x, const CsT* cs, int64_t n, int64_t d, int32_t w, float
     // (more costs registers, and with them resident waves, on the shapes that have rows to spare).
     const int64_t wgs = (int64_t)grid.x * grid.y;
     switch (rpb <= 5 ? rpb : wgs <= 256 ? 4 : 1) {
-#define CONEF_QUERY_CASE(RB)                                                                                         \
-    case RB:                                                                                                         \
-        hipLaunchKernelGGL((cs_query_kernel<CsT, true, RB>), grid, dim3(256), 0, stream, x, cs, n, d, mod, alpha, hs, \
-                           rpb);                                                                                     \
+#define CONEF_QUERY_CASE(RB)                                                                                          \
+    case RB:                                                                                                          \
+        if (vw == 4)                                                                                                  \
+            hipLaunchKernelGGL((cs_query_kernel<CsT, 4, RB>), grid, dim3(256), 0, stream, x, cs, n, d, mod, alpha, hs, \
+                               rpb);                                                                                  \
+        else                                                                                                          \
+            hipLaunchKernelGGL((cs_query_kernel<CsT, 2, RB>), grid, dim3(256), 0, stream, x, cs, n, d, mod, alpha, hs, \
+                               rpb);                                                                                  \
         break
         CONEF_QUERY_CASE(1);
         CONEF_QUERY_CASE(2);
