@@ -58,6 +58,10 @@ inline bool conef_rowlist_shape(int64_t n, int64_t d, int32_t w, bool cells, Con
     if (rb > 16) rb = 16;
     if (rb < 1) rb = 1;
     while (rb > 1 && conef_rowlist_lds((int)rb, d, w, cells) > 64 * 1024) --rb;
+    // rows that are not a whole number of 16-byte quads: tiles of 2 (4) rows start on a quad again,
+    // and the fronts then read a tile as one flat run of quads
+    if (d % 4 == 2 && rb > 1) rb &= ~(int64_t)1;
+    else if (d % 2 == 1 && rb >= 4) rb &= ~(int64_t)3;
     size_t lds = conef_rowlist_lds((int)rb, d, w, cells);
     if (lds > kConefRowlistLdsLimit) return false;
     s->rb = (int)rb;
@@ -80,7 +84,8 @@ struct ConefListVec {
     {
         const float* base = vec + row0 * d;
         const int total = rows * d;
-        if (vec_ok) {
+        // a tile is one contiguous run: 16-byte accesses whenever it starts on a 16-byte boundary
+        if (vec_ok || (reinterpret_cast<uintptr_t>(base) & 15u) == 0) {
             // eight loads in flight per thread; indices past the end are clamped, not branched around
             const int total4 = total >> 2;
             for (int q0 = threadIdx.x; q0 < total4; q0 += 8 * kConefRowlistThreads) {
@@ -96,6 +101,7 @@ struct ConefListVec {
                     if (q < total4) reinterpret_cast<float4*>(vals)[q] = t[u];
                 }
             }
+            for (int e = (total4 << 2) + threadIdx.x; e < total; e += kConefRowlistThreads) vals[e] = base[e];
         } else {
             for (int e0 = threadIdx.x; e0 < total; e0 += 8 * kConefRowlistThreads) {
                 float t[8];
@@ -189,6 +195,57 @@ struct ConefListRandBlock {
                     reinterpret_cast<float4*>(base)[q] = o;
                     reinterpret_cast<float4*>(vals)[q] = v;
                 }
+            }
+        } else if ((reinterpret_cast<uintptr_t>(base) & 15u) == 0) {
+            // rows that are not whole quads, but the tile starts on one: the tile as one flat run of
+            // quads, whose four elements may sit in two rows
+            const int total = rows * d, total4 = total >> 2;
+            for (int q0 = threadIdx.x; q0 < total4; q0 += 4 * kConefRowlistThreads) {
+                float4 g[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    int q = q0 + u * kConefRowlistThreads;
+                    g[u] = reinterpret_cast<const float4*>(base)[q < total4 ? q : total4 - 1];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    int q = q0 + u * kConefRowlistThreads;
+                    if (q >= total4) break;
+                    const int e = q << 2;
+                    int row = e / d, col = e - row * d;
+                    const float gv[4] = {g[u].x, g[u].y, g[u].z, g[u].w};
+                    uint32_t p[4];
+                    float c[4], o[4], v[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        p[k] = pk[col];
+                        c[k] = cells[row * w + (p[k] & 0x7fffffffu)];
+                        if (++col == d) {
+                            col = 0;
+                            ++row;
+                        }
+                    }
+                    const int64_t f = f0 + e;
+                    if ((f < blk.end && f + 4 > blk.start) || f < blk.rest) {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) v[k] = finish(f + k, gv[k], c[k], p[k], &o[k]);
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            o[k] = 0.f;
+                            v[k] = __fadd_rn(gv[k], conef_query_term(c[k], p[k], alpha));
+                        }
+                    }
+                    reinterpret_cast<float4*>(base)[q] = make_float4(o[0], o[1], o[2], o[3]);
+                    reinterpret_cast<float4*>(vals)[q] = make_float4(v[0], v[1], v[2], v[3]);
+                }
+            }
+            for (int e = (total4 << 2) + threadIdx.x; e < total; e += kConefRowlistThreads) {
+                const int row = e / d, col = e - row * d;
+                const uint32_t p = pk[col];
+                float o;
+                vals[e] = finish(f0 + e, base[e], cells[row * w + (p & 0x7fffffffu)], p, &o);
+                base[e] = o;
             }
         } else {
             const int total = rows * d;
