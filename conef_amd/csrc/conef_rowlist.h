@@ -77,45 +77,44 @@ inline bool conef_rowlist_shape(int64_t n, int64_t d, int32_t w, bool cells, Con
 // DenseCS.update: the value is the dense tensor itself.
 struct ConefListVec {
     const float* vec;
-    bool vec_ok;           // 16-byte accesses allowed: base aligned and d % 4 == 0
+    bool vec_ok;           // base 16-byte aligned and d % 4 == 0 (the tile copy works either way)
     static constexpr bool kNeedsCells = false;
     __device__ __forceinline__ void stage(int64_t row0, int rows, int d, int, float* vals, const float*,
                                           const uint32_t*) const
     {
         const float* base = vec + row0 * d;
         const int total = rows * d;
-        // a tile is one contiguous run: 16-byte accesses whenever it starts on a 16-byte boundary
-        if (vec_ok || (reinterpret_cast<uintptr_t>(base) & 15u) == 0) {
-            // eight loads in flight per thread; indices past the end are clamped, not branched around
-            const int total4 = total >> 2;
-            for (int q0 = threadIdx.x; q0 < total4; q0 += 8 * kConefRowlistThreads) {
-                float4 t[8];
+        // A tile is one contiguous run: up to three leading elements bring it to a 16-byte
+        // boundary, 16-byte loads from there (eight in flight per thread; indices past the end are
+        // clamped, not branched around), the last few elements one by one.
+        int lead = (int)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(base) & 15u)) & 15u) >> 2);
+        if (lead > total) lead = total;
+        const int total4 = (total - lead) >> 2;
+        const float4* src4 = reinterpret_cast<const float4*>(base + lead);
+        for (int q0 = threadIdx.x; q0 < total4; q0 += 8 * kConefRowlistThreads) {
+            float4 t[8];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    int q = q0 + u * kConefRowlistThreads;
-                    t[u] = reinterpret_cast<const float4*>(base)[q < total4 ? q : total4 - 1];
-                }
+            for (int u = 0; u < 8; ++u) {
+                int q = q0 + u * kConefRowlistThreads;
+                t[u] = src4[q < total4 ? q : total4 - 1];
+            }
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    int q = q0 + u * kConefRowlistThreads;
-                    if (q < total4) reinterpret_cast<float4*>(vals)[q] = t[u];
+            for (int u = 0; u < 8; ++u) {
+                int q = q0 + u * kConefRowlistThreads;
+                if (q < total4) {
+                    if (lead == 0) {
+                        reinterpret_cast<float4*>(vals)[q] = t[u];
+                    } else {
+                        float* o = vals + lead + (q << 2);
+                        o[0] = t[u].x; o[1] = t[u].y; o[2] = t[u].z; o[3] = t[u].w;
+                    }
                 }
             }
-            for (int e = (total4 << 2) + threadIdx.x; e < total; e += kConefRowlistThreads) vals[e] = base[e];
-        } else {
-            for (int e0 = threadIdx.x; e0 < total; e0 += 8 * kConefRowlistThreads) {
-                float t[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    int e = e0 + u * kConefRowlistThreads;
-                    t[u] = base[e < total ? e : total - 1];
-                }
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    int e = e0 + u * kConefRowlistThreads;
-                    if (e < total) vals[e] = t[u];
-                }
-            }
+        }
+        const int rest = total - (total4 << 2);          // leading and trailing elements, at most 6
+        if ((int)threadIdx.x < rest) {
+            const int e = (int)threadIdx.x < lead ? (int)threadIdx.x : (int)threadIdx.x + (total4 << 2);
+            vals[e] = base[e];
         }
     }
 };
@@ -196,22 +195,27 @@ struct ConefListRandBlock {
                     reinterpret_cast<float4*>(vals)[q] = v;
                 }
             }
-        } else if ((reinterpret_cast<uintptr_t>(base) & 15u) == 0) {
-            // rows that are not whole quads, but the tile starts on one: the tile as one flat run of
-            // quads, whose four elements may sit in two rows
-            const int total = rows * d, total4 = total >> 2;
+        } else {
+            // Rows that are not whole aligned quads: the tile as one flat run.  Up to three leading
+            // elements bring it to a 16-byte boundary; from there quads, whose four elements may
+            // sit in two rows; the last few elements one by one.
+            const int total = rows * d;
+            int lead = (int)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(base) & 15u)) & 15u) >> 2);
+            if (lead > total) lead = total;
+            const int total4 = (total - lead) >> 2;
+            float4* base4 = reinterpret_cast<float4*>(base + lead);
             for (int q0 = threadIdx.x; q0 < total4; q0 += 4 * kConefRowlistThreads) {
                 float4 g[4];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     int q = q0 + u * kConefRowlistThreads;
-                    g[u] = reinterpret_cast<const float4*>(base)[q < total4 ? q : total4 - 1];
+                    g[u] = base4[q < total4 ? q : total4 - 1];
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     int q = q0 + u * kConefRowlistThreads;
                     if (q >= total4) break;
-                    const int e = q << 2;
+                    const int e = lead + (q << 2);
                     int row = e / d, col = e - row * d;
                     const float gv[4] = {g[u].x, g[u].y, g[u].z, g[u].w};
                     uint32_t p[4];
@@ -236,32 +240,23 @@ struct ConefListRandBlock {
                             v[k] = __fadd_rn(gv[k], conef_query_term(c[k], p[k], alpha));
                         }
                     }
-                    reinterpret_cast<float4*>(base)[q] = make_float4(o[0], o[1], o[2], o[3]);
-                    reinterpret_cast<float4*>(vals)[q] = make_float4(v[0], v[1], v[2], v[3]);
+                    base4[q] = make_float4(o[0], o[1], o[2], o[3]);
+                    if (lead == 0) {
+                        reinterpret_cast<float4*>(vals)[q] = make_float4(v[0], v[1], v[2], v[3]);
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) vals[e + k] = v[k];
+                    }
                 }
             }
-            for (int e = (total4 << 2) + threadIdx.x; e < total; e += kConefRowlistThreads) {
+            const int rest = total - (total4 << 2);      // leading and trailing elements, at most 6
+            if ((int)threadIdx.x < rest) {
+                const int e = (int)threadIdx.x < lead ? (int)threadIdx.x : (int)threadIdx.x + (total4 << 2);
                 const int row = e / d, col = e - row * d;
                 const uint32_t p = pk[col];
                 float o;
                 vals[e] = finish(f0 + e, base[e], cells[row * w + (p & 0x7fffffffu)], p, &o);
                 base[e] = o;
-            }
-        } else {
-            const int total = rows * d;
-            int row = threadIdx.x / d, col = threadIdx.x - row * d;
-            const int srow = kConefRowlistThreads / d, sc = kConefRowlistThreads - srow * d;
-            for (int e = threadIdx.x; e < total; e += kConefRowlistThreads) {
-                uint32_t p = pk[col];
-                float o;
-                vals[e] = finish(f0 + e, base[e], cells[row * w + (p & 0x7fffffffu)], p, &o);
-                base[e] = o;
-                row += srow;
-                col += sc;
-                if (col >= d) {
-                    col -= d;
-                    ++row;
-                }
             }
         }
     }

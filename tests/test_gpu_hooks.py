@@ -58,7 +58,10 @@ def test_randomblock_dense_ef_bit_exact(oracle, shapes, ratio):
 @pytest.mark.parametrize("shapes,ratio,ss", [([(6, 5, 3), (7,), (4, 9)], 0.3, 0.5), (RESNET20_SHAPES, 0.1, 0.2),
                                              ([(5, 26_000)], 0.1, 0.1), ([(40, 650), (650,), (26, 650)], 0.05, 0.1),
                                              ([(5, 26_003)], 0.55, 0.1), ([(3, 40_001), (7, 30_000)], 0.97, 0.3),
-                                             ([(2, 50_000)], 1.0, 0.2)])
+                                             ([(2, 50_000)], 1.0, 0.2),
+                                             # tensors that start 4, 8 and 12 bytes past a 16-byte boundary
+                                             ([(1,), (21, 650), (2,), (33, 1023), (64, 576)], 0.2, 0.1),
+                                             ([(3,), (40, 650), (2,), (64, 576), (7, 333)], 0.3, 0.1)])
 @pytest.mark.parametrize("bucket_cls", [FakeGradBucket, OldApiGradBucket])
 def test_randomblock_conef_parity(oracle, shapes, ratio, ss, bucket_cls):
     from conef_amd.RandomBlock_hook import RandomBlock_hook, RandomBlockState

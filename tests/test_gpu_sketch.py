@@ -234,6 +234,25 @@ def test_planned_update_bit_exact(oracle, n, d, ss, kind):
         np.testing.assert_array_equal(to_np(cs.cs), o.cs)
 
 
+@pytest.mark.parametrize("n,d,ss", [(2100, 650, 0.1), (33, 1023, 0.3), (64, 576, 0.2), (1, 2, 0.5), (3, 5, 0.5)])
+def test_planned_update_unaligned_start(oracle, n, d, ss):
+    """Row lists read a tile as one flat run; the tensor may start 4, 8 or 12 bytes past a 16-byte
+    boundary (a parameter in the middle of a bucket)."""
+    from conef_amd.compressors.CountSketch import DenseCS
+    rng = np.random.RandomState(n + d)
+    cs = DenseCS(n, d, ss)
+    o = oracle.DenseCS(n, d, ss)
+    for off in (1, 2, 3):
+        v = (rng.randn(n, d) * 1e-3).astype(np.float32)
+        arena = torch.zeros(n * d + 8, device="cuda")
+        vd = arena[off:off + n * d].view(n, d)
+        vd.copy_(dev(v))
+        cs.update(vd, 0.9)
+        o.update(v, 0.9)
+        np.testing.assert_array_equal(to_np(cs.cs), o.cs)
+        np.testing.assert_array_equal(to_np(vd), v)                       # the input is only read
+
+
 @pytest.mark.parametrize("chunk,tbin", [(1024, 64), (2048, 512), (8192, 256), (4096, 128)])
 def test_planned_update_any_tiling(oracle, monkeypatch, chunk, tbin):
     from conef_amd.compressors.CountSketch import DenseCS
