@@ -358,7 +358,11 @@ def hook_steps(args, results):
         for _ in range(3):
             step()
         torch.cuda.synchronize()
-        reps = 5
+        # enough repetitions for about 40 ms of timed work (small models: a step is tens of microseconds)
+        t_probe = time.perf_counter()
+        step()
+        torch.cuda.synchronize()
+        reps = max(5, min(400, int(0.04 / max(time.perf_counter() - t_probe, 1e-5))))
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
         e0.record()

@@ -886,12 +886,8 @@ struct GsBatch {
 };
 
 template <int RP, int RPT>
-__global__ void __launch_bounds__(kGsRegThreads)
-gram_schmidt_reg_kernel(GsBatch batch, int r, float eps)
+__device__ __forceinline__ void gs_reg_body(float* __restrict__ a, int rows, float (&red)[2][4][RP], int r, float eps)
 {
-    float* __restrict__ a = batch.a[blockIdx.x];
-    const int rows = batch.rows[blockIdx.x];
-    __shared__ float red[2][4][RP];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int nrt = (rows + kGsRegThreads - 1) / kGsRegThreads;      // row slots in use (uniform)
     float v[RPT][RP];
@@ -928,6 +924,33 @@ gram_schmidt_reg_kernel(GsBatch batch, int r, float eps)
             }
         }
     }
+}
+
+template <int RP, int RPT>
+__global__ void __launch_bounds__(kGsRegThreads)
+gram_schmidt_reg_kernel(GsBatch batch, int r, float eps)
+{
+    __shared__ float red[2][4][RP];
+    gs_reg_body<RP, RPT>(batch.a[blockIdx.x], batch.rows[blockIdx.x], red, r, eps);
+}
+
+// The same, for a launch whose matrices differ in height: every workgroup takes the body sized
+// for its own matrix (1, 4, 16 or all row slots a thread), so the short factors of a bucket are
+// not a launch of their own in front of the tall ones.  A workgroup runs exactly the code the
+// one-size kernel would run on its matrix.
+template <int RP>
+__global__ void __launch_bounds__(kGsRegThreads)
+gram_schmidt_reg_mixed_kernel(GsBatch batch, int r, float eps)
+{
+    __shared__ float red[2][4][RP];
+    constexpr int kAll = kGsRegFloats / RP;
+    float* a = batch.a[blockIdx.x];
+    const int rows = batch.rows[blockIdx.x];
+    const int nrt = (rows + kGsRegThreads - 1) / kGsRegThreads;
+    if (nrt <= 1) gs_reg_body<RP, 1>(a, rows, red, r, eps);
+    else if (nrt <= 4 && kAll >= 4) gs_reg_body<RP, (kAll >= 4 ? 4 : kAll)>(a, rows, red, r, eps);
+    else if (nrt <= 16 && kAll >= 16) gs_reg_body<RP, (kAll >= 16 ? 16 : kAll)>(a, rows, red, r, eps);
+    else gs_reg_body<RP, kAll>(a, rows, red, r, eps);
 }
 
 // Matrices beyond one workgroup's registers: the same register-resident scheme over up to 128
@@ -1361,8 +1384,22 @@ inline int gs_reg_class(const float* a, int64_t rows, int r)
     return all;
 }
 
+// slots: the one class all matrices of the batch share, or 0 for a batch of mixed classes
 inline int gs_launch_reg_batch(const GsBatch& batch, int count, int r, int slots, float eps, hipStream_t s)
 {
+    if (slots == 0) {
+#define CONEF_GSM(RP) \
+    hipLaunchKernelGGL((gram_schmidt_reg_mixed_kernel<RP>), dim3((unsigned)count), dim3(kGsRegThreads), 0, s, batch, r, eps)
+        switch (rank_bound(r)) {
+            case 1: CONEF_GSM(1); break;
+            case 2: CONEF_GSM(2); break;
+            case 4: CONEF_GSM(4); break;
+            case 8: CONEF_GSM(8); break;
+            default: return CONEF_ERR_INVALID;
+        }
+#undef CONEF_GSM
+        return (int)hipGetLastError();
+    }
 #define CONEF_GSR_GO(RP, RPT) \
     hipLaunchKernelGGL((gram_schmidt_reg_kernel<RP, (RPT)>), dim3((unsigned)count), dim3(kGsRegThreads), 0, s, batch, r, eps)
 #define CONEF_GSR(RP)                                                       \
@@ -1840,16 +1877,22 @@ int conef_gram_schmidt_batch_f32(float* const* mats, const int64_t* rows, const 
             done[(size_t)k] = 1;
             continue;
         }
+        // all matrices of this rank that fit one workgroup's registers, whatever their height
         GsBatch batch;
         int nb = 0;
+        bool mixed = false;
+        const bool mix_ok = rank_bound(ranks[k]) <= 8;     // above that the unrolled bodies are too large to pair up
         for (int j = k; j < count && nb < kGsBatchMax; ++j) {
-            if (done[(size_t)j] || ranks[j] != ranks[k] || gs_reg_class(mats[j], rows[j], ranks[j]) != cls) continue;
+            if (done[(size_t)j] || ranks[j] != ranks[k]) continue;
+            const int cj = gs_reg_class(mats[j], rows[j], ranks[j]);
+            if (cj < 0 || (cj != cls && !mix_ok)) continue;
+            mixed = mixed || cj != cls;
             batch.a[nb] = mats[j];
             batch.rows[nb] = (int)rows[j];
             ++nb;
             done[(size_t)j] = 1;
         }
-        int rc = gs_launch_reg_batch(batch, nb, ranks[k], cls, eps, s);
+        int rc = gs_launch_reg_batch(batch, nb, ranks[k], mixed ? 0 : cls, eps, s);
         if (rc != CONEF_OK) return rc;
     }
     return CONEF_OK;
