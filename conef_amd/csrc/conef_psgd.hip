@@ -1836,37 +1836,49 @@ int conef_gram_schmidt_batch_f32(float* const* mats, const int64_t* rows, const 
     // kernels of conef_gs_lanes.h: matrices of one rank and class share launches (up to 48 matrices
     // of the one-workgroup kernel; up to 24 matrices and 128 workgroups of the other)
     const bool ws_ok = workspace && workspace_bytes >= (int64_t)sizeof(GslWs) && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0;
-    for (int k = 0; k < count; ++k) {
-        if (done[(size_t)k]) continue;
-        const GslChoice ck = gsl_choose(rows[k], ranks[k]);
-        if (ck.kind == 0 || (ck.kind == 2 && !ws_ok)) continue;
-        GslBatch grid;
-        GswBatch single;
-        std::vector<int> members;
-        int nb = 0, wgs = 0;
-        const int cap = ck.kind == 1 ? kGswBatchMax : kGslMaxItems;
-        for (int j = k; j < count && nb < cap; ++j) {
-            if (done[(size_t)j] || ranks[j] != ranks[k]) continue;
-            const GslChoice cj = gsl_choose(rows[j], ranks[j]);
-            if (cj.kind != ck.kind || cj.rpt != ck.rpt) continue;
-            if (ck.kind == 2 && wgs + cj.wgs > kGslMaxWgs) continue;
-            if (ck.kind == 1) {
-                single.a[nb] = mats[j];
-                single.rows[nb] = (int)rows[j];
-            } else {
-                grid.a[nb] = mats[j];
-                grid.elements[nb] = rows[j] * ranks[j];
-                grid.first[nb] = wgs;
+    // Two rounds: first the launches of the several-workgroup kernel, then what is left for the
+    // one-workgroup kernel.  A launch of the former lasts about r exchanges whatever it holds, so
+    // it also takes the bucket's shorter factors of the same rank while it has workgroups to
+    // spare, each on its own group of workgroups: they are then no launch of their own.
+    for (int round = 2; round >= 1; --round) {
+        for (int k = 0; k < count; ++k) {
+            if (done[(size_t)k]) continue;
+            const GslChoice ck = gsl_choose(rows[k], ranks[k]);
+            if (ck.kind != round || (ck.kind == 2 && !ws_ok)) continue;
+            GslBatch grid;
+            GswBatch single;
+            std::vector<int> members;
+            int nb = 0, wgs = 0;
+            const int cap = ck.kind == 1 ? kGswBatchMax : kGslMaxItems;
+            for (int j = ck.kind == 2 ? 0 : k; j < count && nb < cap; ++j) {      // guests may come before the lead
+                if (done[(size_t)j] || ranks[j] != ranks[k]) continue;
+                GslChoice cj = gsl_choose(rows[j], ranks[j]);
+                if (ck.kind == 2 && cj.kind == 1) {       // a shorter factor as a guest of this launch
+                    const int64_t per = (int64_t)kGslThreads * ck.rpt;
+                    cj.kind = 2;
+                    cj.rpt = ck.rpt;
+                    cj.wgs = (int)((rows[j] * ranks[j] + per - 1) / per);
+                }
+                if (cj.kind != ck.kind || cj.rpt != ck.rpt) continue;
+                if (ck.kind == 2 && wgs + cj.wgs > kGslMaxWgs) continue;
+                if (ck.kind == 1) {
+                    single.a[nb] = mats[j];
+                    single.rows[nb] = (int)rows[j];
+                } else {
+                    grid.a[nb] = mats[j];
+                    grid.elements[nb] = rows[j] * ranks[j];
+                    grid.first[nb] = wgs;
+                }
+                wgs += cj.wgs;
+                ++nb;
+                members.push_back(j);
             }
-            wgs += cj.wgs;
-            ++nb;
-            members.push_back(j);
+            if (ck.kind == 2) grid.first[nb] = wgs;
+            const int rc = ck.kind == 1 ? gsw_launch(single, nb, ranks[k], ck.rpt, eps, s)
+                                        : gsl_launch(grid, nb, ranks[k], ck.rpt, wgs, eps, workspace, s);
+            if (rc != CONEF_OK) break;      // the other kernels below take what is left
+            for (int j : members) done[(size_t)j] = 1;
         }
-        if (ck.kind == 2) grid.first[nb] = wgs;
-        const int rc = ck.kind == 1 ? gsw_launch(single, nb, ranks[k], ck.rpt, eps, s)
-                                    : gsl_launch(grid, nb, ranks[k], ck.rpt, wgs, eps, workspace, s);
-        if (rc != CONEF_OK) break;      // the other kernels below take what is left
-        for (int j : members) done[(size_t)j] = 1;
     }
     for (int k = 0; k < count; ++k) {
         if (done[(size_t)k]) continue;
