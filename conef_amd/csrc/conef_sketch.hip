@@ -120,6 +120,53 @@ cs3_query_kernel(float* __restrict__ x, const float* __restrict__ cs0, const flo
     }
 }
 
+// The same with a thread on 4 consecutive columns of 16-byte aligned rows, RB rows at a time, every
+// load of a batch (the values and 12 gathered cells a row) requested before the first is used; the
+// six hashes of a column are paid once per row group.  Same arithmetic per element as above.
+template <int RB>
+__global__ void __launch_bounds__(256)
+cs3_query_vec_kernel(float* __restrict__ x, const float* __restrict__ cs0, const float* __restrict__ cs1,
+                     const float* __restrict__ cs2, int64_t n, int64_t d, ConefMod mod, float alpha, int rows_per_block)
+{
+    const int64_t c0 = (blockIdx.x * (int64_t)blockDim.x + threadIdx.x) * 4;
+    if (c0 >= d) return;                      // d is a multiple of 4 here
+    uint32_t pk[3][4];
+#pragma unroll
+    for (int h = 0; h < 3; ++h) {
+        ConefSeeds s = conef_hash3_seeds(h, /*for_query=*/true);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) pk[h][k] = conef_bucket_sign((int32_t)(c0 + k), mod, s.a, s.b, s.sa, s.sb);
+    }
+    const float* cs[3] = {cs0, cs1, cs2};
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
+    for (int64_t r = r0; r < r1; r += RB) {
+        float4 v[RB];
+        float cell[RB][3][4];
+#pragma unroll
+        for (int u = 0; u < RB; ++u) {
+            const int64_t rr = r + u < r1 ? r + u : r1 - 1;     // clamped: the loads are unconditional
+            v[u] = *reinterpret_cast<const float4*>(x + rr * d + c0);
+#pragma unroll
+            for (int h = 0; h < 3; ++h)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) cell[u][h][k] = cs[h][rr * (int64_t)mod.w + (pk[h][k] & 0x7fffffffu)];
+        }
+#pragma unroll
+        for (int u = 0; u < RB; ++u) {
+            if (r + u < r1) {
+                float in[4] = {v[u].x, v[u].y, v[u].z, v[u].w}, o[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    o[k] = __fadd_rn(in[k], conef_median3(conef_query_term(cell[u][0][k], pk[0][k], alpha),
+                                                          conef_query_term(cell[u][1][k], pk[1][k], alpha),
+                                                          conef_query_term(cell[u][2][k], pk[2][k], alpha)));
+                *reinterpret_cast<float4*>(x + (r + u) * d + c0) = make_float4(o[0], o[1], o[2], o[3]);
+            }
+        }
+    }
+}
+
 // three-sketch update (CountSketchHash3.py:27-98); out buffers start as copies of the snapshots
 __global__ void __launch_bounds__(256)
 cs3_update_kernel(const float* __restrict__ vec, const float* __restrict__ in0, const float* __restrict__ in1,
@@ -353,6 +400,18 @@ int conef_cs3_query_f32(float* x, const float* cs0, const float* cs1, const floa
     if (n < 0 || d < 0 || w < 1 || w > (1 << 30) || d > 0x7fffffffLL) return CONEF_ERR_INVALID;
     if (n == 0 || d == 0) return CONEF_OK;
     if (!x || !cs0 || !cs1 || !cs2) return CONEF_ERR_INVALID;
+    if (d % 4 == 0 && aligned16(x)) {
+        const int64_t cb = (d + 1023) / 1024;
+        const int rows = rows_per_block_for(n, cb);
+        dim3 g4((unsigned)cb, (unsigned)((n + rows - 1) / rows));
+        if (rows == 1)
+            hipLaunchKernelGGL(cs3_query_vec_kernel<1>, g4, dim3(256), 0, (hipStream_t)stream, x, cs0, cs1, cs2, n, d,
+                               conef_make_mod(w), alpha, rows);
+        else
+            hipLaunchKernelGGL(cs3_query_vec_kernel<4>, g4, dim3(256), 0, (hipStream_t)stream, x, cs0, cs1, cs2, n, d,
+                               conef_make_mod(w), alpha, rows);
+        return (int)hipGetLastError();
+    }
     int64_t col_blocks = (d + 255) / 256;
     int rpb = rows_per_block_for(n, col_blocks);
     dim3 grid((unsigned)col_blocks, (unsigned)((n + rpb - 1) / rpb));

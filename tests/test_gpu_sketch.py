@@ -136,7 +136,7 @@ def test_half_sketch_parity(oracle, n, d, ss):
     np.testing.assert_array_equal(to_np(cs.cs), o.cs)
 
 
-@pytest.mark.parametrize("n,d,ss", [(3, 17, 0.3), (64, 576, 0.2), (5, 50_000, 0.1)])
+@pytest.mark.parametrize("n,d,ss", [(3, 17, 0.3), (64, 576, 0.2), (5, 50_000, 0.1), (641, 1028, 0.2), (1, 4096, 0.1)])
 def test_hash3_parity(oracle, n, d, ss):
     from conef_amd.compressors.CountSketchHash3 import DenseCSHash3
     rng = np.random.RandomState(d + 1)
