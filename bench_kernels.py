@@ -328,6 +328,7 @@ def hook_steps(args, results):
          lambda: (hPowerSGDState(None, matrix_approximation_rank=8, start_powerSGD_iter=2, use_error_compression=True,
                                  topk_ratio=0.4), hpowerSGD_hook)),
         # the same steps with the buckets spread over side streams (hook_streams, not in the reference)
+        ("hook cfg3 WRN-28-10, PowerSGD r=4 + sketch 20%%, %d streams" % ns, wrn, psgd(4, 0.2, ns)),
         ("hook cfg5 BERT-large, PowerSGD r=8 + sketch 10%%, %d streams" % ns, bert, psgd(8, 0.1, ns)),
         ("hook cfg5 BERT-large, PowerSGD r=32 + sketch 10%%, %d streams" % ns, bert, psgd(32, 0.1, ns)),
         ("hook cfg5 BERT-large, hPowerSGD r=8 + top-k error, %d streams" % ns, bert,

@@ -2298,10 +2298,19 @@ int pqt_sketch_group(const ConefPsgdItem* items, const std::vector<int>& members
     std::vector<RowlistResidualItem<RP, FAST>> table;
     std::vector<int> blocks;
     size_t lds = 0;
+    // Full-height tiles when the bucket has 600 of them that way (over two a CU); shorter ones otherwise.
+    // (Resident workgroups are bounded by LDS, so fewer, fuller tiles mean fewer rounds of them.)
+    int64_t full_tiles = 0;
+    for (int j : members) {
+        ConefRowlistShape shape;
+        if (!conef_rowlist_shape(items[j].n, items[j].m, items[j].w, false, &shape, 0)) return CONEF_ERR_INVALID;
+        full_tiles += shape.tiles;
+    }
+    const int companions = full_tiles >= 600 ? 0 : (int)members.size();
     for (int j : members) {
         const ConefPsgdItem& it = items[j];
         ConefRowlistShape shape;
-        if (!conef_rowlist_shape(it.n, it.m, it.w, false, &shape, (int)members.size())) return CONEF_ERR_INVALID;
+        if (!conef_rowlist_shape(it.n, it.m, it.w, false, &shape, companions)) return CONEF_ERR_INVALID;
         RowlistResidualItem<RP, FAST> t = {{it.x, it.p, it.q, it.r},
                                            conef_rowlist_view((const ConefPlanHeader*)it.plan_host, it.plan_dev),
                                            it.cs, it.cs, it.n, (int)it.m, it.w, shape.rb};
@@ -2501,6 +2510,13 @@ int conef_psgd_sketch_update_batch_f32(const ConefPsgdItem* items, int32_t count
     std::vector<RowlistVecItem> table;
     std::vector<int> blocks;
     size_t lds = 0;
+    int64_t full_tiles = 0;     // as in pqt_sketch_group: full-height tiles when there are 600 of them
+    for (int k = 0; k < count; ++k) {
+        ConefRowlistShape shape;
+        if (conef_rowlist_shape(items[k].n, items[k].m, items[k].w, ConefListVec::kNeedsCells, &shape, 0))
+            full_tiles += shape.tiles;
+    }
+    const int companions = full_tiles >= 600 ? 0 : count;
     for (int k = 0; k < count; ++k) {
         const ConefPsgdItem& it = items[k];
         const ConefPlanHeader* hp = (const ConefPlanHeader*)it.plan_host;
@@ -2508,7 +2524,7 @@ int conef_psgd_sketch_update_batch_f32(const ConefPsgdItem* items, int32_t count
             !conef_plan_matches(hp, it.n, it.m, it.w, a, b) || hp->kind != kConefPlanRowlist)
             return CONEF_ERR_INVALID;
         ConefRowlistShape shape;
-        if (!conef_rowlist_shape(it.n, it.m, it.w, ConefListVec::kNeedsCells, &shape, count)) return CONEF_ERR_INVALID;
+        if (!conef_rowlist_shape(it.n, it.m, it.w, ConefListVec::kNeedsCells, &shape, companions)) return CONEF_ERR_INVALID;
         RowlistVecItem t = {{it.err, aligned16(it.err) && it.m % 4 == 0}, conef_rowlist_view(hp, it.plan_dev), it.cs, it.cs,
                             it.n, (int)it.m, it.w, shape.rb};
         table.push_back(t);

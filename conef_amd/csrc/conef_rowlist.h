@@ -47,14 +47,15 @@ inline size_t conef_rowlist_lds(int rb, int64_t d, int32_t w, bool cells)
 // Rows per tile: about 32 KB of values (several tiles per CU), but no more than leaves a
 // thousand tiles for the 256 CUs.
 // `companions`: matrices of about this size that share the launch (a batch leaves enough tiles
-// for the machine with taller tiles per matrix).
+// for the machine with taller tiles per matrix); 0: full-height tiles whatever the count (for a
+// batch whose caller has checked that it has tiles enough that way).
 inline bool conef_rowlist_shape(int64_t n, int64_t d, int32_t w, bool cells, ConefRowlistShape* s, int companions = 1)
 {
     if (d < 1 || d > kConefRowlistMaxCols || n < 1 || w < 1) return false;
     int64_t rb = 8192 / d;
     // tiles to spare: half-height ones, twice as many resident per CU (a quarter was slower again)
     if (rb >= 2 && n / rb >= 2048) rb = (rb + 1) / 2;
-    if (rb > n * companions / 1024) rb = n * companions / 1024;
+    if (companions > 0 && rb > n * companions / 1024) rb = n * companions / 1024;
     if (rb > 16) rb = 16;
     if (rb < 1) rb = 1;
     while (rb > 1 && conef_rowlist_lds((int)rb, d, w, cells) > 64 * 1024) --rb;
