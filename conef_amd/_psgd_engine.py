@@ -8,6 +8,7 @@ streaming passes over its memory: the error add is fused into the first product,
 (dense, or count-sketched) into the last.
 """
 import logging
+import os
 
 import torch
 import torch.distributed as dist
@@ -127,7 +128,7 @@ class _RoundPlan:
     and layout, so that a step costs a handful of foreign calls however many tensors it has."""
     __slots__ = ("key", "shapes", "work", "passthrough", "before", "after", "total_ps", "total_qs", "arena_key", "ps",
                  "qs", "items", "count", "sketches", "fused_sketch", "batched_update", "residual_offsets",
-                 "topk_table")
+                 "topk_table", "q_next", "q_next_ptrs", "q_next_ready", "made")
 
 
 def _build_round(state, grads, shapes, key, error_mode):
@@ -159,6 +160,12 @@ def _build_round(state, grads, shapes, key, error_mode):
     plan.fused_sketch = False
     plan.batched_update = False
     plan.topk_table = None
+    # Second buffer for the Q factors, orthogonalised at the end of a round for the bucket's next
+    # round (conef_psgd_round_ahead_f32).  Derived data: q_memory_dict keeps what the reference
+    # keeps, and the flag falls with the plan whenever the state is replaced.
+    plan.q_next = plan.q_next_ptrs = None
+    plan.q_next_ready = False
+    plan.made = None
     plan.residual_offsets = []
     off = 0
     for _, n, m, _ in plan.work:
@@ -262,6 +269,10 @@ def _run_round(state, bucket, error_mode):
             p_idx += n * rank
             q_idx += m * rank
         plan.arena_key = (p_mem.data_ptr(), q_mem.data_ptr())
+        plan.q_next = None
+        plan.q_next_ready = False
+    if need_randomize_qs:
+        plan.q_next_ready = False
     qs = plan.qs
 
     # error memory of every matrix in the table (created on first use; pointers that can move
@@ -340,9 +351,32 @@ def _run_round(state, bucket, error_mode):
         mode3 = 3 if error_mode == "conef" and plan.batched_update else 1
     else:
         mode3 = 0
-    rc = lib.conef_psgd_round_f32(items, count, mode1, mode3, float(alpha), float(state.beta) if mode3 in (2, 3) else 0.0,
-                                  eps, HASH_A, HASH_B, ws_ptr, ws_len, stream)
-    _lib.check(rc, "conef_psgd_round_f32")
+    if mode3 == 2 and state.warm_start and count and count <= 24 and os.environ.get("CONEF_ROUND_AHEAD", "1") != "0":
+        # The bucket's next round starts by orthogonalising the Q factors this round leaves
+        # (powerSGD_hook.py:496-497): a few workgroups and an idle machine.  Workgroups of this
+        # round's last launch do it instead, into a second buffer, where the kernel allows
+        # (CONEF_ROUND_AHEAD=0 keeps the reference's order, for comparisons).
+        import ctypes
+        if plan.q_next is None:
+            plan.q_next = torch.empty_like(q_mem)
+            offs, off = [], 0
+            for _, n, m, rank in work:
+                offs.append(off)
+                off += m * rank
+            plan.q_next_ptrs = (ctypes.c_void_p * count)(*[plan.q_next.data_ptr() + 4 * o for o in offs])
+            plan.made = ctypes.c_int32(0)
+            plan.q_next_ready = False
+        flags = (1 if plan.q_next_ready else 0) | 2
+        rc = lib.conef_psgd_round_ahead_f32(items, count, mode1, mode3, float(alpha), float(state.beta), eps, HASH_A,
+                                            HASH_B, plan.q_next_ptrs, flags, ctypes.byref(plan.made), ws_ptr, ws_len,
+                                            stream)
+        _lib.check(rc, "conef_psgd_round_ahead_f32")
+        plan.q_next_ready = bool(plan.made.value)
+    else:
+        plan.q_next_ready = False
+        rc = lib.conef_psgd_round_f32(items, count, mode1, mode3, float(alpha), float(state.beta) if mode3 in (2, 3) else 0.0,
+                                      eps, HASH_A, HASH_B, ws_ptr, ws_len, stream)
+        _lib.check(rc, "conef_psgd_round_f32")
     if error_mode == "topk":
         plan.topk_table = topk_sparsify_all([errs[cnt] for cnt in range(count)], state.topk_ratio, plan.topk_table)
     elif residual is not None and mode3 != 3:

@@ -886,8 +886,10 @@ struct GsBatch {
 };
 
 template <int RP, int RPT>
-__device__ __forceinline__ void gs_reg_body(float* __restrict__ a, int rows, float (&red)[2][4][RP], int r, float eps)
+__device__ __forceinline__ void gs_reg_body(float* a, int rows, float (&red)[2][4][RP], int r, float eps,
+                                            const float* src = nullptr)
 {
+    if (!src) src = a;          // in place unless the matrix is to be read from elsewhere
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int nrt = (rows + kGsRegThreads - 1) / kGsRegThreads;      // row slots in use (uniform)
     float v[RPT][RP];
@@ -897,7 +899,7 @@ __device__ __forceinline__ void gs_reg_body(float* __restrict__ a, int rows, flo
 #pragma unroll
         for (int c = 0; c < RP; ++c) v[t][c] = 0.f;
         if (t < nrt && k < rows) {
-            const float* row = a + (int64_t)k * r;
+            const float* row = src + (int64_t)k * r;
             if (RP >= 4 && r == RP) {
 #pragma unroll
                 for (int c = 0; c < RP; c += 4) ld4(row + c, &v[t][c]);
@@ -939,19 +941,34 @@ gram_schmidt_reg_kernel(GsBatch batch, int r, float eps)
 // not a launch of their own in front of the tall ones.  A workgroup runs exactly the code the
 // one-size kernel would run on its matrix.
 template <int RP>
+__device__ __forceinline__ void gs_reg_any_height(float* a, int rows, float (&red)[2][4][RP], int r, float eps,
+                                                  const float* src = nullptr)
+{
+    constexpr int kAll = kGsRegFloats / RP;
+    const int nrt = (rows + kGsRegThreads - 1) / kGsRegThreads;
+    if (nrt <= 1) gs_reg_body<RP, 1>(a, rows, red, r, eps, src);
+    else if (nrt <= 4 && kAll >= 4) gs_reg_body<RP, (kAll >= 4 ? 4 : kAll)>(a, rows, red, r, eps, src);
+    else if (nrt <= 16 && kAll >= 16) gs_reg_body<RP, (kAll >= 16 ? 16 : kAll)>(a, rows, red, r, eps, src);
+    else gs_reg_body<RP, kAll>(a, rows, red, r, eps, src);
+}
+
+template <int RP>
 __global__ void __launch_bounds__(kGsRegThreads)
 gram_schmidt_reg_mixed_kernel(GsBatch batch, int r, float eps)
 {
     __shared__ float red[2][4][RP];
-    constexpr int kAll = kGsRegFloats / RP;
-    float* a = batch.a[blockIdx.x];
-    const int rows = batch.rows[blockIdx.x];
-    const int nrt = (rows + kGsRegThreads - 1) / kGsRegThreads;
-    if (nrt <= 1) gs_reg_body<RP, 1>(a, rows, red, r, eps);
-    else if (nrt <= 4 && kAll >= 4) gs_reg_body<RP, (kAll >= 4 ? 4 : kAll)>(a, rows, red, r, eps);
-    else if (nrt <= 16 && kAll >= 16) gs_reg_body<RP, (kAll >= 16 ? 16 : kAll)>(a, rows, red, r, eps);
-    else gs_reg_body<RP, kAll>(a, rows, red, r, eps);
+    gs_reg_any_height<RP>(batch.a[blockIdx.x], batch.rows[blockIdx.x], red, r, eps);
 }
+
+// Matrices to orthogonalise out of place by workgroups that ride along in another kernel's launch.
+constexpr int kGsAheadRowSlots = 4;      // rows a thread of such a workgroup holds at most
+struct GsAhead {
+    const float* src[kPsgdBatchMax];
+    float* dst[kPsgdBatchMax];
+    int rows[kPsgdBatchMax];
+    int count, r;
+    float eps;
+};
 
 // Matrices beyond one workgroup's registers: the same register-resident scheme over up to 128
 // workgroups launched cooperatively (all resident at once).  A column step ends with every
@@ -2292,8 +2309,36 @@ psgd_residual_rowlist_batch_kernel(PsgdBatch<RowlistResidualItem<RP, FAST>> b, d
                                                           one_minus_beta, local);
 }
 
+// The same launch with a few more workgroups in front that orthogonalise the bucket's new Q factors
+// into a second buffer (Q itself is still being read by the other workgroups): the reference does
+// that at the start of the bucket's next round (powerSGD_hook.py:496-497), where it is a launch of
+// half a dozen workgroups with the machine idle around it; here it costs nothing.
 template <int RP, bool FAST>
-int pqt_sketch_group(const ConefPsgdItem* items, const std::vector<int>& members, float beta, hipStream_t s)
+__global__ void __launch_bounds__(kConefRowlistThreads)
+psgd_residual_rowlist_gs_batch_kernel(PsgdBatch<RowlistResidualItem<RP, FAST>> b, double one_minus_beta, GsAhead g)
+{
+    static_assert(kConefRowlistThreads == kGsRegThreads, "one block size for both kinds of workgroup");
+    if ((int)blockIdx.x < g.count) {
+        // at most kGsAheadRowSlots rows a thread: the taller bodies hold over a hundred values in
+        // registers, and this kernel's allocation is what every workgroup of the launch gets
+        __shared__ float red[2][4][RP];
+        if (g.rows[blockIdx.x] <= kGsRegThreads)
+            gs_reg_body<RP, 1>(g.dst[blockIdx.x], g.rows[blockIdx.x], red, g.r, g.eps, g.src[blockIdx.x]);
+        else
+            gs_reg_body<RP, kGsAheadRowSlots>(g.dst[blockIdx.x], g.rows[blockIdx.x], red, g.r, g.eps, g.src[blockIdx.x]);
+        return;
+    }
+    const int bx = (int)blockIdx.x - g.count;
+    int i = 0;
+    while (i + 1 < b.count && bx >= b.first[i + 1]) ++i;
+    const RowlistResidualItem<RP, FAST>& it = b.item[i];
+    conef_rowlist_body<float, ListPsgdResidual<RP, FAST>>(it.front, it.plan, it.cs_in, it.cs_out, it.n, it.d, it.w, it.rb,
+                                                          one_minus_beta, bx - b.first[i]);
+}
+
+template <int RP, bool FAST>
+int pqt_sketch_group(const ConefPsgdItem* items, const std::vector<int>& members, float beta, hipStream_t s,
+                     const GsAhead* ahead = nullptr)
 {
     std::vector<RowlistResidualItem<RP, FAST>> table;
     std::vector<int> blocks;
@@ -2324,13 +2369,28 @@ int pqt_sketch_group(const ConefPsgdItem* items, const std::vector<int>& members
         if (e != hipSuccess) return (int)e;
     }
     const double omb = 1. - (double)beta;
+    if (ahead && ahead->count > 0 && table.size() <= (size_t)kPsgdBatchMax) {
+        auto fused = psgd_residual_rowlist_gs_batch_kernel<RP, FAST>;
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute((const void*)fused, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return (int)e;
+        }
+        const GsAhead g = *ahead;
+        return run_batches(table, blocks, [&](const PsgdBatch<RowlistResidualItem<RP, FAST>>& bt, int grid) {
+            hipLaunchKernelGGL(fused, dim3((unsigned)(grid + g.count)), dim3(kConefRowlistThreads), lds, s, bt, omb, g);
+        });
+    }
     return run_batches(table, blocks, [&](const PsgdBatch<RowlistResidualItem<RP, FAST>>& bt, int grid) {
         hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kConefRowlistThreads), lds, s, bt, omb);
     });
 }
 
-int pqt_batch(const ConefPsgdItem* items, int count, int mode, float beta, int32_t a, int32_t b, hipStream_t s)
+// ahead: the Q factors to orthogonalise alongside (mode 2, one rank class over the whole bucket
+// only); *ahead_used says whether that was done.
+int pqt_batch(const ConefPsgdItem* items, int count, int mode, float beta, int32_t a, int32_t b, hipStream_t s,
+              const GsAhead* ahead = nullptr, bool* ahead_used = nullptr)
 {
+    if (ahead_used) *ahead_used = false;
     std::vector<char> done((size_t)count, 0);
     for (int k = 0; k < count; ++k) {
         if (done[(size_t)k]) continue;
@@ -2382,15 +2442,18 @@ int pqt_batch(const ConefPsgdItem* items, int count, int mode, float beta, int32
                     done[(size_t)j] = 1;
                 }
                 int rc = CONEF_ERR_INVALID;
+                const GsAhead* ride = (ahead && ahead->count > 0 && members.size() == (size_t)count &&
+                                       count <= kPsgdBatchMax && rank_bound(ahead->r) == rp) ? ahead : nullptr;
 #define CONEF_PQS(RP)                                                                  \
     do {                                                                               \
         if (RP >= 16) break;                                                           \
-        if (fast) rc = pqt_sketch_group<(RP < 16 ? RP : 8), true>(items, members, beta, s);  \
-        else rc = pqt_sketch_group<(RP < 16 ? RP : 8), false>(items, members, beta, s);      \
+        if (fast) rc = pqt_sketch_group<(RP < 16 ? RP : 8), true>(items, members, beta, s, ride);  \
+        else rc = pqt_sketch_group<(RP < 16 ? RP : 8), false>(items, members, beta, s, ride);      \
     } while (0)
                 CONEF_RANK_SWITCH(lead.r, CONEF_PQS)
 #undef CONEF_PQS
                 if (rc != CONEF_OK) return rc;
+                if (ride && ahead_used) *ahead_used = true;
                 continue;
             }
             int rc;
@@ -2549,11 +2612,13 @@ int conef_psgd_sketch_update_batch_f32(const ConefPsgdItem* items, int32_t count
 // (pqt_mode 0, 1, 2 as in conef_psgd_pqt_batch_f32; 3 = mode 1 followed by
 // conef_psgd_sketch_update_batch_f32 on the residuals).  The same launches as the separate calls,
 // in the same order; what it saves is the caller's trips through its foreign-function interface.
-int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, float alpha,
-                         float beta, float eps, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
-                         void* stream)
+int conef_psgd_round_ahead_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, float alpha,
+                               float beta, float eps, int32_t a, int32_t b, float* const* q_next, int32_t flags,
+                               int32_t* made, void* workspace, int64_t workspace_bytes, void* stream)
 {
+    if (made) *made = 0;
     if (count < 0 || (count > 0 && !items) || pqt_mode < 0 || pqt_mode > 3) return CONEF_ERR_INVALID;
+    if ((flags & (CONEF_ROUND_Q_READY | CONEF_ROUND_MAKE_NEXT)) && (!q_next || !made)) return CONEF_ERR_INVALID;
     if (count == 0) return CONEF_OK;
     std::vector<float*> mats((size_t)count);
     std::vector<int64_t> rows((size_t)count);
@@ -2564,9 +2629,20 @@ int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_m
         rows[(size_t)k] = items[k].m;
         ranks[(size_t)k] = items[k].r;
     }
-    int rc = conef_gram_schmidt_batch_f32(mats.data(), rows.data(), ranks.data(), count, eps, workspace, workspace_bytes, stream);
-    if (rc != CONEF_OK) return rc;
-    rc = conef_psgd_mq_batch_f32(items, count, mq_mode, alpha, a, b, workspace, workspace_bytes, stream);
+    int rc = CONEF_OK;
+    if (flags & CONEF_ROUND_Q_READY) {
+        // q_next holds this round's Q factors, orthogonalised at the end of the bucket's last round
+        std::vector<ConefPsgdItem> with_q(items, items + count);
+        for (int k = 0; k < count; ++k) {
+            if (!q_next[k]) return CONEF_ERR_INVALID;
+            with_q[(size_t)k].q = q_next[k];
+        }
+        rc = conef_psgd_mq_batch_f32(with_q.data(), count, mq_mode, alpha, a, b, workspace, workspace_bytes, stream);
+    } else {
+        rc = conef_gram_schmidt_batch_f32(mats.data(), rows.data(), ranks.data(), count, eps, workspace, workspace_bytes, stream);
+        if (rc != CONEF_OK) return rc;
+        rc = conef_psgd_mq_batch_f32(items, count, mq_mode, alpha, a, b, workspace, workspace_bytes, stream);
+    }
     if (rc != CONEF_OK) return rc;
     for (int k = 0; k < count; ++k) {
         mats[(size_t)k] = items[k].p;
@@ -2576,10 +2652,45 @@ int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_m
     if (rc != CONEF_OK) return rc;
     rc = conef_psgd_mtp_batch_f32(items, count, workspace, workspace_bytes, stream);
     if (rc != CONEF_OK) return rc;
-    rc = conef_psgd_pqt_batch_f32(items, count, pqt_mode == 3 ? 1 : pqt_mode, pqt_mode == 2 ? beta : 0.f, a, b, stream);
+    // The new Q factors orthogonalised into q_next by workgroups of the last launch: only where that
+    // launch is the residual-sketch kernel over the whole bucket and every Q fits one workgroup's
+    // registers.
+    GsAhead ahead;
+    ahead.count = 0;
+    if ((flags & CONEF_ROUND_MAKE_NEXT) && pqt_mode == 2 && count <= kPsgdBatchMax && rank_bound(items[0].r) <= 8) {
+        bool ok = true;
+        for (int k = 0; k < count && ok; ++k)
+            ok = q_next[k] && items[k].r == items[0].r && aligned16(q_next[k]) &&
+                 gs_reg_class(items[k].q, items[k].m, items[k].r) >= 0 &&
+                 items[k].m <= (int64_t)kGsAheadRowSlots * kGsRegThreads;
+        if (ok) {
+            for (int k = 0; k < count; ++k) {
+                ahead.src[k] = items[k].q;
+                ahead.dst[k] = q_next[k];
+                ahead.rows[k] = (int)items[k].m;
+            }
+            ahead.count = count;
+            ahead.r = items[0].r;
+            ahead.eps = eps;
+        }
+    }
+    bool used = false;
+    for (int k = 0; k < count; ++k)
+        if ((pqt_mode == 1 || pqt_mode == 3) && !items[k].err) return CONEF_ERR_INVALID;
+    rc = pqt_batch(items, count, pqt_mode == 3 ? 1 : pqt_mode, pqt_mode == 2 ? beta : 0.f, a, b, (hipStream_t)stream,
+                   ahead.count ? &ahead : nullptr, &used);
     if (rc != CONEF_OK) return rc;
+    if (made) *made = used ? 1 : 0;
     if (pqt_mode == 3) rc = conef_psgd_sketch_update_batch_f32(items, count, beta, a, b, stream);
     return rc;
+}
+
+int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, float alpha,
+                         float beta, float eps, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
+                         void* stream)
+{
+    return conef_psgd_round_ahead_f32(items, count, mq_mode, pqt_mode, alpha, beta, eps, a, b, nullptr, 0, nullptr,
+                                      workspace, workspace_bytes, stream);
 }
 
 // dense error feedback on the parts of a bucket that are not compressed: x += e; e = 0

@@ -294,6 +294,22 @@ int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_m
                          float beta, float eps, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
                          void* stream);
 
+/* The same round for callers that keep a second buffer per Q factor (q_next[k], [m,r] like items[k].q).
+ * The reference orthogonalises a bucket's Q factors at the start of the bucket's next round
+ * (powerSGD_hook.py:496-497), a launch of a few workgroups with the machine idle around it.  Here
+ * flags & CONEF_ROUND_MAKE_NEXT asks for that to be done at the end of this round instead, out of
+ * place into q_next, by workgroups that ride along in the round's last launch; *made tells whether it
+ * was (only for pqt_mode 2 over a bucket of at most 24 matrices of one rank <= 8 whose Q factors have
+ * at most 1024 rows).  items[k].q keeps what the reference keeps there.  In the next round
+ * flags & CONEF_ROUND_Q_READY says q_next holds the orthogonal Q factors: the first step is left out
+ * and P = M Q reads them.  Same arithmetic on the same values either way.  No counterpart in the
+ * reference's interface. */
+#define CONEF_ROUND_Q_READY 1
+#define CONEF_ROUND_MAKE_NEXT 2
+int conef_psgd_round_ahead_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, float alpha,
+                               float beta, float eps, int32_t a, int32_t b, float* const* q_next, int32_t flags,
+                               int32_t* made, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Dense error feedback on a stretch of the bucket that is not compressed: x += err; err = 0
  * (the copy-minus-result of powerSGD_hook.py:558 is exactly zero there). */
 int conef_ef_passthrough_f32(float* x, float* err, int64_t count, void* stream);

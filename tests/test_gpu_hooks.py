@@ -586,6 +586,73 @@ def test_powersgd_rounds_on_side_streams(mode):
         np.testing.assert_array_equal(x, y)
 
 
+@pytest.mark.parametrize("rank,ss", [(8, 0.1), (4, 0.2), (2, 0.5)])
+def test_q_factors_orthogonalised_by_the_last_launch(monkeypatch, oracle, rank, ss):
+    """Where a bucket's Q factors are short enough, workgroups of the round's last launch
+    orthogonalise the new Q into a second buffer and the next round starts from it instead of
+    running Gram-Schmidt first.  Same kernels' arithmetic on the same values: bucket, P, Q and
+    sketches equal the reference order's bit for bit, step after step, also across a bucket that
+    does not qualify (a Q factor of 4096 rows) and a checkpoint."""
+    import io
+    from conef_amd.powerSGD_hook import PowerSGDState, powerSGD_hook
+    buckets = [[(1024, 256), (256,), (256, 1024), (640, 768)], [(4096, 128), (128, 4096)], [(64, 576), (10, 64), (33, 40)]]
+
+    def make():
+        st = PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, use_error_compression=True,
+                           sketch_size=ss, beta=0.9)
+        st.iter = 2
+        return st
+
+    def steps(st, first, count):
+        outs = []
+        for step in range(first, first + count):
+            gen = torch.Generator().manual_seed(300 + step)
+            flats = [(torch.randn(numel_of(b), generator=gen) * 1e-3).cuda() for b in buckets]
+            futs = [powerSGD_hook(st, FakeGradBucket(f, b, index=i, is_last=i == len(buckets) - 1))
+                    for i, (f, b) in enumerate(zip(flats, buckets))]
+            outs.append([to_np(f.wait()) for f in futs])
+        torch.cuda.synchronize()
+        return outs
+
+    def snapshot(st):
+        keep = []
+        for i in range(len(buckets)):
+            keep += [to_np(st.p_memory_dict[i]), to_np(st.q_memory_dict[i])] + [to_np(cs.cs) for cs in st.error_dict[i].values()]
+        return keep
+
+    monkeypatch.setenv("CONEF_ROUND_AHEAD", "0")
+    plain = make()
+    outs_plain = steps(plain, 0, 4)
+    monkeypatch.setenv("CONEF_ROUND_AHEAD", "1")
+    ahead = make()
+    outs_ahead = steps(ahead, 0, 4)
+    used = [ahead.round_cache[i].q_next_ready for i in range(len(buckets))]
+    assert used[0] and not used[1], used           # the second bucket has a Q factor of 4096 rows
+    for a, b in zip(outs_plain, outs_ahead):
+        for x, y in zip(a, b):
+            np.testing.assert_array_equal(x, y)
+    for x, y in zip(snapshot(plain), snapshot(ahead)):
+        np.testing.assert_array_equal(x, y)
+    # the second buffer holds the orthogonalised form of the stored Q
+    plan = ahead.round_cache[0]
+    raw, nxt, off = to_np(ahead.q_memory_dict[0]), to_np(plan.q_next), 0
+    for _, n, m, r in plan.work:
+        want = raw[off:off + m * r].reshape(m, r).copy()
+        oracle.gram_schmidt(want, 0.0)
+        assert_close(nxt[off:off + m * r].reshape(m, r), want, what="orthogonalised Q of a [%d,%d] matrix" % (n, m))
+        off += m * r
+    # a restored state has no second buffer yet and orthogonalises in the round: same results
+    buf = io.BytesIO()
+    torch.save(ahead.state_dict(), buf)
+    buf.seek(0)
+    resumed = make()
+    resumed.load_state_dict(torch.load(buf, weights_only=False))
+    for a, b, c in zip(steps(plain, 4, 2), steps(ahead, 4, 2), steps(resumed, 4, 2)):
+        for x, y, z in zip(a, b, c):
+            np.testing.assert_array_equal(x, y)
+            np.testing.assert_array_equal(x, z)
+
+
 def test_powersgd_state_errors_and_warmup():
     from conef_amd.powerSGD_hook import PowerSGDState, _should_compress, powerSGD_hook
     with pytest.raises(ValueError, match="Expect `start_powerSGD_iter` > 1"):
