@@ -351,7 +351,8 @@ def _run_round(state, bucket, error_mode):
         mode3 = 3 if error_mode == "conef" and plan.batched_update else 1
     else:
         mode3 = 0
-    if mode3 == 2 and state.warm_start and count and count <= 24 and os.environ.get("CONEF_ROUND_AHEAD", "1") != "0":
+    if (mode3 in (0, 1, 2) and state.matrix_approximation_rank <= 8 and state.warm_start and count and count <= 24
+            and os.environ.get("CONEF_ROUND_AHEAD", "1") != "0"):
         # The bucket's next round starts by orthogonalising the Q factors this round leaves
         # (powerSGD_hook.py:496-497): a few workgroups and an idle machine.  Workgroups of this
         # round's last launch do it instead, into a second buffer, where the kernel allows
@@ -367,7 +368,7 @@ def _run_round(state, bucket, error_mode):
             plan.made = ctypes.c_int32(0)
             plan.q_next_ready = False
         flags = (1 if plan.q_next_ready else 0) | 2
-        rc = lib.conef_psgd_round_ahead_f32(items, count, mode1, mode3, float(alpha), float(state.beta), eps, HASH_A,
+        rc = lib.conef_psgd_round_ahead_f32(items, count, mode1, mode3, float(alpha), float(state.beta) if mode3 == 2 else 0.0, eps, HASH_A,
                                             HASH_B, plan.q_next_ptrs, flags, ctypes.byref(plan.made), ws_ptr, ws_len,
                                             stream)
         _lib.check(rc, "conef_psgd_round_ahead_f32")

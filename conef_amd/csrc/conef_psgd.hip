@@ -2336,6 +2336,29 @@ psgd_residual_rowlist_gs_batch_kernel(PsgdBatch<RowlistResidualItem<RP, FAST>> b
                                                           one_minus_beta, bx - b.first[i]);
 }
 
+// The dense M = P Q^T kernel (with or without the residual written out) with the same riders.
+template <int RP, int MODE, bool FAST>
+__global__ void __launch_bounds__(256)
+psgd_pqt_gs_batch_kernel(PsgdBatch<PqtItem> b, GsAhead g)
+{
+    static_assert(kGsRegThreads == 256, "one block size for both kinds of workgroup");
+    if ((int)blockIdx.x < g.count) {
+        __shared__ float red[2][4][RP];
+        if (g.rows[blockIdx.x] <= kGsRegThreads)
+            gs_reg_body<RP, 1>(g.dst[blockIdx.x], g.rows[blockIdx.x], red, g.r, g.eps, g.src[blockIdx.x]);
+        else
+            gs_reg_body<RP, kGsAheadRowSlots>(g.dst[blockIdx.x], g.rows[blockIdx.x], red, g.r, g.eps, g.src[blockIdx.x]);
+        return;
+    }
+    const int bx = (int)blockIdx.x - g.count;
+    int i = 0;
+    while (i + 1 < b.count && bx >= b.first[i + 1]) ++i;
+    const PqtItem& it = b.item[i];
+    const int local = bx - b.first[i];
+    psgd_pqt_body<RP, MODE, FAST>(it.x, it.err, it.p, it.q, it.n, it.m, it.r, it.rows_per_slab, local % it.col_tiles,
+                                  local / it.col_tiles);
+}
+
 template <int RP, bool FAST>
 int pqt_sketch_group(const ConefPsgdItem* items, const std::vector<int>& members, float beta, hipStream_t s,
                      const GsAhead* ahead = nullptr)
@@ -2488,9 +2511,18 @@ int pqt_batch(const ConefPsgdItem* items, int count, int mode, float beta, int32
             done[(size_t)j] = 1;
         }
         int rc = CONEF_OK;
+        const GsAhead* ride = (ahead && ahead->count > 0 && table.size() == (size_t)count && count <= kPsgdBatchMax &&
+                               rank_bound(ahead->r) == rp) ? ahead : nullptr;
+        GsAhead g;
+        g.count = 0;
+        if (ride) g = *ride;
 #define CONEF_PQB_GO(RP, MODE, F)                                                                                  \
     run_batches(table, blocks, [&](const PsgdBatch<PqtItem>& bt, int grid) {                                       \
-        hipLaunchKernelGGL((psgd_pqt_batch_kernel<RP, MODE, F>), dim3((unsigned)grid), dim3(256), 0, s, bt);       \
+        if (ride)                                                                                                  \
+            hipLaunchKernelGGL((psgd_pqt_gs_batch_kernel<RP, MODE, F>), dim3((unsigned)(grid + g.count)), dim3(256), 0, s, \
+                               bt, g);                                                                             \
+        else                                                                                                       \
+            hipLaunchKernelGGL((psgd_pqt_batch_kernel<RP, MODE, F>), dim3((unsigned)grid), dim3(256), 0, s, bt);   \
     })
 #define CONEF_PQB(RP)                                                          \
     do {                                                                       \
@@ -2507,6 +2539,7 @@ int pqt_batch(const ConefPsgdItem* items, int count, int mode, float beta, int32
 #undef CONEF_PQB
 #undef CONEF_PQB_GO
         if (rc != CONEF_OK) return rc;
+        if (ride && ahead_used) *ahead_used = true;
     }
     return CONEF_OK;
 }
@@ -2653,11 +2686,10 @@ int conef_psgd_round_ahead_f32(const ConefPsgdItem* items, int32_t count, int32_
     rc = conef_psgd_mtp_batch_f32(items, count, workspace, workspace_bytes, stream);
     if (rc != CONEF_OK) return rc;
     // The new Q factors orthogonalised into q_next by workgroups of the last launch: only where that
-    // launch is the residual-sketch kernel over the whole bucket and every Q fits one workgroup's
-    // registers.
+    // launch covers the whole bucket (one rank, at most 8) and every Q factor is short.
     GsAhead ahead;
     ahead.count = 0;
-    if ((flags & CONEF_ROUND_MAKE_NEXT) && pqt_mode == 2 && count <= kPsgdBatchMax && rank_bound(items[0].r) <= 8) {
+    if ((flags & CONEF_ROUND_MAKE_NEXT) && pqt_mode <= 2 && count <= kPsgdBatchMax && rank_bound(items[0].r) <= 8) {
         bool ok = true;
         for (int k = 0; k < count && ok; ++k)
             ok = q_next[k] && items[k].r == items[0].r && aligned16(q_next[k]) &&

@@ -299,7 +299,7 @@ int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_m
  * (powerSGD_hook.py:496-497), a launch of a few workgroups with the machine idle around it.  Here
  * flags & CONEF_ROUND_MAKE_NEXT asks for that to be done at the end of this round instead, out of
  * place into q_next, by workgroups that ride along in the round's last launch; *made tells whether it
- * was (only for pqt_mode 2 over a bucket of at most 24 matrices of one rank <= 8 whose Q factors have
+ * was (only for pqt_mode 0..2 over a bucket of at most 24 matrices of one rank <= 8 whose Q factors have
  * at most 1024 rows).  items[k].q keeps what the reference keeps there.  In the next round
  * flags & CONEF_ROUND_Q_READY says q_next holds the orthogonal Q factors: the first step is left out
  * and P = M Q reads them.  Same arithmetic on the same values either way.  No counterpart in the

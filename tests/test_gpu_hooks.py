@@ -586,20 +586,29 @@ def test_powersgd_rounds_on_side_streams(mode):
         np.testing.assert_array_equal(x, y)
 
 
-@pytest.mark.parametrize("rank,ss", [(8, 0.1), (4, 0.2), (2, 0.5)])
-def test_q_factors_orthogonalised_by_the_last_launch(monkeypatch, oracle, rank, ss):
+@pytest.mark.parametrize("rank,ss,mode", [(8, 0.1, "conef"), (4, 0.2, "conef"), (2, 0.5, "conef"), (8, 0.1, "ef"),
+                                          (4, 0.1, "topk"), (8, 0.1, "plain")])
+def test_q_factors_orthogonalised_by_the_last_launch(monkeypatch, oracle, rank, ss, mode):
     """Where a bucket's Q factors are short enough, workgroups of the round's last launch
     orthogonalise the new Q into a second buffer and the next round starts from it instead of
     running Gram-Schmidt first.  Same kernels' arithmetic on the same values: bucket, P, Q and
     sketches equal the reference order's bit for bit, step after step, also across a bucket that
     does not qualify (a Q factor of 4096 rows) and a checkpoint."""
     import io
-    from conef_amd.powerSGD_hook import PowerSGDState, powerSGD_hook
+    from conef_amd.hPowerSGD_hook import hPowerSGDState, hpowerSGD_hook
+    from conef_amd.powerSGD_hook import PowerSGDState
+    from conef_amd.powerSGD_hook import powerSGD_hook as plain_hook
     buckets = [[(1024, 256), (256,), (256, 1024), (640, 768)], [(4096, 128), (128, 4096)], [(64, 576), (10, 64), (33, 40)]]
+    powerSGD_hook = hpowerSGD_hook if mode == "topk" else plain_hook
 
     def make():
-        st = PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, use_error_compression=True,
-                           sketch_size=ss, beta=0.9)
+        if mode == "topk":
+            st = hPowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, use_error_compression=True,
+                                topk_ratio=0.4)
+        else:
+            st = PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2,
+                               use_error_feedback=mode != "plain", use_error_compression=mode == "conef",
+                               sketch_size=ss, beta=0.9)
         st.iter = 2
         return st
 
@@ -617,7 +626,12 @@ def test_q_factors_orthogonalised_by_the_last_launch(monkeypatch, oracle, rank, 
     def snapshot(st):
         keep = []
         for i in range(len(buckets)):
-            keep += [to_np(st.p_memory_dict[i]), to_np(st.q_memory_dict[i])] + [to_np(cs.cs) for cs in st.error_dict[i].values()]
+            keep += [to_np(st.p_memory_dict[i]), to_np(st.q_memory_dict[i])]
+            err = st.error_dict.get(i)
+            if isinstance(err, dict):
+                keep += [to_np(e.cs if hasattr(e, "cs") else e) for e in err.values()]
+            elif err is not None:
+                keep.append(to_np(err))
         return keep
 
     monkeypatch.setenv("CONEF_ROUND_AHEAD", "0")
