@@ -66,6 +66,15 @@ def test_argument_validation_without_gpu(lib):
     assert lib.conef_topk_sparsify_f32(1, 100, 10, 0, 0, 0) == -1               # no workspace
     assert lib.conef_topk_sparsify_f32(1, 100, 100, 0, 0, 0) == 0               # k >= numel: nothing to do
     assert lib.conef_topk_workspace_bytes(1 << 20) >= 4 * 1024
+    # the round that orthogonalises the next round's Q factors: its flags need the second buffers and the answer slot
+    from conef_amd import _lib
+    items = (_lib.PsgdItem * 1)()
+    made = ctypes.c_int32(7)
+    assert lib.conef_psgd_round_ahead_f32(items, 1, 0, 0, 0.0, 0.0, 0.0, 1, 1, None, 2, ctypes.byref(made), 0, 0, 0) == -1
+    assert made.value == 0
+    assert lib.conef_psgd_round_ahead_f32(items, 1, 0, 0, 0.0, 0.0, 0.0, 1, 1, None, 1, None, 0, 0, 0) == -1
+    assert lib.conef_psgd_round_ahead_f32(items, 0, 0, 0, 0.0, 0.0, 0.0, 1, 1, None, 0, None, 0, 0, 0) == 0     # empty bucket
+    assert lib.conef_psgd_round_ahead_f32(items, 1, 0, 4, 0.0, 0.0, 0.0, 1, 1, None, 0, None, 0, 0, 0) == -1    # pqt_mode
     # shapes: short rows may update in place, the flat 25 MB bucket may not
     assert lib.conef_cs_update_inplace_ok(640, 5760, 1152) == 1
     assert lib.conef_cs_update_inplace_ok(5, 1_300_000, 130_000) == 0
