@@ -250,6 +250,23 @@ def main():
         hook_steps(args, results)
     if not args.json:
         print("done: %d cases" % len(results))
+    teardown()
+
+
+def teardown():
+    """Returns every piece of device memory and every stream this process created while the HIP
+    runtime is still whole: waits for the device, drops the library's shared pools, then gives
+    torch's cached blocks back to the runtime.  Under a profiler that finalises itself in an exit
+    handler, whatever is still allocated when the interpreter has gone is freed after the tool."""
+    import gc
+
+    import torch
+    import conef_amd
+    torch.cuda.synchronize()
+    conef_amd.release()
+    gc.collect()
+    torch.cuda.empty_cache()
+    torch.cuda.synchronize()
 
 
 def hook_steps(args, results):
@@ -382,6 +399,7 @@ def hook_steps(args, results):
         else:
             print("%-58s %8.3f ms/step wall  %8.3f ms gpu  %8.1f MB gradient in %2d buckets  %7.1f GB/s of gradient" % (
                 name, wall, gpu, rec["gradient_MB"], len(buckets), rec["gradient_GBs"]), flush=True)
+        del state, hook, fakes, grads, step        # the case's device state goes before the next case (and before exit)
 
 
 if __name__ == "__main__":

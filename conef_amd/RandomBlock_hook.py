@@ -5,7 +5,8 @@ arguments, defaults, fields and error messages (:60-115), same ``RandomBlock_hoo
 contract (:138-295).  What differs is how a step executes: for each >=2-D gradient the reference
 issues a query kernel, a clone, slice copies, memsets, an update kernel, a zero_ and copies back;
 here one fused gfx950 kernel reads the gradient once and leaves payload, decompressed gradient and
-new error state behind (``conef_randblock_conef_step_f32`` / ``conef_randblock_ef_step_f32``).
+new error state behind, and all tensors of a bucket go through it in ONE foreign call
+(``conef_randblock_step_batch_f32``) from a table that is built once per bucket.
 """
 import logging
 
@@ -16,7 +17,7 @@ import torch.distributed as dist
 from . import _bucket
 from . import _lib
 from ._checkpoint import Checkpointable
-from .compressors.CountSketch import DenseCS
+from .compressors.CountSketch import HASH_A, HASH_B, DenseCS
 
 
 class RandomBlockState(Checkpointable):
@@ -46,6 +47,7 @@ class RandomBlockState(Checkpointable):
         "compression_stats_logging_frequency",
         "next_stats_report",
         "compressed_tensor_memory",
+        "round_cache",
     ]
 
     def __init__(
@@ -83,6 +85,7 @@ class RandomBlockState(Checkpointable):
         self.compression_stats_logging_frequency = max(1, compression_stats_logging_frequency)
         self.next_stats_report = 0
         self.compressed_tensor_memory = {}
+        self.round_cache = {}     # bucket index -> launch table (derived data, never checkpointed)
 
     def maybe_increase_iter(self, bucket):
         # the last bucket to be reduced closes an iteration
@@ -101,6 +104,42 @@ class RandomBlockState(Checkpointable):
 
 def _block_size(state, numel):
     return max(1, int(state.compression_ratio * numel))      # RandomBlock_hook.py:207,216
+
+
+class _BucketTable:
+    """What a bucket's step needs, worked out once: the >= 2-D gradients as matrices, their block
+    sizes, payload slices and the item table the batch entry point reads.  Rebuilt when the
+    bucket's buffer or layout changes."""
+    __slots__ = ("key", "shapes", "matrices", "uncompressed", "numels", "blocks", "offsets", "items", "count")
+
+
+def _build_table(state, grads, shapes, key, device, bucket_index, errors):
+    t = _BucketTable()
+    t.key, t.shapes = key, shapes
+    t.matrices = [g.view(g.shape[0], -1) for g in grads if g.ndimension() > 1]
+    t.uncompressed = [g for g in grads if g.ndimension() <= 1]
+    t.numels = [m.numel() for m in t.matrices]
+    t.blocks = [_block_size(state, n) for n in t.numels]
+    t.count = len(t.matrices)
+    for cnt, matrix in enumerate(t.matrices):
+        if len(errors) <= cnt:
+            if state.use_error_compression:
+                errors.append(DenseCS(matrix.shape[0], matrix.shape[1], state.sketch_size, device=device))
+            else:
+                errors.append(torch.zeros_like(matrix))
+    if bucket_index not in state.compressed_tensor_memory:
+        state.compressed_tensor_memory[bucket_index] = torch.empty(sum(t.blocks), dtype=torch.float32, device=device)
+    payload_all = state.compressed_tensor_memory[bucket_index]
+    t.items = (_lib.RandBlockItem * max(t.count, 1))()
+    t.offsets, idx = [], 0
+    for cnt, (matrix, block) in enumerate(zip(t.matrices, t.blocks)):
+        it = t.items[cnt]
+        it.x = matrix.data_ptr()
+        it.payload = payload_all.data_ptr() + 4 * idx
+        it.n, it.m, it.block = matrix.shape[0], matrix.shape[1], block
+        t.offsets.append(idx)
+        idx += block
+    return t
 
 
 def RandomBlock_hook(state: RandomBlockState, bucket) -> torch.futures.Future[torch.Tensor]:
@@ -123,41 +162,51 @@ def RandomBlock_hook(state: RandomBlockState, bucket) -> torch.futures.Future[to
         raise KeyError(bucket_index)
     errors = state.error_dict.setdefault(bucket_index, [])
 
-    matrices, uncompressed = [], []
-    for tensor in _bucket.gradients(bucket):
-        if tensor.ndimension() > 1:
-            matrices.append(tensor.view(tensor.shape[0], -1))
-        else:
-            uncompressed.append(tensor)
-
-    for cnt, matrix in enumerate(matrices):
-        if len(errors) <= cnt:
-            if state.use_error_compression:
-                errors.append(DenseCS(matrix.shape[0], matrix.shape[1], state.sketch_size, device=device))
-            else:
-                errors.append(torch.zeros_like(matrix))
-
-    if bucket_index not in state.compressed_tensor_memory:
-        total = sum(_block_size(state, m.numel()) for m in matrices)
-        state.compressed_tensor_memory[bucket_index] = torch.empty(total, dtype=torch.float32, device=device)
-    payload_all = state.compressed_tensor_memory[bucket_index]
+    grads = _bucket.gradients(bucket)
+    shapes = [g.shape for g in grads]
+    payload_all = state.compressed_tensor_memory.get(bucket_index)
+    key = (input_tensor.data_ptr(), input_tensor.numel(), bool(state.use_error_compression), state.compression_ratio,
+           payload_all.data_ptr() if payload_all is not None else 0)
+    table = state.round_cache.get(bucket_index)
+    if table is None or table.key != key or table.shapes != shapes or len(errors) < table.count:
+        table = _build_table(state, grads, shapes, key, device, bucket_index, errors)
+        payload_all = state.compressed_tensor_memory[bucket_index]
+        table.key = key[:4] + (payload_all.data_ptr(),)
+        state.round_cache[bucket_index] = table
+    items, count = table.items, table.count
 
     alpha = 1 - state.beta          # python double, rounded to fp32 at the boundary (reference :190)
-    spans, idx = [], 0
-    for matrix, error in zip(matrices, errors):
-        numel = matrix.numel()
-        block = _block_size(state, numel)
-        start = int(state.rng.choice(numel))                   # one draw per tensor, in bucket order (:218)
-        payload = payload_all[idx: idx + block]
-        n, m = matrix.shape
+    starts = []
+    randint = state.rng.randint     # RandomState.choice(n) of an int n draws randint(0, n): same stream (:218)
+    written = []
+    for cnt in range(count):
+        it = items[cnt]
+        start = int(randint(0, table.numels[cnt]))             # one draw per tensor, in bucket order (:218)
+        it.start = start
+        starts.append(start)
+        error = errors[cnt]
         if state.use_error_compression:
-            error.randblock_step(matrix, payload, start, block, alpha, state.beta)
+            plan = error.plan()
+            it.w = error.range
+            it.cs_in = error.cs.data_ptr()
+            if plan is not None:
+                # the binned step reads the old sketch while it writes the new one
+                out = error.cs if plan.in_place else error.spare_buffer()
+                it.plan_host, it.plan_dev = plan.host_ptr, plan.device.data_ptr()
+                it.staging = None if plan.in_place else plan.workspace.data_ptr()
+            else:
+                out = error.next_buffer()
+                it.plan_host = it.plan_dev = it.staging = None
+            it.cs_out = out.data_ptr()
+            written.append(out)
         else:
-            rc = lib.conef_randblock_ef_step_f32(matrix.data_ptr(), error.data_ptr(), payload.data_ptr(), numel,
-                                                 start, block, stream)
-            _lib.check(rc, "conef_randblock_ef_step_f32")
-        spans.append((matrix, start, block, idx))
-        idx += block
+            it.err = error.data_ptr()
+    if count:
+        rc = lib.conef_randblock_step_batch_f32(items, count, 2 if state.use_error_compression else 1, float(alpha),
+                                                float(state.beta), HASH_A, HASH_B, stream)
+        _lib.check(rc, "conef_randblock_step_batch_f32")
+    for error, out in zip(errors, written):
+        error.commit(out)
 
     if world_size == 1:
         # every all-reduce is the identity: the fused kernels already left zeros + block in place
@@ -166,6 +215,8 @@ def RandomBlock_hook(state: RandomBlockState, bucket) -> torch.futures.Future[to
 
     # More than one rank (not exercised on the single-GPU boxes this was developed on): average the
     # small tensors and the payload, then put the averaged block back.
+    uncompressed = table.uncompressed
+    spans = [(m, st, bl, off) for m, st, bl, off in zip(table.matrices, starts, table.blocks, table.offsets)]
     flat_small = (torch.cat([t.view(-1) for t in uncompressed]) if uncompressed
                   else torch.tensor([], device=device, dtype=input_tensor.dtype))
     fut = dist.all_reduce(flat_small, group=group, async_op=True).get_future()

@@ -2,8 +2,9 @@
 
 Drop-in for the reference's communication/UnbiasedRandomBlock_hook.py (state :12-95, hook :98-219):
 the kept block is divided by block/numel so the compressed gradient is unbiased; there is no error
-state.  One fused gfx950 kernel per >=2-D gradient writes the scaled payload and the decompressed
-gradient (``conef_randblock_unbiased_step_f32``).
+state.  One fused gfx950 kernel writes the scaled payload and the decompressed gradient of every
+>=2-D gradient of a bucket (``conef_randblock_step_batch_f32``, mode 0: one foreign call and one
+launch per bucket, from a table built once).
 """
 import logging
 
@@ -29,6 +30,7 @@ class UnbiasedRandomBlockState(Checkpointable):
         "compression_stats_logging_frequency",
         "next_stats_report",
         "compressed_tensor_memory",
+        "round_cache",
     ]
 
     def __init__(
@@ -52,6 +54,7 @@ class UnbiasedRandomBlockState(Checkpointable):
         self.compression_stats_logging_frequency = max(1, compression_stats_logging_frequency)
         self.next_stats_report = 0
         self.compressed_tensor_memory = {}
+        self.round_cache = {}     # bucket index -> launch table (derived data, never checkpointed)
 
     def maybe_increase_iter(self, bucket):
         if _bucket.is_last(bucket):
@@ -74,27 +77,43 @@ def UnbiasedRandomBlock_hook(state: UnbiasedRandomBlockState, bucket) -> torch.f
     device = input_tensor.device
     bucket_index = _bucket.index(bucket)
 
-    tensors, uncompressed = [], []
-    for tensor in _bucket.gradients(bucket):
-        (tensors if tensor.ndimension() > 1 else uncompressed).append(tensor)
-
-    blocks = [max(1, int(state.compression_ratio * t.nelement())) for t in tensors]
-    if bucket_index not in state.compressed_tensor_memory:
-        state.compressed_tensor_memory[bucket_index] = torch.empty(sum(blocks), dtype=torch.float32,
-                                                                   device=device)
+    grads = _bucket.gradients(bucket)
+    shapes = [g.shape for g in grads]
+    payload_all = state.compressed_tensor_memory.get(bucket_index)
+    key = (input_tensor.data_ptr(), input_tensor.numel(), state.compression_ratio,
+           payload_all.data_ptr() if payload_all is not None else 0)
+    table = state.round_cache.get(bucket_index)
+    if table is None or table[0] != key or table[1] != shapes:
+        # worked out once per bucket: the >= 2-D gradients, their block sizes and the item table
+        tensors = [g for g in grads if g.ndimension() > 1]
+        uncompressed = [g for g in grads if g.ndimension() <= 1]
+        numels = [t.nelement() for t in tensors]
+        blocks = [max(1, int(state.compression_ratio * n)) for n in numels]
+        if payload_all is None:
+            payload_all = torch.empty(sum(blocks), dtype=torch.float32, device=device)
+            state.compressed_tensor_memory[bucket_index] = payload_all
+        items = (_lib.RandBlockItem * max(len(tensors), 1))()
+        offsets, idx = [], 0
+        for it, tensor, numel, block in zip(items, tensors, numels, blocks):
+            it.x, it.payload = tensor.data_ptr(), payload_all.data_ptr() + 4 * idx
+            it.n, it.m, it.block = tensor.shape[0], numel // tensor.shape[0], block     # prob = block / numel is formed in the library (:155)
+            offsets.append(idx)
+            idx += block
+        table = (key[:3] + (payload_all.data_ptr(),), shapes, tensors, uncompressed, numels, blocks, offsets, items)
+        state.round_cache[bucket_index] = table
+    _, _, tensors, uncompressed, numels, blocks, offsets, items = table
     payload_all = state.compressed_tensor_memory[bucket_index]
 
-    spans, idx = [], 0
-    for tensor, block in zip(tensors, blocks):
-        numel = tensor.nelement()
-        prob = block / numel                                    # :155
-        start = int(state.rng.choice(numel))                    # :157
-        payload = payload_all[idx: idx + block]
-        rc = lib.conef_randblock_unbiased_step_f32(tensor.data_ptr(), payload.data_ptr(), numel, start, block,
-                                                   float(prob), stream)
-        _lib.check(rc, "conef_randblock_unbiased_step_f32")
-        spans.append((tensor, start, block, idx))
-        idx += block
+    starts = []
+    randint = state.rng.randint     # RandomState.choice(n) of an int n draws randint(0, n): same stream (:157)
+    for it, numel in zip(items, numels):
+        start = int(randint(0, numel))                          # :157
+        it.start = start
+        starts.append(start)
+    if tensors:
+        rc = lib.conef_randblock_step_batch_f32(items, len(tensors), 0, 0.0, 0.0, 0, 0, stream)
+        _lib.check(rc, "conef_randblock_step_batch_f32")
+    spans = list(zip(tensors, starts, blocks, offsets))
 
     if world_size == 1:
         state.maybe_increase_iter(bucket)

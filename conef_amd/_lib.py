@@ -76,12 +76,20 @@ SIGNATURES = {
     "conef_topk_sparsify_f32": [_P, _I64, _I64, _P, _I64, _P],
     "conef_topk_batch_workspace_bytes": [_P, _I32],
     "conef_topk_sparsify_batch_f32": [_P, _P, _P, _I32, _P, _I64, _P],
+    "conef_randblock_step_batch_f32": [_P, _I32, _I32, _F32, _F32, _I32, _I32, _P],
 }
 
 class PsgdItem(ctypes.Structure):
     """ConefPsgdItem of include/conef_hip.h: one matrix of a bucket for the batch entry points."""
     _fields_ = [("x", _P), ("err", _P), ("cs", _P), ("plan_host", _P), ("plan_dev", _P), ("p", _P), ("q", _P),
                 ("n", _I64), ("m", _I64), ("r", _I32), ("w", _I32)]
+
+
+class RandBlockItem(ctypes.Structure):
+    """ConefRandBlockItem of include/conef_hip.h: one tensor of a bucket for conef_randblock_step_batch_f32."""
+    _fields_ = [("x", _P), ("err", _P), ("cs_in", _P), ("cs_out", _P), ("payload", _P), ("plan_host", _P),
+                ("plan_dev", _P), ("staging", _P), ("n", _I64), ("m", _I64), ("start", _I64), ("block", _I64),
+                ("w", _I32), ("reserved", _I32)]
 
 
 _RETURNS_I64 = ("conef_topk_workspace_bytes", "conef_topk_batch_workspace_bytes", "conef_plan_bytes",

@@ -9,11 +9,13 @@ import numpy as np
 import torch
 
 from . import _lib
+from . import _pools
 
 
 class SketchPlan:
-    """plan bytes on the host (read for launch geometry), the same bytes on the device, and the
-    staging buffer the two passes hand records through."""
+    """plan bytes on the host (read for launch geometry) and the same bytes on the device.  Plans
+    are immutable: ``SketchPlan.shared`` hands every sketch of one shape on a device the same
+    object.  The staging buffer of a binned plan is not part of it (``workspace``)."""
 
     def __init__(self, n, d, w, a, b, device, chunk_cols=0, bin_buckets=0, sign_seeds=None):
         """``sign_seeds``: (sa, sb) of the sign hash; None means the single-hash sketch's (a + 2, b + 3)."""
@@ -27,10 +29,27 @@ class SketchPlan:
                                               bin_buckets)
         _lib.check(rc, "conef_plan_build_host_seeded")
         self.device = torch.from_numpy(self.host).to(device)
-        ws = lib.conef_plan_workspace_bytes(self.host.ctypes.data)
-        self.workspace = torch.empty(max(ws, 16), dtype=torch.uint8, device=device)
+        self.workspace_bytes = int(lib.conef_plan_workspace_bytes(self.host.ctypes.data))
         self.kind = lib.conef_plan_kind(self.host.ctypes.data)
         self.key = (n, d, w, a, b)
+
+    @classmethod
+    def shared(cls, n, d, w, a, b, device, chunk_cols=0, bin_buckets=0, sign_seeds=None):
+        """The process-wide plan for this shape, seeds, tiling and device (built on first use);
+        raises ValueError when the shape has none."""
+        device = torch.device(device)
+        if device.type == "cuda" and device.index is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        sa, sb = sign_seeds if sign_seeds is not None else (a + 2, b + 3)
+        key = (int(n), int(d), int(w), int(a), int(b), int(sa), int(sb), int(chunk_cols), int(bin_buckets), device)
+        return _pools.plan(key, lambda: cls(n, d, w, a, b, device, chunk_cols, bin_buckets, sign_seeds))
+
+    @property
+    def workspace(self):
+        """Staging buffer of a binned plan for work on torch's current stream: one buffer per
+        (device, stream), shared by every sketch, live only inside a call."""
+        dev = self.device.device
+        return _pools.staging(dev, torch.cuda.current_stream(dev).cuda_stream, max(self.workspace_bytes, 16))
 
     @property
     def host_ptr(self):

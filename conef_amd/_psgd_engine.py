@@ -13,7 +13,7 @@ import os
 import torch
 import torch.distributed as dist
 
-from . import _bucket, _lib
+from . import _bucket, _lib, _pools
 from .compressors.CountSketch import HASH_A, HASH_B, DenseCS
 
 
@@ -52,31 +52,9 @@ def orthogonalize_all(matrices, epsilon, ws_ptr, ws_len, stream):
     _lib.check(rc, "conef_gram_schmidt_batch_f32")
 
 
-_WORKSPACES = {}
-
-
-def _workspace(device, stream, nbytes):
-    """Device scratch for sums that cross workgroups: one buffer per (device, stream), grown on
-    demand.  Kernels that use it are ordered by that stream."""
-    key = (device, stream)
-    ws = _WORKSPACES.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
-        _WORKSPACES[key] = ws
-    return ws
-
-
-_SCRATCH = {}
-
-
-def _scratch_f32(device, stream, numel):
-    """fp32 scratch for a residual that only lives between two launches on ``stream``."""
-    key = (device, stream)
-    buf = _SCRATCH.get(key)
-    if buf is None or buf.numel() < numel:
-        buf = torch.empty(numel, dtype=torch.float32, device=device)
-        _SCRATCH[key] = buf
-    return buf
+# one buffer per (device, stream), grown on demand; held and released by conef_amd._pools
+_workspace = _pools.workspace
+_scratch_f32 = _pools.scratch_f32
 
 
 def topk_sparsify(err, topk_ratio, workspace=None):
@@ -175,17 +153,7 @@ def _build_round(state, grads, shapes, key, error_mode):
     return plan
 
 
-_SIDE_STREAMS = {}
-
-
-def _side_stream(device, bucket_index, count):
-    """Side stream ``bucket_index % count`` of ``device`` (default priority), created on first use.
-    A bucket keeps its stream from step to step, so its state is only ever touched in order."""
-    pool = _SIDE_STREAMS.get((device, count))
-    if pool is None:
-        pool = [torch.cuda.Stream(device=device) for _ in range(count)]
-        _SIDE_STREAMS[(device, count)] = pool
-    return pool[bucket_index % count]
+_side_stream = _pools.side_stream
 
 
 def run_round(state, bucket, error_mode):

@@ -15,7 +15,8 @@ INCLUDE = os.path.join(os.path.dirname(HERE), "include")     # the public C head
 LIBDIR = os.path.join(HERE, "lib")
 LIBPATH = os.path.join(LIBDIR, "libconef_hip.so")
 
-SOURCES = ["conef_sketch.hip", "conef_randblock.hip", "conef_psgd.hip", "conef_topk.hip", "conef_plan.hip"]
+SOURCES = ["conef_sketch.hip", "conef_randblock.hip", "conef_randblock_batch.hip", "conef_psgd.hip", "conef_topk.hip",
+           "conef_plan.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -55,7 +56,7 @@ def build(verbose=False):
             print(res.stderr, file=sys.stderr)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(4, len(sources))) as pool:
+    with ThreadPoolExecutor(max_workers=min(6, len(sources))) as pool:
         objs = list(pool.map(compile_one, sources))
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIBPATH] + objs
     res = subprocess.run(cmd, capture_output=True, text=True)

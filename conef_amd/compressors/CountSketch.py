@@ -91,7 +91,7 @@ class DenseCS:
             tbin = int(os.environ.get("CONEF_PLAN_BIN", "0"))
             if SketchPlan.applicable(self.N, self.D, self.range, chunk, tbin):
                 try:
-                    self._plan = SketchPlan(self.N, self.D, self.range, self.a, self.b, self.cs.device, chunk, tbin)
+                    self._plan = SketchPlan.shared(self.N, self.D, self.range, self.a, self.b, self.cs.device, chunk, tbin)
                 except ValueError:       # e.g. one bucket collects more columns than a bin image can hold
                     self._plan = False
         if self._plan is False:

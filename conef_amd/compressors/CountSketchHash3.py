@@ -63,7 +63,7 @@ class DenseCSHash3:
             self._plans = False
             if os.environ.get("CONEF_PLAN", "1") != "0" and SketchPlan.applicable(self.N, self.D, self.range):
                 try:
-                    self._plans = [SketchPlan(self.N, self.D, self.range, a, b, self.cs0.device, sign_seeds=(sa, sb))
+                    self._plans = [SketchPlan.shared(self.N, self.D, self.range, a, b, self.cs0.device, sign_seeds=(sa, sb))
                                    for a, b, sa, sb in self.HASHES]
                 except ValueError:
                     self._plans = False

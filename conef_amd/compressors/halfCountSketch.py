@@ -33,7 +33,7 @@ class DenseCS:
         """Row-list plan (built on first use) or None; CONEF_PLAN=0 disables it."""
         if self._plan is None and os.environ.get("CONEF_PLAN", "1") != "0":
             if SketchPlan.applicable(self.N, self.D, self.range):
-                plan = SketchPlan(self.N, self.D, self.range, self.a, self.b, self.cs.device)
+                plan = SketchPlan.shared(self.N, self.D, self.range, self.a, self.b, self.cs.device)
                 self._plan = plan if plan.kind == SketchPlan.ROWLIST else False
         return self._plan or None
 

@@ -183,6 +183,33 @@ int conef_randblock_gather_f32(const float* x, float* payload, int64_t numel, in
 int conef_randblock_scatter_f32(float* x, const float* payload, int64_t numel, int64_t start, int64_t block,
                                 void* stream);
 
+/* One tensor of a bucket for conef_randblock_step_batch_f32 (a HOST array of these is read before
+ * the call returns; the pointers inside are device pointers unless the name says host). */
+typedef struct ConefRandBlockItem {
+    float* x;              /* [n,m] gradient, in place */
+    float* err;            /* mode 1: dense error, n*m floats */
+    const float* cs_in;    /* mode 2: sketch [n,w] read ... */
+    float* cs_out;         /* ... and written (may equal cs_in except on a binned plan) */
+    float* payload;        /* `block` floats */
+    const void* plan_host; /* mode 2: the sketch's plan (host copy) or NULL for the unplanned kernels */
+    const void* plan_dev;  /*         the same bytes on the device */
+    void* staging;         /*         binned plans: conef_plan_workspace_bytes(plan_host) bytes */
+    int64_t n, m;
+    int64_t start, block;  /* the wrap-around block [start, start+block) of the flat tensor */
+    int32_t w;             /* mode 2: sketch width */
+    int32_t reserved;
+} ConefRandBlockItem;
+
+/* The fused step of every >= 2-D tensor of a bucket in one call.  mode 0: unbiased block
+ * (conef_randblock_unbiased_step_f32 with prob = fl32(block / numel)); mode 1: dense error feedback
+ * (conef_randblock_ef_step_f32); mode 2: count-sketched error (conef_randblock_conef_step[_planned]_f32).
+ * Dense steps of all items share one launch, and so do sketched steps on row-list plans; results are
+ * bit-identical to the single-tensor entry points.
+ * Replaces the per-tensor loops RandomBlock_hook.py:215-245 and UnbiasedRandomBlock_hook.py:150-170
+ * (and the query loop RandomBlock_hook.py:171-193) for a whole bucket. */
+int conef_randblock_step_batch_f32(const ConefRandBlockItem* items, int32_t count, int32_t mode, float alpha,
+                                   float beta, int32_t a, int32_t b, void* stream);
+
 /* ------------------------------------------------------------------ PowerSGD ---------- */
 /* M is [n,m], Q is [m,r], P is [n,r], 1 <= r <= 32. */
 

@@ -178,6 +178,36 @@ def randblock_conef_step(x, cs, payload, start, block, alpha, beta, a=HASH_A, b=
                                              start, block, np.float32(alpha), np.float32(beta), a, b)
 
 
+def randblock_conef_step_threaded(x, cs, payload, start, block, alpha, beta, threads, a=HASH_A, b=HASH_B):
+    """The same step with the rows of the sketch (they are independent: every row reads and writes
+    only its own cells) spread over ``threads`` host threads; the foreign calls release the GIL.
+    Same arithmetic per row, so bit-identical to ``randblock_conef_step``.  Used for CPU timing."""
+    from concurrent.futures import ThreadPoolExecutor
+    n, m = x.shape
+    numel = n * m
+    end = min(start + block, numel)
+    rest = block - (end - start)
+    flat = x.reshape(-1)
+
+    def per_row(fn):
+        with ThreadPoolExecutor(max_workers=max(1, min(threads, n))) as pool:
+            list(pool.map(fn, range(n)))
+
+    per_row(lambda r: cs_query(x[r:r + 1], cs[r:r + 1], alpha, a, b))
+    payload[:end - start] = flat[start:end]
+    cp = x.copy()
+    cpf = cp.reshape(-1)
+    cpf[start:end] = 0
+    if rest > 0:
+        payload[end - start:] = flat[:rest]
+        cpf[:rest] = 0
+    per_row(lambda r: cs_update(cp[r:r + 1], cs[r:r + 1], beta, a, b))
+    flat[:] = 0
+    flat[start:end] = payload[:end - start]
+    if rest > 0:
+        flat[:rest] = payload[end - start:]
+
+
 def block_bounds(numel, ratio, start):
     """RandomBlock_hook.py:216-223 -> (block, end, rest)."""
     block = max(1, int(ratio * numel))

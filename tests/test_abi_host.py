@@ -75,6 +75,19 @@ def test_argument_validation_without_gpu(lib):
     assert lib.conef_psgd_round_ahead_f32(items, 1, 0, 0, 0.0, 0.0, 0.0, 1, 1, None, 1, None, 0, 0, 0) == -1
     assert lib.conef_psgd_round_ahead_f32(items, 0, 0, 0, 0.0, 0.0, 0.0, 1, 1, None, 0, None, 0, 0, 0) == 0     # empty bucket
     assert lib.conef_psgd_round_ahead_f32(items, 1, 0, 4, 0.0, 0.0, 0.0, 1, 1, None, 0, None, 0, 0, 0) == -1    # pqt_mode
+    # the one-call-per-bucket random-block step: every item is checked before anything is enqueued
+    rb = (_lib.RandBlockItem * 2)()
+    for it in rb:
+        it.x, it.payload, it.err, it.n, it.m, it.start, it.block = 1, 1, 1, 4, 10, 3, 4
+    assert lib.conef_randblock_step_batch_f32(rb, 2, 3, 0.1, 0.9, 1, 1, 0) == -1        # unknown mode
+    assert lib.conef_randblock_step_batch_f32(rb, -1, 0, 0.1, 0.9, 1, 1, 0) == -1
+    assert lib.conef_randblock_step_batch_f32(None, 1, 0, 0.1, 0.9, 1, 1, 0) == -1
+    assert lib.conef_randblock_step_batch_f32(rb, 0, 1, 0.1, 0.9, 1, 1, 0) == 0         # a bucket without matrices
+    rb[1].start = 40
+    assert lib.conef_randblock_step_batch_f32(rb, 2, 0, 0.1, 0.9, 1, 1, 0) == -1        # start == numel in the second item
+    rb[1].start, rb[1].err = 3, None
+    assert lib.conef_randblock_step_batch_f32(rb, 2, 1, 0.1, 0.9, 1, 1, 0) == -1        # dense mode without an error tensor
+    assert lib.conef_randblock_step_batch_f32(rb, 2, 2, 0.1, 0.9, 1, 1, 0) == -1        # sketched mode without sketches
     # shapes: short rows may update in place, the flat 25 MB bucket may not
     assert lib.conef_cs_update_inplace_ok(640, 5760, 1152) == 1
     assert lib.conef_cs_update_inplace_ok(5, 1_300_000, 130_000) == 0
@@ -125,6 +138,11 @@ def test_states_and_host_logic_need_no_gpu():
     assert (s.compression_ratio, s.beta, s.sketch_size, s.use_error_feedback, s.use_error_compression) == \
         (0.1, 0.9, 0.5, True, False)
     assert [int(s.rng.choice(6_500_000)) for _ in range(2)] == [6413414, 6423388]
+    # the hooks draw block offsets with randint(0, n): the stream choice(n) draws from for an int n
+    # (RandomBlock_hook.py:218, UnbiasedRandomBlock_hook.py:157), on every size class of the generator
+    a, b = np.random.RandomState(42), np.random.RandomState(42)
+    sizes = [6_500_000, 33278 * 650, 2600 * 650, 17, 1, 2, 255, 256, 65_536, 2 ** 31 - 1, 2 ** 31 + 5, 2 ** 33 + 1] * 20
+    assert [int(a.choice(n)) for n in sizes] == [int(b.randint(0, n)) for n in sizes]
     p = PowerSGDState(None, start_powerSGD_iter=2)
     assert (p.matrix_approximation_rank, p.min_compression_rate, p.warm_start, p.beta, p.sketch_size) == \
         (1, 2, True, 0.9, 0.5)
@@ -154,3 +172,48 @@ def test_hooks_refuse_host_tensors():
     ps.iter = 2
     with pytest.raises(ValueError, match="no CPU path"):
         powerSGD_hook(ps, FakeGradBucket(g, [(4, 10)]))
+
+
+def test_plans_are_shared_and_released():
+    """One plan per (shape, seeds, tiling, device), however many sketches ask for it; release()
+    drops the pool without invalidating a plan somebody still holds."""
+    import torch
+    import conef_amd
+    from conef_amd import _pools
+    from conef_amd._plan import SketchPlan
+    conef_amd.release()
+    cpu = torch.device("cpu")
+    p1 = SketchPlan.shared(40, 650, 65, 994443, 609478, cpu)
+    p2 = SketchPlan.shared(40, 650, 65, 994443, 609478, cpu)
+    p3 = SketchPlan.shared(40, 650, 65, 994443, 609478, cpu, sign_seeds=(7, 9))
+    p4 = SketchPlan.shared(5, 130_000, 13_000, 994443, 609478, cpu)
+    assert p1 is p2 and p3 is not p1
+    assert p1.kind == SketchPlan.ROWLIST and p1.workspace_bytes == 0
+    assert p4.kind == SketchPlan.BINNED and p4.workspace_bytes >= 4 * 5 * 130_000
+    held = _pools.held_bytes()
+    assert held["plans"] == p1.device.numel() + p3.device.numel() + p4.device.numel() and held["staging"] == 0
+    with pytest.raises(ValueError):
+        SketchPlan.shared(9, 1_300_000, 130_000, 994443, 609478, cpu)      # long rows and more than 8 of them
+    with pytest.raises(ValueError):                                       # ... remembered, not rebuilt
+        SketchPlan.shared(9, 1_300_000, 130_000, 994443, 609478, cpu)
+    conef_amd.release()
+    assert _pools.held_bytes()["plans"] == 0
+    assert p1.header()["w"] == 65                                        # still valid for its holder
+    assert SketchPlan.shared(40, 650, 65, 994443, 609478, cpu) is not p1
+
+
+def test_threaded_oracle_step_is_the_single_threaded_one(oracle):
+    """The CPU baseline spreads the sketch rows over host threads: same bits as the fused C step."""
+    rng = np.random.RandomState(3)
+    n, m, w, block = 5, 20_000, 2_000, 9_000
+    x0 = (rng.randn(n, m) * 1e-3).astype(np.float32)
+    cs_a = (rng.randn(n, w) * 1e-3).astype(np.float32)
+    cs_b = cs_a.copy()
+    for start in (95_000, 12_345):              # one block that wraps, one that does not
+        xa, xb = x0.copy(), x0.copy()
+        pa, pb = np.empty(block, np.float32), np.empty(block, np.float32)
+        oracle.randblock_conef_step(xa, cs_a, pa, start, block, 0.1, 0.9)
+        oracle.randblock_conef_step_threaded(xb, cs_b, pb, start, block, 0.1, 0.9, threads=3)
+        np.testing.assert_array_equal(xa, xb)
+        np.testing.assert_array_equal(pa, pb)
+        np.testing.assert_array_equal(cs_a, cs_b)

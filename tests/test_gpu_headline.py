@@ -1,7 +1,7 @@
 """The headline configuration at full size: RandomBlock 10 % + count-sketch 10 % on a flat 6.5 M
 element bucket viewed [5, 1_300_000], heavy-tailed gradients, error carried across steps.
-Checked against the oracle for a few steps (bit for bit: the planned path adds in the oracle's
-order) and through size-independent properties for more."""
+Checked against the oracle over the configuration's 100 steps (bit for bit: the planned path adds
+in the oracle's order) and through size-independent properties."""
 import numpy as np
 import pytest
 import torch
@@ -21,8 +21,9 @@ def test_headline_steps_match_oracle_bit_for_bit(oracle):
     st.iter = 2
     ost = oracle.RandomBlockOracle(compression_ratio=0.1, use_error_compression=True, sketch_size=0.1, beta=0.9,
                                    random_seed=42)
-    for step in range(3):
-        g = heavy_tail_gradient(L, seed=500 + step)
+    bases = [heavy_tail_gradient(L, seed=500 + k) for k in range(6)]
+    for step in range(100):         # the configuration's own length, error carried from step to step
+        g = bases[step % 6] if step < 6 else bases[step % 6].roll(step * 7919)
         gd = g.cuda()
         RandomBlock_hook(st, FakeGradBucket(gd, [(N, M)])).wait()
         og = g.numpy().copy()
@@ -30,7 +31,8 @@ def test_headline_steps_match_oracle_bit_for_bit(oracle):
         np.testing.assert_array_equal(to_np(gd), og)
         np.testing.assert_array_equal(to_np(st.compressed_tensor_memory[0]), ost.compressed_tensor_memory[0])
         np.testing.assert_array_equal(to_np(st.error_dict[0][0].cs), ost.error_dict[0][0].cs)
-    assert ost.last_starts == [1692743]          # third draw of RandomState(42).choice(6.5 M)
+        if step == 2:
+            assert ost.last_starts == [1692743]          # third draw of RandomState(42).choice(6.5 M)
     assert st.error_dict[0][0].range == 130_000 and st.compressed_tensor_memory[0].numel() == 650_000
 
 

@@ -22,7 +22,8 @@ def grads(total, seed, sigma=1e-3):
     return (torch.randn(total, generator=g) * sigma).float()
 
 
-def run_steps(hook, state, ostate, shapes, steps, bucket_cls=FakeGradBucket, seed0=100, check=None):
+def run_steps(hook, state, ostate, shapes, steps, bucket_cls=FakeGradBucket, seed0=100, check=None, resync=None):
+    """``resync(step)``, when given, runs after a step's check: see ``psgd_resync_factory``."""
     total = numel_of(shapes)
     state.iter = getattr(state, "start_compression_iter", None) or state.start_powerSGD_iter
     for step in range(steps):
@@ -33,6 +34,8 @@ def run_steps(hook, state, ostate, shapes, steps, bucket_cls=FakeGradBucket, see
         og = g.numpy().copy()
         ostate.step(0, og, shapes)
         check(step, gd, og)
+        if resync is not None:
+            resync(step)
     return state
 
 
@@ -205,7 +208,9 @@ def test_products_parity(oracle):
                          # ranks 9..32 run on the matrix cores when the shapes allow
                          (1024, 1024, 32, 0), (1000, 516, 32, 0), (33, 4096, 16, 0), (2049, 1000, 20, 0),
                          (4096, 1024, 32, 0), (30522, 128, 32, 0), (100, 130, 32, 0), (77, 129, 16, 0),
-                         (640, 5760, 32, 3), (64, 64, 17, 0), (31, 8192, 9, 0), (1024, 4096, 32, 4)]:
+                         (640, 5760, 32, 3), (64, 64, 17, 0), (31, 8192, 9, 0), (1024, 4096, 32, 4),
+                         # the BERT-large matrices at their full shapes, both ranks of that configuration
+                         (30522, 1024, 8, 0), (30522, 1024, 32, 0), (4096, 1024, 8, 0), (1024, 4096, 8, 0)]:
         M = rng.randn(n, m).astype(np.float32)
         Q = rng.randn(m, r).astype(np.float32)
         P = rng.randn(n, r).astype(np.float32)
@@ -251,6 +256,8 @@ def test_batch_products_parity(oracle):
              # matrix-core items share launches when m % 4 == 0 and the matrix is 16-byte aligned
              (1024, 1024, 32, 0), (1000, 516, 32, 0), (4096, 1024, 32, 0), (33, 4096, 16, 0), (100, 130, 32, 0),
              (2049, 1000, 20, 0), (77, 128, 16, 1), (1024, 4096, 32, 0)] + [(96 + k, 200, 4, 0) for k in range(30)]
+    # the BERT-large matrices at full shape, as a bucket holds them
+    specs += [(30522, 1024, 8, 0), (4096, 1024, 8, 0), (1024, 4096, 8, 0), (30522, 1024, 32, 0)]
     for mode in (0, 1):
         items = (_lib.PsgdItem * len(specs))()
         keep, host = [], []
@@ -408,6 +415,28 @@ def psgd_check_factory(st, ost, mode):
     return check
 
 
+def psgd_resync_factory(st, ost, mode, free_steps=4):
+    """Error feedback and warm start feed a step's rounding differences back into the next step's
+    input, where Gram-Schmidt on small factors amplifies them: two fp32 evaluations of the same
+    round drift apart by more than 1e-5 after enough steps, whatever the order of their sums.  The
+    first ``free_steps`` steps run free (device and oracle each on their own state); from then on
+    the oracle restarts every step from the device's state, so that every further step is still
+    held to 1e-5 on its own arithmetic while the device carries its error on."""
+    def resync(step):
+        if step + 1 < free_steps:
+            return
+        for arr, view in zip(ost.p_memory_dict[0], _views(st.p_memory_dict[0], ost.p_memory_dict[0])):
+            arr[...] = to_np(view)
+        for arr, view in zip(ost.q_memory_dict[0], _views(st.q_memory_dict[0], ost.q_memory_dict[0])):
+            arr[...] = to_np(view)
+        if mode == "ef":
+            ost.error_dict[0][...] = to_np(st.error_dict[0])
+        elif mode in ("conef", "conef_v2"):
+            for k in ost.error_dict[0]:
+                ost.error_dict[0][k].cs[...] = to_np(st.error_dict[0][k].cs)
+    return resync
+
+
 def _views(flat, like):
     out, off = [], 0
     for arr in like:
@@ -432,9 +461,11 @@ def test_powersgd_hook_parity(oracle, shapes, rank, ss, mode):
                        use_error_feedback=mode is not None, use_error_compression=mode == "conef",
                        sketch_size=ss, beta=0.9)
     ost = oracle.PowerSGDOracle(matrix_approximation_rank=rank, error_mode=mode, sketch_size=ss, beta=0.9)
-    run_steps(powerSGD_hook, st, ost, shapes, 4, check=psgd_check_factory(st, ost, mode))
+    steps = 10 if shapes is RESNET20_SHAPES else 4      # the ResNet-20 configuration is quoted at 10 steps
+    run_steps(powerSGD_hook, st, ost, shapes, steps, check=psgd_check_factory(st, ost, mode),
+              resync=psgd_resync_factory(st, ost, mode))
     rate, before, after = st.compression_stats()
-    assert before == 4 * numel_of(shapes) and 0 < after < before and rate > 1
+    assert before == steps * numel_of(shapes) and 0 < after < before and rate > 1
 
 
 @pytest.mark.parametrize("shapes,rank,ss", PSGD_CASES[:3])
@@ -681,6 +712,127 @@ def test_powersgd_state_errors_and_warmup():
     powerSGD_hook(st, FakeGradBucket(g, [(64, 64)])).wait()
     assert st.iter == 4 and not torch.equal(g, ref)
     assert torch.linalg.matrix_rank(g.view(64, 64).cpu().double(), tol=1e-4) <= 2
+
+
+def _state_for(mode, rank, ss, **kw):
+    from conef_amd.hPowerSGD_hook import hPowerSGDState, hpowerSGD_hook
+    from conef_amd.powerSGD_hook import PowerSGDState, powerSGD_hook
+    if mode == "topk":
+        return hPowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, use_error_compression=True,
+                              topk_ratio=0.4, **kw), hpowerSGD_hook
+    return PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2,
+                         use_error_feedback=mode is not None, use_error_compression=mode == "conef", sketch_size=ss,
+                         beta=0.9, **kw), powerSGD_hook
+
+
+def _error_check(st, ost, mode, what):
+    def check(step, gd, og):
+        assert_close(gd, og, what="%s: decompressed bucket, step %d" % (what, step))
+        if mode == "ef":
+            assert_close(st.error_dict[0], ost.error_dict[0], what="%s: dense error, step %d" % (what, step))
+        elif mode == "conef":
+            for k in ost.error_dict[0]:
+                assert_close(st.error_dict[0][k].cs, ost.error_dict[0][k].cs, what="%s: sketch %d step %d" % (what, k, step))
+        elif mode == "topk":
+            for k in ost.error_dict[0]:
+                got, want = to_np(st.error_dict[0][k]), ost.error_dict[0][k]
+                assert np.count_nonzero(got) == np.count_nonzero(want)
+                same = (got != 0) == (want != 0)
+                assert same.mean() > 0.999
+                assert_close(np.where(same, got, 0), np.where(same, want, 0), what="%s: top-k error %d" % (what, k))
+    return check
+
+
+@pytest.mark.parametrize("shapes,rank,ss", [PSGD_CASES[1], PSGD_CASES[2], PSGD_CASES[3]])
+@pytest.mark.parametrize("mode", [None, "ef", "conef", "topk"])
+def test_powersgd_hooks_without_warm_start(oracle, shapes, rank, ss, mode):
+    """warm_start=False (powerSGD_hook.py:434-436,479-494,566-568): every call draws fresh Q
+    factors from the state's seed stream (one randint per call, then one CPU randn per factor),
+    orthogonalises them, and drops the P / Q arenas at its end."""
+    if mode == "topk" and rank == 32:
+        pytest.skip("the top-k configuration is quoted at rank 8")
+    st, hook = _state_for(mode, rank, ss, warm_start=False)
+    ost = oracle.PowerSGDOracle(matrix_approximation_rank=rank, error_mode=mode, sketch_size=ss, beta=0.9,
+                                topk_ratio=0.4, warm_start=False)
+    check = _error_check(st, ost, mode, "cold start")
+    seeds = []
+
+    def check_and_note(step, gd, og):
+        check(step, gd, og)
+        seeds.append(ost.last_seed)
+        assert not st.p_memory_dict and not st.q_memory_dict        # dropped at the end of the call (:566-568)
+
+    run_steps(hook, st, ost, shapes, 4, check=check_and_note)
+    assert seeds[:3] == [209652396, 398764591, 924231285]           # RandomState(0).randint(1e9): one draw per call
+    assert st.iter == 6
+
+
+@pytest.mark.parametrize("eps", [1e-8, 1e-2])
+@pytest.mark.parametrize("mode", ["ef", "conef", "topk"])
+@pytest.mark.parametrize("ahead", ["0", "1"])
+def test_powersgd_hooks_with_orthogonalization_epsilon(monkeypatch, oracle, mode, eps, ahead):
+    """orthogonalization_epsilon != 0 (powerSGD_hook.py:24-30): col /= (norm + eps) in every
+    Gram-Schmidt of the round, through the hooks, with the next round's Q factors orthogonalised
+    inside the round's last launch (1) and at the start of the next round (0)."""
+    monkeypatch.setenv("CONEF_ROUND_AHEAD", ahead)
+    for shapes, rank, ss in (PSGD_CASES[1], PSGD_CASES[2], PSGD_CASES[3]):
+        if mode == "topk" and rank == 32:
+            continue
+        st, hook = _state_for(mode, rank, ss, orthogonalization_epsilon=eps)
+        ost = oracle.PowerSGDOracle(matrix_approximation_rank=rank, error_mode=mode, sketch_size=ss, beta=0.9,
+                                    topk_ratio=0.4, orthogonalization_epsilon=eps)
+        run_steps(hook, st, ost, shapes, 4, check=psgd_check_factory(st, ost, mode))
+        # eps really took part: the factors are not orthonormal by about eps / norm at eps = 1e-2
+        if eps == 1e-2:
+            p = _views(st.p_memory_dict[0], ost.p_memory_dict[0])[0].double()
+            assert float((p.t() @ p - torch.eye(p.shape[1], device="cuda", dtype=torch.float64)).abs().max()) > 1e-3
+
+
+@pytest.mark.parametrize("eps,warm", [(1e-8, True), (1e-2, True), (0, False), (1e-2, False)])
+def test_batched_powersgd_hook_epsilon_and_cold_start(oracle, eps, warm):
+    from conef_amd.powerSGD_hook import PowerSGDState, batched_powerSGD_hook
+    for total, rank in ((5000, 2), (268_346, 1), (40_000, 4)):
+        st = PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, warm_start=warm,
+                           orthogonalization_epsilon=eps)
+        ost = oracle.BatchedPowerSGDOracle(matrix_approximation_rank=rank, warm_start=warm, orthogonalization_epsilon=eps)
+
+        def check(step, gd, og):
+            assert_close(gd, og, what="batched eps %g warm %s: bucket, step %d" % (eps, warm, step))
+            assert_close(st.error_dict[0], ost.error_dict[0], what="padded dense error, step %d" % step)
+            if warm:
+                assert_close(st.p_memory_dict[0], ost.p_memory_dict[0], what="P")
+                assert_close(st.q_memory_dict[0], ost.q_memory_dict[0], what="Q")
+            else:
+                assert not st.p_memory_dict and not st.q_memory_dict
+
+        run_steps(batched_powerSGD_hook, st, ost, [(total,)], 3, check=check)
+
+
+def test_gram_schmidt_nearly_parallel_columns(oracle):
+    """Ill-conditioned input: columns that differ from one direction by 1e-3, as a warm-started
+    factor of a nearly rank-one gradient has them.  Classical Gram-Schmidt amplifies rounding
+    differences by the condition number, so the bar is what two fp32 evaluations of the reference's
+    own formula differ by: the span is compared (projector onto the columns), not the columns."""
+    from conef_amd._psgd_engine import orthogonalize
+    rng = np.random.RandomState(5)
+    for rows, r in [(1024, 8), (4096, 8), (1024, 32), (4096, 32), (30522, 8), (700, 4)]:
+        base = rng.randn(rows, 1).astype(np.float32)
+        a = (base + 1e-3 * rng.randn(rows, r)).astype(np.float32)
+        want = a.copy()
+        oracle.gram_schmidt(want, 0.0)
+        got = torch.from_numpy(a).cuda()
+        orthogonalize(got)
+        g64 = got.double().cpu().numpy()
+        # the first column is a plain normalisation: tight
+        assert_close(g64[:, 0], want[:, 0], what="first column [%d,%d]" % (rows, r))
+        # all columns: within the amplified rounding (condition number about 1e3 sqrt(r)), and
+        # orthonormal to what fp32 Gram-Schmidt keeps at that conditioning (the oracle's own result
+        # sits at 6e-5 for [30522,8]; the order of the sums moves it by a small factor)
+        amp = 1e-5 * 1e3 * 4
+        assert np.abs(g64 - want).max() <= amp * np.abs(want).max(), (rows, r, np.abs(g64 - want).max())
+        dev_eye = np.abs(g64.T @ g64 - np.eye(r)).max()
+        ora_eye = np.abs(want.astype(np.float64).T @ want.astype(np.float64) - np.eye(r)).max()
+        assert dev_eye <= max(8 * ora_eye, 2e-3), (rows, r, dev_eye, ora_eye)
 
 
 # ------------------------------------------------------- unbiased random matrix --
