@@ -19,7 +19,7 @@ _I64 = ctypes.c_int64
 _I32 = ctypes.c_int32
 _F32 = ctypes.c_float
 
-# name -> argtypes; every function returns int (0 = ok, >0 hipError_t, -1 invalid argument),
+# name -> argtypes; every function returns int (0 = ok, >0 hipError_t, -1 invalid argument, -2 too large),
 # except the *_bytes functions, which return a byte count as int64
 SIGNATURES = {
     "conef_version": [],
@@ -76,6 +76,7 @@ SIGNATURES = {
     "conef_topk_sparsify_f32": [_P, _I64, _I64, _P, _I64, _P],
     "conef_topk_batch_workspace_bytes": [_P, _I32],
     "conef_topk_sparsify_batch_f32": [_P, _P, _P, _I32, _P, _I64, _P],
+    "conef_topk_sparsify_noalloc_f32": [_P, _I64, _I64, _P],
     "conef_randblock_step_batch_f32": [_P, _I32, _I32, _F32, _F32, _I32, _I32, _P],
 }
 
@@ -124,6 +125,8 @@ def check(code, what):
     if code != 0:
         if code == -1:
             raise ValueError("%s: invalid argument" % what)
+        if code == -2:
+            raise ValueError("%s: input larger than the entry point's stated maximum" % what)
         raise ConefLibraryError("%s: HIP error %d" % (what, code))
 
 

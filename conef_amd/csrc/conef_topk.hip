@@ -16,7 +16,10 @@
 // and clears the ties past the first `remaining` of them.  More than 1024 such ties (a tensor of
 // repeated values) are settled by one workgroup walking the tensor in index order instead: exact,
 // slow, and of no practical concern.  Nothing returns to the host between passes.
+#include <mutex>
+
 #include "conef_device.h"
+#include "conef_hip.h"
 
 namespace {
 
@@ -334,6 +337,46 @@ inline int64_t topk_hist_groups(int64_t numel)
     return g < 1 ? 1 : g > 512 ? 512 : g;
 }
 
+
+// ---- selection state of the entry point that allocates nothing ------------------------------
+// One TopkState per GPU, inside the code object: every GPU the library runs on holds its own
+// copy at its own address until the process ends.  `scratch` is only a host-side handle of the
+// symbol; device code and hipMemsetAsync need the address hipGetSymbolAddress returns for the
+// device that is current, looked up once per device and kept.
+constexpr size_t kScratchBytes = (sizeof(TopkState) + 255) / 256 * 256;      // 29 184 bytes
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kScratchMaxDevices = 64;
+std::mutex g_scratch_lock;
+void* g_scratch_ptr[kScratchMaxDevices] = {};
+
+// Address of the current device's copy of `scratch`, or null with *err set.
+inline void* topk_scratch_of_current_device(int* err)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        *err = (int)e;
+        return nullptr;
+    }
+    if (dev < 0 || dev >= kScratchMaxDevices) {
+        *err = CONEF_ERR_INVALID;
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            *err = e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol;
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    *err = CONEF_OK;
+    return g_scratch_ptr[dev];
+}
+
 }  // namespace
 
 extern "C" {
@@ -410,6 +453,30 @@ int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const
             hipLaunchKernelGGL(topk_hist_batch_kernel, dim3((unsigned)wgs), dim3(256), 0, s, b, pass);
         hipLaunchKernelGGL(topk_filter_batch_kernel, dim3((unsigned)wgs), dim3(256), 0, s, b);
     }
+    return (int)hipGetLastError();
+}
+
+
+// conef_topk_sparsify_f32 for callers that may not allocate (HIP graph capture, serving loops):
+// the selection state lives in the library's own per-GPU scratch (29 184 bytes), so no workspace
+// is passed.  The device the stream belongs to must be current.  Calls on one GPU share that
+// scratch: calls that may overlap there (different streams, different threads) race; calls on
+// one stream are safe back to back because the first kernel of a call resets the state.
+int conef_topk_sparsify_noalloc_f32(float* x, int64_t numel, int64_t k, void* stream)
+{
+    if (numel < 1 || k < 1 || !x) return CONEF_ERR_INVALID;
+    if (numel > CONEF_TOPK_NOALLOC_MAX_NUMEL) return CONEF_ERR_TOO_LARGE;
+    if (k >= numel) return CONEF_OK;
+    int err = CONEF_OK;
+    void* ptr = topk_scratch_of_current_device(&err);
+    if (!ptr) return err;
+    hipStream_t s = (hipStream_t)stream;
+    TopkState* st = (TopkState*)ptr;
+    const int64_t g = topk_hist_groups(numel);
+    hipLaunchKernelGGL(topk_init_kernel, dim3(1), dim3(256), 0, s, st, (uint32_t)k);      // clears what the last call left
+    for (int pass = 0; pass < kPasses; ++pass)
+        hipLaunchKernelGGL(topk_hist_kernel, dim3((unsigned)g), dim3(256), 0, s, x, numel, st, pass);
+    hipLaunchKernelGGL(topk_filter_kernel, dim3((unsigned)g), dim3(256), 0, s, x, numel, st);
     return (int)hipGetLastError();
 }
 

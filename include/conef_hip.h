@@ -10,11 +10,13 @@
  *     stream has run the call (the one exception, conef_hash_table_host_i32, takes host memory);
  *   - `stream` is a hipStream_t (NULL = the default stream); every call is asynchronous on it,
  *     never synchronises the host, never allocates or frees device memory, keeps no global or
- *     thread-local state and may be called from any thread;
+ *     thread-local state and may be called from any thread (the one exception is
+ *     conef_topk_sparsify_noalloc_f32, which works in a per-GPU scratch array of the library);
  *   - scalars (alpha, beta, hash seeds) travel by value - the reference passes them as pointers
  *     to 1-element device tensors it allocates per call (CountSketch.py:144,167);
  *   - matrices are dense row-major fp32; a sketch is [n, w] row-major, fp32 unless the name says f16;
- *   - return value: 0 = enqueued, -1 = invalid argument (nothing enqueued), > 0 = hipError_t.
+ *   - return value: 0 = enqueued, -1 = invalid argument, -2 = input larger than the entry point's
+ *     stated maximum (nothing enqueued either way), > 0 = hipError_t.
  *   - empty inputs (n == 0 or d == 0) are accepted and do nothing.
  *
  * Floating point: multiplications and additions are done in the order the reference's kernels
@@ -32,6 +34,7 @@ extern "C" {
 
 #define CONEF_OK 0
 #define CONEF_ERR_INVALID (-1)
+#define CONEF_ERR_TOO_LARGE (-2) /* an input exceeds the stated maximum of the entry point */
 
 /* Library ABI version (1). */
 int conef_version(void);
@@ -360,6 +363,17 @@ int conef_topk_sparsify_f32(float* x, int64_t numel, int64_t k, void* workspace,
 int64_t conef_topk_batch_workspace_bytes(const int64_t* numels, int32_t count);
 int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const int64_t* ks, int32_t count,
                                   void* workspace, int64_t workspace_bytes, void* stream);
+
+/* conef_topk_sparsify_f32 without a workspace argument and without any allocation.  No counterpart
+ * in the reference: it is for callers that cannot allocate device memory - code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The selection state (29 184
+ * bytes) lives in a per-GPU scratch array inside the library, which every GPU the library runs on
+ * holds until the process ends.  The device `stream` belongs to must be the current device.
+ * numel > CONEF_TOPK_NOALLOC_MAX_NUMEL returns CONEF_ERR_TOO_LARGE (nothing enqueued).  All calls on
+ * one GPU share the scratch: back-to-back calls on one stream are safe (a call first resets it),
+ * calls that can overlap on one GPU (other streams, other threads) race. */
+#define CONEF_TOPK_NOALLOC_MAX_NUMEL 0xffffffffLL
+int conef_topk_sparsify_noalloc_f32(float* x, int64_t numel, int64_t k, void* stream);
 
 #ifdef __cplusplus
 }

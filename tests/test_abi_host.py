@@ -88,6 +88,13 @@ def test_argument_validation_without_gpu(lib):
     rb[1].start, rb[1].err = 3, None
     assert lib.conef_randblock_step_batch_f32(rb, 2, 1, 0.1, 0.9, 1, 1, 0) == -1        # dense mode without an error tensor
     assert lib.conef_randblock_step_batch_f32(rb, 2, 2, 0.1, 0.9, 1, 1, 0) == -1        # sketched mode without sketches
+    # the top-k entry point that allocates nothing: argument checks come before any device call
+    assert lib.conef_topk_sparsify_noalloc_f32(1, 1 << 32, 10, 0) == -2                 # beyond its stated maximum
+    assert lib.conef_topk_sparsify_noalloc_f32(1, 100, 0, 0) == -1
+    assert lib.conef_topk_sparsify_noalloc_f32(None, 100, 10, 0) == -1
+    assert lib.conef_topk_sparsify_noalloc_f32(1, 100, 100, 0) == 0                     # k >= numel: nothing to do
+    with pytest.raises(ValueError, match="stated maximum"):
+        _lib.check(-2, "conef_topk_sparsify_noalloc_f32")
     # shapes: short rows may update in place, the flat 25 MB bucket may not
     assert lib.conef_cs_update_inplace_ok(640, 5760, 1152) == 1
     assert lib.conef_cs_update_inplace_ok(5, 1_300_000, 130_000) == 0
