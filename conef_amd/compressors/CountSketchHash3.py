@@ -33,7 +33,8 @@ class DenseCSHash3:
 
     def load_state_dict(self, d):
         if (d["N"], d["D"], d["range"]) != (self.N, self.D, self.range):
-            raise ValueError("sketch shape mismatch")
+            raise ValueError("sketch shape mismatch: have (%d,%d,%d), state holds (%d,%d,%d)" % (
+                self.N, self.D, self.range, d["N"], d["D"], d["range"]))
         for k in ("cs0", "cs1", "cs2"):
             getattr(self, k).copy_(torch.from_numpy(d[k]).to(self.cs0.device))
 
@@ -44,6 +45,17 @@ class DenseCSHash3:
         for k in ("cs0", "cs1", "cs2"):
             setattr(obj, k, torch.from_numpy(d[k]).to(obj.cs0.device).contiguous())
         return obj
+
+    # pickling carries the state, not the library handle (the reference class pickles too)
+    __getstate__ = state_dict
+
+    def __setstate__(self, d):
+        device = torch.device("cuda", torch.cuda.current_device())
+        self.N, self.D, self.blk_size, self.range = d["N"], d["D"], d["blk_size"], d["range"]
+        for k in ("cs0", "cs1", "cs2"):
+            setattr(self, k, torch.from_numpy(d[k]).to(device))
+        self._spare = self._plans = self._value = None
+        self._lib = _lib.load()
 
     def _check(self, t, name):
         _lib.require_device_f32(t, name)

@@ -43,8 +43,12 @@ class DenseCS:
 
     def load_state_dict(self, d):
         if (d["N"], d["D"], d["range"]) != (self.N, self.D, self.range):
-            raise ValueError("sketch shape mismatch")
+            raise ValueError("sketch shape mismatch: have (%d,%d,%d), state holds (%d,%d,%d)" % (
+                self.N, self.D, self.range, d["N"], d["D"], d["range"]))
         self.cs.copy_(torch.from_numpy(d["cs"]).to(self.cs.device))
+        self.a = int(d.get("a", HASH_A))
+        self.b = int(d.get("b", HASH_B))
+        self._plan = None          # a plan belongs to its hash seeds
 
     @classmethod
     def from_state_dict(cls, d, device=None):
@@ -54,6 +58,18 @@ class DenseCS:
         obj.a, obj.b = int(d.get("a", HASH_A)), int(d.get("b", HASH_B))
         obj._inplace = bool(obj._lib.conef_cs_update_inplace_ok(obj.N, obj.D, obj.range))
         return obj
+
+    # pickling carries the state, not the library handle (the reference class pickles too)
+    __getstate__ = state_dict
+
+    def __setstate__(self, d):
+        device = torch.device("cuda", torch.cuda.current_device())
+        self.N, self.D, self.blk_size, self.range = d["N"], d["D"], d["blk_size"], d["range"]
+        self.cs = torch.from_numpy(d["cs"]).to(device)
+        self.a, self.b = int(d.get("a", HASH_A)), int(d.get("b", HASH_B))
+        self._lib = _lib.load()
+        self._inplace = bool(self._lib.conef_cs_update_inplace_ok(self.N, self.D, self.range))
+        self._plan = None
 
     def _check(self, t, name):
         _lib.require_device_f32(t, name)

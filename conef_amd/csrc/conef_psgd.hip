@@ -11,6 +11,8 @@
 // the passes that touch M anyway.  Sums that cross workgroups meet through a caller-provided
 // workspace in a fixed order: no atomics, results do not change from run to run.
 #include <type_traits>
+#include <algorithm>
+#include <atomic>
 #include <vector>
 
 #include "conef_device.h"
@@ -18,6 +20,7 @@
 #include "conef_plan.h"
 #include "conef_psgd_mfma.h"
 #include "conef_gs_lanes.h"
+#include "conef_gs_gram.h"
 #include "conef_hip.h"      // ConefPsgdItem, and a check of this file's definitions against the public header
 
 extern "C" int conef_cs_query_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
@@ -1376,6 +1379,8 @@ inline int64_t gs_sums_floats(int64_t rows, int r)
     int64_t grid = (int64_t)(sizeof(GsGridWs) + 3) / 4;
     int64_t lanes = (int64_t)(sizeof(GslWs) + 3) / 4;
     if (lanes > grid) grid = lanes;
+    int64_t gramws = (int64_t)(sizeof(GsgWs) + 3) / 4;
+    if (gramws > grid) grid = gramws;
     return steps > grid ? steps : grid;
 }
 
@@ -1517,6 +1522,47 @@ inline int gsl_launch(const GslBatch& batch, int count, int r, int rpt, int wgs,
     hipError_t e = hipLaunchCooperativeKernel(fn, dim3((unsigned)wgs), dim3(kGslThreads), args, 0, s);
     if (e != hipSuccess) (void)hipGetLastError();
     return (int)e;
+}
+
+// Kernel of conef_gs_gram.h (one exchange between workgroups instead of one per column).  It can
+// take any matrix that is exactly 8, 16 or 32 wide and 16-byte aligned (gsg_can); it is the better
+// kernel (gsg_wants) at ranks 16 and 32 above 1024 rows and at rank 8 above the 4096 rows one
+// workgroup's registers hold: a launch lasts 20 to 30 us whatever it holds, where the
+// column-by-column kernels pay per step and per workgroup involved.  Shorter factors of rank 16 or
+// 32 join a launch that a taller one of their bucket needs anyway (each on its own workgroups);
+// short rank-8 factors stay with the row-per-thread kernel, which also orthogonalises them inside
+// the last launch of a round.
+inline bool gsg_can(const float* a, int64_t rows, int r)
+{
+    return (r == 8 || r == 16 || r == 32) && aligned16(a) && rows <= 0x7fffffffLL;
+}
+
+inline bool gsg_wants(const float* a, int64_t rows, int r)
+{
+    if (!gsg_can(a, rows, r)) return false;
+    return r >= 16 ? rows > 1024 : rows * r > (int64_t)kGsRegThreads * kGsRegFloats;
+}
+
+std::atomic<unsigned> g_gsg_launches{0};
+
+// One launch over `count` matrices of rank r (workgroup ranges in batch.first).  A normal launch:
+// at most 128 workgroups of 256 threads, which a GPU that is running anything else still holds
+// side by side; the waits inside are bounded either way.
+inline int gsg_launch(const GsgBatch& batch, int count, int r, int wgs, float eps, void* workspace, hipStream_t s)
+{
+    unsigned tag = (g_gsg_launches.fetch_add(1u) + 1u) * 0x9E3779B9u;
+    if (tag == 0u) tag = 1u;
+    GsgWs* ws = (GsgWs*)workspace;
+    if (r == 32) hipLaunchKernelGGL(gsg_kernel<32>, dim3((unsigned)wgs), dim3(kGsgThreads), 0, s, batch, count, eps, ws, tag);
+    else if (r == 16) hipLaunchKernelGGL(gsg_kernel<16>, dim3((unsigned)wgs), dim3(kGsgThreads), 0, s, batch, count, eps, ws, tag);
+    else if (r == 8) hipLaunchKernelGGL(gsg_kernel<8>, dim3((unsigned)wgs), dim3(kGsgThreads), 0, s, batch, count, eps, ws, tag);
+    else return CONEF_ERR_INVALID;
+    return (int)hipGetLastError();
+}
+
+inline bool gsg_workspace_ok(const void* workspace, int64_t workspace_bytes)
+{
+    return workspace && workspace_bytes >= (int64_t)sizeof(GsgWs) && (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0;
 }
 
 inline bool psgd_args_ok(int64_t n, int64_t m, int32_t r)
@@ -1750,6 +1796,19 @@ int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* w
     if (rows < 1 || rows > 0x7fffffffLL || r < 1 || r > kMaxRank || !a) return CONEF_ERR_INVALID;
     hipStream_t s = (hipStream_t)stream;
     const int rp = rank_bound(r);
+    if (gsg_wants(a, rows, r)) {
+        GsgBatch one;
+        int slab, wgs;
+        gsg_split(rows, r, &slab, &wgs);
+        if (wgs == 1 || gsg_workspace_ok(workspace, workspace_bytes)) {
+            one.a[0] = a;
+            one.rows[0] = (int)rows;
+            one.slab[0] = slab;
+            one.first[0] = 0;
+            one.first[1] = wgs;
+            return gsg_launch(one, 1, r, wgs, eps, workspace, s);
+        }
+    }
     {
         const GslChoice ch = gsl_choose(rows, r);
         if (ch.kind == 1) {
@@ -1849,6 +1908,39 @@ int conef_gram_schmidt_batch_f32(float* const* mats, const int64_t* rows, const 
     std::vector<char> done((size_t)count, 0);
     for (int k = 0; k < count; ++k) {
         if (rows[k] < 1 || rows[k] > 0x7fffffffLL || ranks[k] < 1 || ranks[k] > kMaxRank || !mats[k]) return CONEF_ERR_INVALID;
+    }
+    // kernel of conef_gs_gram.h: matrices of one rank share launches, each on its own workgroups
+    const bool gram_ws_ok = gsg_workspace_ok(workspace, workspace_bytes);
+    for (int k = 0; k < count; ++k) {
+        if (done[(size_t)k] || !gsg_wants(mats[k], rows[k], ranks[k])) continue;
+        GsgBatch batch;
+        std::vector<int> members;
+        int nb = 0, wgs = 0;
+        // the matrices that want this kernel first, then (ranks 16 and 32) the bucket's shorter ones as guests
+        for (int pass = 0; pass < 2; ++pass) {
+            for (int j = 0; j < count && nb < kGsgMaxItems; ++j) {
+                if (done[(size_t)j] || ranks[j] != ranks[k] || !gsg_can(mats[j], rows[j], ranks[j])) continue;
+                const bool wants = gsg_wants(mats[j], rows[j], ranks[j]);
+                if (pass == 0 ? !wants : (wants || ranks[j] < 16)) continue;
+                if (std::find(members.begin(), members.end(), j) != members.end()) continue;
+                int slab, w;
+                gsg_split(rows[j], ranks[j], &slab, &w);
+                if (w > 1 && !gram_ws_ok) continue;
+                if (wgs + w > kGsgMaxWgs) continue;
+                batch.a[nb] = mats[j];
+                batch.rows[nb] = (int)rows[j];
+                batch.slab[nb] = slab;
+                batch.first[nb] = wgs;
+                wgs += w;
+                ++nb;
+                members.push_back(j);
+            }
+        }
+        if (nb == 0) continue;
+        batch.first[nb] = wgs;
+        const int rc = gsg_launch(batch, nb, ranks[k], wgs, eps, workspace, s);
+        if (rc != CONEF_OK) return rc;
+        for (int j : members) done[(size_t)j] = 1;
     }
     // kernels of conef_gs_lanes.h: matrices of one rank and class share launches (up to 48 matrices
     // of the one-workgroup kernel; up to 24 matrices and 128 workgroups of the other)

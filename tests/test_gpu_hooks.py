@@ -949,3 +949,20 @@ def test_sketch_variants_round_trip():
         back.update(v, 0.9)
         for nme in names:
             assert torch.equal(getattr(sk, nme), getattr(back, nme))
+        # pickling carries the state and not the library handle, as the reference's classes pickle;
+        # load_state_dict brings the hash seeds along
+        import pickle
+        again = pickle.loads(pickle.dumps(sk))
+        assert type(again) is cls
+        again.update(v, 0.9)
+        sk.update(v, 0.9)
+        for nme in names:
+            assert torch.equal(getattr(sk, nme), getattr(again, nme))
+        if cls is HalfDenseCS:
+            other = cls(6, 3000, 0.13)
+            sd = sk.state_dict()
+            sd["a"], sd["b"] = 12345, 678
+            other.load_state_dict(sd)
+            assert (other.a, other.b) == (12345, 678)
+            with pytest.raises(ValueError, match=r"have \(6,3000,390\), state holds \(7,3000,390\)"):
+                other.load_state_dict(dict(sd, N=7))
