@@ -159,6 +159,14 @@ class DenseCS:
     def query(self, grad_plus_error, alpha):
         """grad_plus_error += alpha * unsketch(cs), in place (CountSketch.py:70-98)."""
         self._check(grad_plus_error, "grad_plus_error")
+        plan = self.plan()
+        if plan is not None:
+            # buckets and signs from the plan's table instead of two hashes and modulos per column
+            rc = self._lib.conef_cs_query_planned_f32(grad_plus_error.data_ptr(), self.cs.data_ptr(), plan.host_ptr,
+                                                      plan.device.data_ptr(), self.N, self.D, self.range, float(alpha),
+                                                      self.a, self.b, _lib.stream_ptr(grad_plus_error))
+            _lib.check(rc, "conef_cs_query_planned_f32")
+            return
         rc = self._lib.conef_cs_query_f32(grad_plus_error.data_ptr(), self.cs.data_ptr(), self.N, self.D,
                                           self.range, float(alpha), self.a, self.b,
                                           _lib.stream_ptr(grad_plus_error))

@@ -105,6 +105,13 @@ class DenseCS:
 
     def query(self, grad_plus_error, alpha):
         self._check(grad_plus_error, "grad_plus_error")
+        plan = self.plan()
+        if plan is not None:
+            rc = self._lib.conef_cs_query_planned_f16(grad_plus_error.data_ptr(), self.cs.data_ptr(), plan.host_ptr,
+                                                      plan.device.data_ptr(), self.N, self.D, self.range, float(alpha),
+                                                      self.a, self.b, _lib.stream_ptr(grad_plus_error))
+            _lib.check(rc, "conef_cs_query_planned_f16")
+            return
         rc = self._lib.conef_cs_query_f16(grad_plus_error.data_ptr(), self.cs.data_ptr(), self.N, self.D,
                                           self.range, float(alpha), self.a, self.b,
                                           _lib.stream_ptr(grad_plus_error))

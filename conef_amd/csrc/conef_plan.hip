@@ -4,7 +4,19 @@
 
 namespace {
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// the sign-hash seeds a plan's tables were built with
+inline bool plan_has_default_sign_seeds(const ConefPlanHeader* hp, int32_t a, int32_t b)
+{
+    return hp->reserved[0] == (((int64_t)(uint32_t)(a + 2) << 32) | (uint32_t)(b + 3));
+}
 }  // namespace
+
+// conef_sketch.hip
+int conef_launch_query_table_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
+                                 int32_t b, const uint32_t* pktab, hipStream_t stream);
+int conef_launch_query_table_f16(float* x, const void* cs_half, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
+                                 int32_t b, const uint32_t* pktab, hipStream_t stream);
 
 extern "C" {
 
@@ -79,6 +91,26 @@ int conef_cs_update_planned_f16(const float* vec, const void* cs_in_half, void* 
     ConefListVec front = {vec, aligned16(vec) && d % 4 == 0};
     return conef_launch_rowlist(front, conef_rowlist_view(hp, plan_dev), (const __half*)cs_in_half,
                                 (__half*)cs_out_half, n, d, w, beta, (hipStream_t)stream);
+}
+
+// DenseCS.query with the buckets and signs of a plan's table instead of hashing (either kind of
+// plan, built for (n, d, w, a, b) with the default sign seeds): same values, bit for bit.
+int conef_cs_query_planned_f32(float* x, const float* cs, const void* plan_host, const void* plan_dev, int64_t n,
+                               int64_t d, int32_t w, float alpha, int32_t a, int32_t b, void* stream)
+{
+    const ConefPlanHeader* hp = (const ConefPlanHeader*)plan_host;
+    if (!conef_plan_matches(hp, n, d, w, a, b) || !plan_dev || !plan_has_default_sign_seeds(hp, a, b)) return CONEF_ERR_INVALID;
+    const uint32_t* pk = (const uint32_t*)((const char*)plan_dev + hp->off_pk);
+    return conef_launch_query_table_f32(x, cs, n, d, w, alpha, a, b, pk, (hipStream_t)stream);
+}
+
+int conef_cs_query_planned_f16(float* x, const void* cs_half, const void* plan_host, const void* plan_dev, int64_t n,
+                               int64_t d, int32_t w, float alpha, int32_t a, int32_t b, void* stream)
+{
+    const ConefPlanHeader* hp = (const ConefPlanHeader*)plan_host;
+    if (!conef_plan_matches(hp, n, d, w, a, b) || !plan_dev || !plan_has_default_sign_seeds(hp, a, b)) return CONEF_ERR_INVALID;
+    const uint32_t* pk = (const uint32_t*)((const char*)plan_dev + hp->off_pk);
+    return conef_launch_query_table_f16(x, cs_half, n, d, w, alpha, a, b, pk, (hipStream_t)stream);
 }
 
 // 0 = binned (needs the workspace, fused step needs cs_out != cs_in), 1 = row lists (no

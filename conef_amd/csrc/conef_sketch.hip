@@ -37,14 +37,22 @@ __global__ void hash_table_kernel(int32_t* bucket, int32_t* sign, int64_t d, Con
 template <typename CsT, int VW, int RB>
 __global__ void __launch_bounds__(256)
 cs_query_kernel(float* __restrict__ x, const CsT* __restrict__ cs, int64_t n, int64_t d, ConefMod mod,
-                float alpha, ConefSeeds hs, int rows_per_block)
+                float alpha, ConefSeeds hs, int rows_per_block, const uint32_t* __restrict__ pktab)
 {
     int64_t c0 = (blockIdx.x * (int64_t)blockDim.x + threadIdx.x) * 4;
     if (c0 >= d) return;
+    // bucket | sign << 31 of the thread's four columns: from a plan's table when the caller has one
+    // (16 bytes a thread instead of eight hashes and modulos), else computed
     uint32_t pk[4];
+    if (pktab && c0 + 4 <= d) {
+        const uint4 t = *reinterpret_cast<const uint4*>(pktab + c0);      // tables are 256-byte aligned, c0 a multiple of 4
+        pk[0] = t.x; pk[1] = t.y; pk[2] = t.z; pk[3] = t.w;
+    } else {
 #pragma unroll
-    for (int k = 0; k < 4; ++k)
-        pk[k] = (c0 + k < d) ? conef_bucket_sign((int32_t)(c0 + k), mod, hs.a, hs.b, hs.sa, hs.sb) : 0u;
+        for (int k = 0; k < 4; ++k)
+            pk[k] = (c0 + k < d) ? (pktab ? pktab[c0 + k] : conef_bucket_sign((int32_t)(c0 + k), mod, hs.a, hs.b, hs.sa, hs.sb))
+                                 : 0u;
+    }
     int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
     int64_t r1 = r0 + rows_per_block < n ? r0 + rows_per_block : n;
     // VW = 4: rows are 16-byte aligned, one float4 per row; VW = 2: 8-byte aligned, two float2
@@ -325,7 +333,7 @@ inline int rows_per_block_for(int64_t n, int64_t col_blocks)
 
 template <typename CsT>
 int launch_query(float* x, const CsT* cs, int64_t n, int64_t d, int32_t w, float alpha, int32_t a, int32_t b,
-                 hipStream_t stream)
+                 hipStream_t stream, const uint32_t* pktab = nullptr)
 {
     if (n < 0 || d < 0 || w < 1 || w > (1 << 30) || d > 0x7fffffffLL) return CONEF_ERR_INVALID;
     if (n == 0 || d == 0) return CONEF_OK;
@@ -337,7 +345,7 @@ int launch_query(float* x, const CsT* cs, int64_t n, int64_t d, int32_t w, float
     const int vw = (d % 4 == 0 && aligned16(x)) ? 4 : (d % 2 == 0 && (reinterpret_cast<uintptr_t>(x) & 7u) == 0) ? 2 : 1;
     ConefMod mod = conef_make_mod(w);
     if (vw == 1) {
-        hipLaunchKernelGGL((cs_query_kernel<CsT, 1, 1>), grid, dim3(256), 0, stream, x, cs, n, d, mod, alpha, hs, rpb);
+        hipLaunchKernelGGL((cs_query_kernel<CsT, 1, 1>), grid, dim3(256), 0, stream, x, cs, n, d, mod, alpha, hs, rpb, pktab);
         return (int)hipGetLastError();
     }
     // Rows in flight per thread: the whole row group when it is small; four at a time when the
@@ -349,10 +357,10 @@ int launch_query(float* x, const CsT* cs, int64_t n, int64_t d, int32_t w, float
     case RB:                                                                                                          \
         if (vw == 4)                                                                                                  \
             hipLaunchKernelGGL((cs_query_kernel<CsT, 4, RB>), grid, dim3(256), 0, stream, x, cs, n, d, mod, alpha, hs, \
-                               rpb);                                                                                  \
+                               rpb, pktab);                                                                           \
         else                                                                                                          \
             hipLaunchKernelGGL((cs_query_kernel<CsT, 2, RB>), grid, dim3(256), 0, stream, x, cs, n, d, mod, alpha, hs, \
-                               rpb);                                                                                  \
+                               rpb, pktab);                                                                           \
         break
         CONEF_QUERY_CASE(1);
         CONEF_QUERY_CASE(2);
@@ -377,6 +385,20 @@ int launch_update(const float* vec, const CsT* cs_in, CsT* cs_out, int64_t n, in
 }
 
 }  // namespace
+
+// The query with buckets and signs read from a table (uint32[d]: bucket | sign bit << 31, the `pk`
+// table of a plan); called by conef_cs_query_planned_f32 / _f16 in conef_plan.hip.
+int conef_launch_query_table_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
+                                 int32_t b, const uint32_t* pktab, hipStream_t stream)
+{
+    return launch_query<float>(x, cs, n, d, w, alpha, a, b, stream, pktab);
+}
+
+int conef_launch_query_table_f16(float* x, const void* cs_half, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
+                                 int32_t b, const uint32_t* pktab, hipStream_t stream)
+{
+    return launch_query<__half>(x, (const __half*)cs_half, n, d, w, alpha, a, b, stream, pktab);
+}
 
 // ============================================================ C entry points ====
 extern "C" {

@@ -159,6 +159,14 @@ int conef_randblock_conef_step_f32(float* x, const float* cs_in, float* cs_out, 
                                    int64_t m, int32_t w, int64_t start, int64_t block, float alpha, float beta,
                                    int32_t a, int32_t b, void* stream);
 
+/* conef_cs_query_f32 / _f16 with every column's bucket and sign read from the plan's table instead of
+ * hashed (a plan of either kind built for (n, d, w, a, b) with the default sign seeds): same values,
+ * bit for bit; on the flat 25 MB bucket the hashing is most of the query's time. */
+int conef_cs_query_planned_f32(float* x, const float* cs, const void* plan_host, const void* plan_dev, int64_t n,
+                               int64_t d, int32_t w, float alpha, int32_t a, int32_t b, void* stream);
+int conef_cs_query_planned_f16(float* x, const void* cs_half, const void* plan_host, const void* plan_dev, int64_t n,
+                               int64_t d, int32_t w, float alpha, int32_t a, int32_t b, void* stream);
+
 /* conef_randblock_conef_step_f32 on a plan (see above).  With a binned plan cs_out must NOT be
  * cs_in (-1): the selected block is finished from the old sketch while the new one is being
  * written.  With a row-list plan it may. */
