@@ -7,6 +7,11 @@ above the 256 MB Infinity Cache where the shape allows), HIP events on the launc
     python bench_kernels.py [--filter substring] [--iters N]
 
 Prints one line per case: microseconds per call, algorithmic bytes, GB/s, fraction of 8 TB/s.
+
+    python -m conef_amd.build --trace && python bench_kernels.py --phase-trace
+
+prints instead when the workgroups of the two passes of the fused RandomBlock + sketch step reach
+their phase boundaries (a build of the same sources that also stores timestamps).
 """
 import argparse
 import json
@@ -26,7 +31,11 @@ def main():
     ap.add_argument("--hook-streams", type=int, default=2, help="side streams of the 'N streams' hook-step lines")
     ap.add_argument("--iters", type=int, default=200)
     ap.add_argument("--json", action="store_true")
+    ap.add_argument("--phase-trace", action="store_true",
+                    help="phase timeline of the binned passes on the flat 25 MB bucket (needs the --trace build)")
     args = ap.parse_args()
+    if args.phase_trace:
+        return phase_trace()
 
     import torch
     from conef_amd import _lib
@@ -255,6 +264,55 @@ def main():
         hook_steps(args, results)
     if not args.json:
         print("done: %d cases" % len(results))
+    teardown()
+
+
+def phase_trace():
+    """Workgroup phase timeline of the staging and accumulate passes, [5, 1300000] bucket, block 650000."""
+    import ctypes
+
+    import numpy as np
+    import torch
+    from conef_amd import _lib
+    from conef_amd.build import TRACE_LIBPATH
+
+    if not os.path.exists(TRACE_LIBPATH):
+        print("no %s: run `python -m conef_amd.build --trace` first" % TRACE_LIBPATH, file=sys.stderr)
+        sys.exit(2)
+    _lib.LIBPATH = TRACE_LIBPATH              # before the first load: every entry point comes from the tracing build
+    lib = _lib.load()
+    lib.conef_trace_read.argtypes = [ctypes.c_void_p]
+    lib.conef_trace_read.restype = ctypes.c_int
+    from conef_amd.compressors.CountSketch import DenseCS
+
+    n, m, block = 5, 1_300_000, 650_000
+    grads = [torch.randn(n, m, device="cuda") * 1e-3 for _ in range(24)]
+    sketches = [DenseCS(n, m, 0.1) for _ in range(12)]
+    payload = torch.empty(block, device="cuda")
+    rng = np.random.RandomState(42)
+    buf = np.zeros((2, 1024, 8), dtype=np.uint64)
+    rows = {0: [], 1: []}
+    for it in range(40):
+        sketches[it % 12].randblock_step(grads[it % 24], payload, int(rng.randint(0, n * m)), block, 0.1, 0.9)
+        torch.cuda.synchronize()
+        if it < 8:
+            continue
+        _lib.check(lib.conef_trace_read(buf.ctypes.data_as(ctypes.c_void_p)), "conef_trace_read")
+        for p in (0, 1):
+            t = buf[p].astype(np.int64)
+            t = t[t[:, 0] > 0]                   # workgroups of this launch
+            rows[p].append((t - t[:, 0].min()) * 0.01)
+    names = {0: ["workgroup starts", "its loads are in LDS", "after the barrier", "stores issued"],
+             1: ["bin threads start", "first records arrived", "bin image complete", "after the barrier",
+                 "lists walked, cells written", "column waves start", "selected block finished", "zeros written"]}
+    for p in (0, 1):
+        a = np.concatenate(rows[p])              # [launches * workgroups, 8]
+        print("pass %s, microseconds after its first workgroup started (%d workgroups per launch)"
+              % ("AB"[p], len(rows[p][0])))
+        for k, name in enumerate(names[p]):
+            v = a[:, k]
+            v = v[v >= 0]
+            print("  %-30s median %6.2f   p90 %6.2f   max %6.2f" % (name, np.median(v), np.percentile(v, 90), v.max()))
     teardown()
 
 

@@ -14,6 +14,9 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")     # the public C header, for the batch item struct
 LIBDIR = os.path.join(HERE, "lib")
 LIBPATH = os.path.join(LIBDIR, "libconef_hip.so")
+# same sources with -DCONEF_TRACE: the two binned passes also write per-workgroup phase timestamps,
+# read back with conef_trace_read (a measuring build; nothing in the package loads it)
+TRACE_LIBPATH = os.path.join(LIBDIR, "libconef_hip_trace.so")
 
 SOURCES = ["conef_sketch.hip", "conef_randblock.hip", "conef_randblock_batch.hip", "conef_psgd.hip", "conef_topk.hip",
            "conef_plan.hip"]
@@ -37,16 +40,18 @@ def _hipcc():
     raise RuntimeError("hipcc not found; the ConEF HIP library cannot be built")
 
 
-def build(verbose=False):
+def build(verbose=False, trace=False):
     hipcc = _hipcc()
     os.makedirs(LIBDIR, exist_ok=True)
-    objdir = os.path.join(LIBDIR, "obj")
+    objdir = os.path.join(LIBDIR, "obj_trace" if trace else "obj")
+    flags = HIPCC_FLAGS + (["-DCONEF_TRACE"] if trace else [])
+    libpath = TRACE_LIBPATH if trace else LIBPATH
     os.makedirs(objdir, exist_ok=True)
     sources = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
 
     def compile_one(src):
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [hipcc] + HIPCC_FLAGS + ["-I", CSRC, "-I", INCLUDE, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc] + flags + ["-I", CSRC, "-I", INCLUDE, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         res = subprocess.run(cmd, capture_output=True, text=True)
@@ -58,12 +63,12 @@ def build(verbose=False):
 
     with ThreadPoolExecutor(max_workers=min(6, len(sources))) as pool:
         objs = list(pool.map(compile_one, sources))
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIBPATH] + objs
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", libpath] + objs
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("link failed:\n%s\n%s" % (res.stdout, res.stderr))
-    return LIBPATH
+    return libpath
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, trace="--trace" in sys.argv[1:]))

@@ -323,6 +323,19 @@ struct ConefStageRandBlock {
     }
 };
 
+// Phase timestamps (100 MHz counter) of every workgroup of the two passes: only in builds that define
+// CONEF_TRACE, read back with conef_trace_read (conef_plan.hip).
+#ifdef CONEF_TRACE
+static __device__ unsigned long long conef_trace_buf[2][1024][8];
+#define CONEF_STAMP(pass, who, slot)                                                                   \
+    do {                                                                                               \
+        if ((int)threadIdx.x == (who) && blockIdx.x < 1024)                                            \
+            conef_trace_buf[pass][blockIdx.x][slot] = (unsigned long long)wall_clock64();              \
+    } while (0)
+#else
+#define CONEF_STAMP(pass, who, slot) do { } while (0)
+#endif
+
 // ------------------------------------------------------------------ pass A ----
 // One workgroup per chunk: loads, permutes the records into the LDS image, and after the barrier
 // the image leaves LDS with linear 16-byte stores.
@@ -332,6 +345,7 @@ conef_binned_stage_kernel(Stage stage, ConefPlanView plan, float* __restrict__ s
 {
     extern __shared__ float conef_img[];   // [chunk_cols][NROWS]
     const int chunk = conef_xcd_major(blockIdx.x, nblocks_padded, plan.flags);
+    CONEF_STAMP(0, 0, 0);
     if (chunk >= plan.nchunks) return;
     const int64_t c_begin = (int64_t)chunk * plan.chunk_cols;
     const int cols = d - c_begin < plan.chunk_cols ? (int)(d - c_begin) : plan.chunk_cols;
@@ -360,7 +374,9 @@ conef_binned_stage_kernel(Stage stage, ConefPlanView plan, float* __restrict__ s
             }
         }
     }
+    CONEF_STAMP(0, 0, 1);
     __syncthreads();
+    CONEF_STAMP(0, 0, 2);
     float* out = staging + c_begin * NROWS;        // 16-byte aligned: c_begin is a multiple of 4
     const int total = cols * NROWS;
     const int total4 = total >> 2;
@@ -369,6 +385,7 @@ conef_binned_stage_kernel(Stage stage, ConefPlanView plan, float* __restrict__ s
         conef_store4(out + 4 * e, v.x, v.y, v.z, v.w, (plan.flags & 4) != 0);
     }
     for (int e = (total4 << 2) + threadIdx.x; e < total; e += blockDim.x) out[e] = conef_img[e];
+    CONEF_STAMP(0, 0, 3);
 }
 
 // Column-order work of the fused RandomBlock step that pass B carries (x == null: none).
@@ -408,6 +425,7 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
         // ---- column-order work of the fused step.  These waves owe the bin's threads nothing:
         // they pass the workgroup's one barrier first and then work on their own.
         __syncthreads();
+        CONEF_STAMP(1, gthreads, 5);
         const int64_t me = blockIdx.x * (int64_t)col_threads + (threadIdx.x - gthreads);
         const int64_t nworkers = (int64_t)gridDim.x * col_threads;
         const int64_t bquads = (bw.block + 3) >> 2;
@@ -450,6 +468,7 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
                 }
             }
         }
+        CONEF_STAMP(1, gthreads, 6);
         const bool vec_ok = (reinterpret_cast<uintptr_t>(bw.x) & 15u) == 0;
         const int64_t nquads = (bw.numel + 3) >> 2;
         for (int64_t q = me; q < nquads; q += nworkers) {
@@ -463,8 +482,10 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
                     if (!any_sel || conef_payload_pos(f + k, bw.blk) < 0) bw.x[f + k] = 0.f;
             }
         }
+        CONEF_STAMP(1, gthreads, 7);
         return;
     }
+    CONEF_STAMP(1, 0, 0);
 
     const int bin_raw = conef_xcd_major(blockIdx.x, nblocks_padded, plan.flags);
     const bool has_bin = bin_raw < plan.nbins;          // padding workgroups only share the column work
@@ -518,6 +539,7 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
 #pragma unroll
         for (int r = 0; r < NROWS; ++r) v[u][r] = srcp[u][k * NROWS + r];
     }
+    CONEF_STAMP(1, 0, 1);       // the first records of my segments have arrived
     if (has_bin)
         for (uint32_t t = threadIdx.x; t < e_last - e_first; t += gthreads) ent_l[t] = plan.ent[e_first + t];
 
@@ -545,7 +567,9 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
             }
         }
     }
+    CONEF_STAMP(1, 0, 2);
     __syncthreads();
+    CONEF_STAMP(1, 0, 3);
 
     if (!active) return;
     // per row: the decay c*aux (double) and the query term for sign +1 do not change along the
@@ -582,6 +606,7 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
         int r = sub + k * nsub;
         if (r < NROWS) cs_out[(int64_t)r * w + j] = acc[k];
     }
+    CONEF_STAMP(1, 0, 4);
 }
 
 // ---------------------------------------------------------------- launcher ----

@@ -147,4 +147,12 @@ int conef_randblock_conef_step_planned_f32(float* x, const float* cs_in, float* 
                                (hipStream_t)stream);
 }
 
+#ifdef CONEF_TRACE
+// copies the phase timestamps of the last binned launch pair to host memory (2 * 1024 * 8 uint64)
+int conef_trace_read(void* host_dst)
+{
+    return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(conef_trace_buf), sizeof(conef_trace_buf));
+}
+#endif
+
 }  // extern "C"
