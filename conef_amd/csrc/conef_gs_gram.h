@@ -94,6 +94,116 @@ __device__ __forceinline__ void gsg_entry(int e, int rp, int* pi, int* pj)
     *pj = i + (e - (i * rp - (i * (i - 1)) / 2));
 }
 
+// The r column steps on the upper triangle of the r x r Gram matrix in LDS (all T threads of the
+// workgroup call this; `gram` must be complete and visible).  Leaves b_ij in coef[i][j] (i < j) and
+// 1 / d_i in dinvf[i]; `dinv` is scratch.
+template <int RP, int T>
+__device__ __forceinline__ void gsg_recurrence(double (*gram)[RP + 1], float (*coef)[RP], double* dinv, float* dinvf,
+                                               float eps, int tid)
+{
+    constexpr int NG = RP * (RP + 1) / 2;
+    // Thread (j, part) owns
+    // entries (j, k), k = j + part, j + part + parts, ...  Step i reads row i (final since the
+    // barrier of step i - 1) and rewrites the rows below it; its coefficients go to `coef`, which
+    // nobody reads before the last barrier.  One barrier per step.
+    // A thread owns the same few entries (j, k), j <= k, throughout.  The r steps run in panels of
+    // four pivots: a panel's pivot rows at the thread's columns and the panel's own 4 x 4 block are
+    // read once, the four steps then run in registers (every thread repeats the small block's
+    // arithmetic, so nobody waits for anybody inside a panel), and one barrier ends the panel:
+    // r / 4 trips through LDS and the barrier instead of r.
+    constexpr int EPT = (NG + T - 1) / T;                   // entries per thread: 1, 1, 3 at ranks 8, 16, 32
+    constexpr int B = RP < 4 ? RP : 4;
+    int ej[EPT], ek[EPT];
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+        const int e = tid + u * T;
+        int i, j2;
+        gsg_entry(e < NG ? e : 0, RP, &i, &j2);
+        ej[u] = e < NG ? i : -1;                            // -1: no entry, never active
+        ek[u] = j2;
+    }
+#pragma unroll 1
+    for (int i0 = 0; i0 < RP; i0 += B) {
+        double P[B][B];                                     // the panel's block, upper triangle
+#pragma unroll
+        for (int a2 = 0; a2 < B; ++a2) {
+#pragma unroll
+            for (int b2 = a2; b2 < B; ++b2) P[a2][b2] = gram[i0 + a2][i0 + b2];
+        }
+        double g[EPT], Rj[EPT][B], Rk[EPT][B];
+        int na[EPT];                                        // steps of this panel that reach the entry
+#pragma unroll
+        for (int u = 0; u < EPT; ++u) {
+            const int dj = ej[u] - i0;
+            na[u] = dj <= 0 ? 0 : (dj < B ? dj : B);
+            const bool on = dj >= 0;                        // rows of the panel itself are read for their coefficients
+            g[u] = gram[on ? ej[u] : i0][on ? ek[u] : i0];
+#pragma unroll
+            for (int a2 = 0; a2 < B; ++a2) {
+                const bool use = a2 < na[u];
+                Rj[u][a2] = gram[i0 + a2][use ? ej[u] : i0 + a2];
+                Rk[u][a2] = gram[i0 + a2][use ? ek[u] : i0 + a2];
+            }
+        }
+        double inv2[B];
+#pragma unroll
+        for (int a2 = 0; a2 < B; ++a2) {
+            // 1 / d^2: hardware estimate and two Newton steps (exact to the last bits of a double)
+            // instead of a division.  With eps = 0, d^2 is the pivot itself and the square root
+            // for 1 / d waits until after the loop.
+            const double piv = P[a2][a2];
+            double dd = piv;
+            if (eps != 0.f) {
+                double y = __builtin_amdgcn_rsq(piv);
+                y = y * (1.5 - 0.5 * piv * y * y);
+                y = y * (1.5 - 0.5 * piv * y * y);
+                const double d = (piv == 0. ? 0. : piv * y) + (double)eps;
+                dd = d * d;
+            }
+            double r = __builtin_amdgcn_rcp(dd);
+            r = fma(fma(-dd, r, 1.), r, r);
+            r = fma(fma(-dd, r, 1.), r, r);
+            inv2[a2] = r;
+            if (tid == 0) dinv[i0 + a2] = piv;
+            // G_jk - b_j G_ik - b_k G_ij + b_j b_k G_ii  =  G_jk - (G_ij G_ik) (2 - G_ii / d^2) / d^2
+            const double scale = r * fma(-piv, r, 2.);
+#pragma unroll
+            for (int b2 = a2 + 1; b2 < B; ++b2) {
+                const double pb = P[a2][b2] * scale;
+#pragma unroll
+                for (int c2 = b2; c2 < B; ++c2) P[b2][c2] = fma(-pb, P[a2][c2], P[b2][c2]);
+            }
+#pragma unroll
+            for (int u = 0; u < EPT; ++u) {
+                if (a2 < na[u]) {
+                    g[u] = fma(-(Rj[u][a2] * Rk[u][a2]), scale, g[u]);
+#pragma unroll
+                    for (int b2 = a2 + 1; b2 < B; ++b2) {
+                        const double pb = P[a2][b2] * scale;
+                        Rj[u][b2] = fma(-pb, Rj[u][a2], Rj[u][b2]);
+                        Rk[u][b2] = fma(-pb, Rk[u][a2], Rk[u][b2]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < EPT; ++u) {
+            if (na[u] > 0) gram[ej[u]][ek[u]] = g[u];
+            const int dj = ej[u] - i0;
+            if (dj >= 0 && dj < B && ek[u] > ej[u]) {       // an entry of pivot row j is final after dj steps
+                double r = inv2[0];
+#pragma unroll
+                for (int a2 = 1; a2 < B; ++a2) r = dj == a2 ? inv2[a2] : r;
+                coef[ej[u]][ek[u]] = (float)(g[u] * r);
+            }
+        }
+        __syncthreads();
+    }
+    if (tid < RP) dinvf[tid] = (float)(1. / (sqrt(dinv[tid]) + (double)eps));
+    __syncthreads();
+
+}
+
 template <int RP>
 __global__ void __launch_bounds__(kGsgThreads)
 gsg_kernel(GsgBatch batch, int count, float eps, GsgWs* ws, unsigned tag)
@@ -246,106 +356,8 @@ gsg_kernel(GsgBatch batch, int count, float eps, GsgWs* ws, unsigned tag)
         return;
     }
 
-    // ---- 3. the r column steps on the upper triangle of the r x r matrix.  Thread (j, part) owns
-    // entries (j, k), k = j + part, j + part + parts, ...  Step i reads row i (final since the
-    // barrier of step i - 1) and rewrites the rows below it; its coefficients go to `coef`, which
-    // nobody reads before the last barrier.  One barrier per step.
-    // A thread owns the same few entries (j, k), j <= k, throughout.  The r steps run in panels of
-    // four pivots: a panel's pivot rows at the thread's columns and the panel's own 4 x 4 block are
-    // read once, the four steps then run in registers (every thread repeats the small block's
-    // arithmetic, so nobody waits for anybody inside a panel), and one barrier ends the panel:
-    // r / 4 trips through LDS and the barrier instead of r.
-    constexpr int EPT = (NG + T - 1) / T;                   // entries per thread: 1, 1, 3 at ranks 8, 16, 32
-    constexpr int B = 4;
-    int ej[EPT], ek[EPT];
-#pragma unroll
-    for (int u = 0; u < EPT; ++u) {
-        const int e = tid + u * T;
-        int i, j2;
-        gsg_entry(e < NG ? e : 0, RP, &i, &j2);
-        ej[u] = e < NG ? i : -1;                            // -1: no entry, never active
-        ek[u] = j2;
-    }
-#pragma unroll 1
-    for (int i0 = 0; i0 < RP; i0 += B) {
-        double P[B][B];                                     // the panel's block, upper triangle
-#pragma unroll
-        for (int a2 = 0; a2 < B; ++a2) {
-#pragma unroll
-            for (int b2 = a2; b2 < B; ++b2) P[a2][b2] = gram[i0 + a2][i0 + b2];
-        }
-        double g[EPT], Rj[EPT][B], Rk[EPT][B];
-        int na[EPT];                                        // steps of this panel that reach the entry
-#pragma unroll
-        for (int u = 0; u < EPT; ++u) {
-            const int dj = ej[u] - i0;
-            na[u] = dj <= 0 ? 0 : (dj < B ? dj : B);
-            const bool on = dj >= 0;                        // rows of the panel itself are read for their coefficients
-            g[u] = gram[on ? ej[u] : i0][on ? ek[u] : i0];
-#pragma unroll
-            for (int a2 = 0; a2 < B; ++a2) {
-                const bool use = a2 < na[u];
-                Rj[u][a2] = gram[i0 + a2][use ? ej[u] : i0 + a2];
-                Rk[u][a2] = gram[i0 + a2][use ? ek[u] : i0 + a2];
-            }
-        }
-        double inv2[B];
-#pragma unroll
-        for (int a2 = 0; a2 < B; ++a2) {
-            // 1 / d^2: hardware estimate and two Newton steps (exact to the last bits of a double)
-            // instead of a division.  With eps = 0, d^2 is the pivot itself and the square root
-            // for 1 / d waits until after the loop.
-            const double piv = P[a2][a2];
-            double dd = piv;
-            if (eps != 0.f) {
-                double y = __builtin_amdgcn_rsq(piv);
-                y = y * (1.5 - 0.5 * piv * y * y);
-                y = y * (1.5 - 0.5 * piv * y * y);
-                const double d = (piv == 0. ? 0. : piv * y) + (double)eps;
-                dd = d * d;
-            }
-            double r = __builtin_amdgcn_rcp(dd);
-            r = fma(fma(-dd, r, 1.), r, r);
-            r = fma(fma(-dd, r, 1.), r, r);
-            inv2[a2] = r;
-            if (tid == 0) dinv[i0 + a2] = piv;
-            // G_jk - b_j G_ik - b_k G_ij + b_j b_k G_ii  =  G_jk - (G_ij G_ik) (2 - G_ii / d^2) / d^2
-            const double scale = r * fma(-piv, r, 2.);
-#pragma unroll
-            for (int b2 = a2 + 1; b2 < B; ++b2) {
-                const double pb = P[a2][b2] * scale;
-#pragma unroll
-                for (int c2 = b2; c2 < B; ++c2) P[b2][c2] = fma(-pb, P[a2][c2], P[b2][c2]);
-            }
-#pragma unroll
-            for (int u = 0; u < EPT; ++u) {
-                if (a2 < na[u]) {
-                    g[u] = fma(-(Rj[u][a2] * Rk[u][a2]), scale, g[u]);
-#pragma unroll
-                    for (int b2 = a2 + 1; b2 < B; ++b2) {
-                        const double pb = P[a2][b2] * scale;
-                        Rj[u][b2] = fma(-pb, Rj[u][a2], Rj[u][b2]);
-                        Rk[u][b2] = fma(-pb, Rk[u][a2], Rk[u][b2]);
-                    }
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < EPT; ++u) {
-            if (na[u] > 0) gram[ej[u]][ek[u]] = g[u];
-            const int dj = ej[u] - i0;
-            if (dj >= 0 && dj < B && ek[u] > ej[u]) {       // an entry of pivot row j is final after dj steps
-                double r = inv2[0];
-#pragma unroll
-                for (int a2 = 1; a2 < B; ++a2) r = dj == a2 ? inv2[a2] : r;
-                coef[ej[u]][ek[u]] = (float)(g[u] * r);
-            }
-        }
-        __syncthreads();
-    }
-    GSG_STAMP(3);
-    if (tid < RP) dinvf[tid] = (float)(1. / (sqrt(dinv[tid]) + (double)eps));
-    __syncthreads();
+    // ---- 3. the r column steps on the r x r matrix
+    gsg_recurrence<RP, T>(gram, coef, dinv, dinvf, eps, tid);
     GSG_STAMP(4);
 
     // ---- 4. the same steps on this workgroup's rows, a row per thread: the reference's column

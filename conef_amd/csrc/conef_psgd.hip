@@ -21,6 +21,7 @@
 #include "conef_psgd_mfma.h"
 #include "conef_gs_lanes.h"
 #include "conef_gs_gram.h"
+#include "conef_psgd_stream.h"
 #include "conef_hip.h"      // ConefPsgdItem, and a check of this file's definitions against the public header
 
 extern "C" int conef_cs_query_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
@@ -233,6 +234,16 @@ psgd_mq_batch_kernel(PsgdBatch<MqItem> b, float alpha, ConefSeeds hs)
     int local;
     const MqItem& it = b.item[psgd_batch_locate(b, &local)];
     psgd_mq_body<RB, RP, MODE, FAST>(it.x, it.err, it.cs, it.pktab, it.q, it.p, it.n, it.m, it.r, it.mod, alpha, hs, local);
+}
+
+// streaming form (conef_psgd_stream.h): the kernel of every matrix whose shape allows 16-byte accesses
+template <int RP, int MODE, int T>
+__global__ void __launch_bounds__(T)
+psgd_mqs_batch_kernel(PsgdBatch<MqsItem> b, float alpha, ConefSeeds hs)
+{
+    int local;
+    const MqsItem& it = b.item[psgd_batch_locate(b, &local)];
+    psgd_mqs_body<RP, MODE, T>(it, alpha, hs, local);
 }
 
 // -------------------------------------------------------------- Q = X^T P ----
@@ -647,48 +658,82 @@ struct ListPsgdResidual {
     {
         float* base = x + row0 * d;
         if (FAST) {
-            // A thread owns column quads c4 = t, t + 256, ... and walks the tile's rows with the
-            // quad's slice of Q (4 x RP floats) in registers: Q is read once per quad and tile, not
-            // once per element.  Two rows are in flight; the row of P is uniform over the workgroup.
-            // Narrow matrices (fewer quads than threads) split the rows over thread groups instead.
+            // A thread owns column quads c4 = t, t + 256, ... and takes the tile's rows two at a time
+            // with the quad's slice of Q (4 x RP floats) in registers: Q is read once per quad and
+            // tile, not once per element.  Narrow matrices (fewer quads than threads) split the rows
+            // over thread groups instead.  The tile's rows of P wait in LDS; the next two rows of the
+            // quad - or the next quad's slice of Q and its first two rows - are requested before the
+            // current two are used, so that a thread has one round trip per tile, not one per step.
+            __shared__ float ptile[16 * RP];              // at most 16 rows a tile
+            for (int i = threadIdx.x; i < rows * RP; i += kConefRowlistThreads) ptile[i] = p[row0 * RP + i];
             const int d4 = d >> 2;
             const int lanes = d4 < kConefRowlistThreads ? d4 : kConefRowlistThreads;
             const int groups = kConefRowlistThreads / lanes, grp = threadIdx.x / lanes;
-            for (int c4 = threadIdx.x - grp * lanes; c4 < d4 && grp < groups; c4 += lanes) {
-                float flat[4 * RP];
+            const int step = 2 * groups;
+            int c4 = threadIdx.x - grp * lanes, rw = 2 * grp;
+            bool have = grp < groups && c4 < d4 && rw < rows;
+            float flat[4 * RP], flatn[4 * RP], x0n[4], x1n[4];
+            auto request_rows = [&](int quad, int row) {
+                const int r1 = row + 1 < rows ? row + 1 : row;
+                ld4(base + (int64_t)row * d + 4 * quad, x0n);
+                ld4(base + (int64_t)r1 * d + 4 * quad, x1n);
+            };
+            if (have) {
 #pragma unroll
                 for (int v = 0; v < RP; ++v) ld4(q + (int64_t)c4 * 4 * RP + 4 * v, flat + 4 * v);
-                for (int rw = 2 * grp; rw < rows; rw += 2 * groups) {
-                    const int r1 = rw + 1 < rows ? rw + 1 : rw;
-                    float x0[4], x1[4], p0[RP], p1[RP];
-                    ld4(base + (int64_t)rw * d + 4 * c4, x0);
-                    ld4(base + (int64_t)r1 * d + 4 * c4, x1);
-                    const float* pa = p + (row0 + rw) * RP;
-                    const float* pb = p + (row0 + r1) * RP;
+                request_rows(c4, rw);
+            }
+            __syncthreads();
+            while (have) {
+                const int cur_c4 = c4, cur_rw = rw;
+                const int r1 = cur_rw + 1 < rows ? cur_rw + 1 : cur_rw;
+                float x0[4], x1[4];
 #pragma unroll
-                    for (int c = 0; c < RP; ++c) {
-                        p0[c] = pa[c];
-                        p1[c] = pb[c];
+                for (int k = 0; k < 4; ++k) {
+                    x0[k] = x0n[k];
+                    x1[k] = x1n[k];
+                }
+                rw += step;
+                bool new_quad = false;
+                if (rw >= rows) {
+                    rw = 2 * grp;
+                    c4 += lanes;
+                    new_quad = true;
+                }
+                have = c4 < d4;
+                if (have) {
+                    if (new_quad) {
+#pragma unroll
+                        for (int v = 0; v < RP; ++v) ld4(q + (int64_t)c4 * 4 * RP + 4 * v, flatn + 4 * v);
                     }
-                    float m0[4] = {0.f, 0.f, 0.f, 0.f}, m1[4] = {0.f, 0.f, 0.f, 0.f}, v0[4], v1[4];
+                    request_rows(c4, rw);
+                }
+                const float* pa = ptile + cur_rw * RP;
+                const float* pb = ptile + r1 * RP;
+                float m0[4] = {0.f, 0.f, 0.f, 0.f}, m1[4] = {0.f, 0.f, 0.f, 0.f}, v0[4], v1[4];
 #pragma unroll
-                    for (int c = 0; c < RP; ++c)
-#pragma unroll
-                        for (int k = 0; k < 4; ++k) {
-                            m0[k] = fmaf(p0[c], flat[k * RP + c], m0[k]);
-                            m1[k] = fmaf(p1[c], flat[k * RP + c], m1[k]);
-                        }
+                for (int c = 0; c < RP; ++c) {
+                    const float p0 = pa[c], p1 = pb[c];
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
-                        v0[k] = __fsub_rn(x0[k], m0[k]);
-                        v1[k] = __fsub_rn(x1[k], m1[k]);
+                        m0[k] = fmaf(p0, flat[k * RP + c], m0[k]);
+                        m1[k] = fmaf(p1, flat[k * RP + c], m1[k]);
                     }
-                    st4(base + (int64_t)rw * d + 4 * c4, m0);
-                    st4(vals + rw * d + 4 * c4, v0);
-                    if (rw + 1 < rows) {
-                        st4(base + (int64_t)r1 * d + 4 * c4, m1);
-                        st4(vals + r1 * d + 4 * c4, v1);
-                    }
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    v0[k] = __fsub_rn(x0[k], m0[k]);
+                    v1[k] = __fsub_rn(x1[k], m1[k]);
+                }
+                st4(base + (int64_t)cur_rw * d + 4 * cur_c4, m0);
+                st4(vals + cur_rw * d + 4 * cur_c4, v0);
+                if (cur_rw + 1 < rows) {
+                    st4(base + (int64_t)r1 * d + 4 * cur_c4, m1);
+                    st4(vals + r1 * d + 4 * cur_c4, v1);
+                }
+                if (new_quad && have) {
+#pragma unroll
+                    for (int t = 0; t < 4 * RP; ++t) flat[t] = flatn[t];
                 }
             }
         } else {
@@ -1258,6 +1303,53 @@ inline MfmaMqShape mfma_mq_shape(int64_t n, int64_t m)
 
 constexpr size_t kMfmaMqLdsLimit = 144 * 1024;
 
+// Launches of the streaming P = X Q kernel over `table` (ranks below 16, shapes that allow 16-byte
+// accesses), kPsgdBatchMax matrices a launch.  kMqsNoFit, with nothing launched: a sketch row too
+// wide for LDS, or too little work for this kernel; the caller then takes the row-block kernel.
+constexpr int kMqsNoFit = -100;
+
+template <int MODE>
+int mqs_run(const std::vector<MqsItem>& table, int rp, float alpha, ConefSeeds hs, hipStream_t s)
+{
+    struct Chunk { size_t k; int nb, T, S; size_t lds; };
+    std::vector<Chunk> chunks;
+    for (size_t k = 0; k < table.size();) {
+        Chunk c;
+        c.k = k;
+        c.nb = (int)std::min(table.size() - k, (size_t)kPsgdBatchMax);
+        if (!mqs_plan_launch(&table[k], c.nb, rp, MODE == 2, &c.T, &c.S, &c.lds)) return kMqsNoFit;
+        chunks.push_back(c);
+        k += (size_t)c.nb;
+    }
+    for (const Chunk& c : chunks) {
+        PsgdBatch<MqsItem> b;
+        int total = 0;
+        for (int i = 0; i < c.nb; ++i) {
+            MqsItem it = table[c.k + (size_t)i];
+            it.gw = mqs_group_width(it.m, c.T);
+            it.S = c.S;
+            b.item[i] = it;
+            b.first[i] = total;
+            total += (int)mqs_workgroups(it.n, it.gw, c.S, c.T);
+        }
+        b.first[c.nb] = total;
+        b.count = c.nb;
+#define CONEF_MQS(RP)                                                                                               \
+    do {                                                                                                            \
+        if (RP >= 16) break;                                                                                        \
+        if (c.T == 256)                                                                                             \
+            hipLaunchKernelGGL((psgd_mqs_batch_kernel<(RP < 16 ? RP : 8), MODE, 256>), dim3((unsigned)total), dim3(256),  \
+                               c.lds, s, b, alpha, hs);                                                             \
+        else                                                                                                        \
+            hipLaunchKernelGGL((psgd_mqs_batch_kernel<(RP < 16 ? RP : 8), MODE, 1024>), dim3((unsigned)total), dim3(1024), \
+                               c.lds, s, b, alpha, hs);                                                             \
+    } while (0)
+        CONEF_RANK_SWITCH(rp, CONEF_MQS)
+#undef CONEF_MQS
+    }
+    return (int)hipGetLastError();
+}
+
 template <int MODE>
 int launch_mq(float* x, const float* err, const float* cs, const uint32_t* pktab, const float* q, float* p, int64_t n,
               int64_t m, int r, int32_t w, float alpha, ConefSeeds hs, void* workspace, int64_t workspace_bytes,
@@ -1298,8 +1390,14 @@ int launch_mq(float* x, const float* err, const float* cs, const uint32_t* pktab
     }
     const bool fast = r == rank_bound(r) && m % 4 == 0 && aligned16(x) && aligned16(q) && (MODE != 1 || aligned16(err)) &&
                       (!pktab || aligned16(pktab));
-    // rows per workgroup: 4 amortises the Q traffic, but small matrices need the workgroups
     const int rp = rank_bound(r);
+    if (fast && rp < 16) {
+        std::vector<MqsItem> one(1);
+        one[0] = MqsItem{x, err, cs, pktab, q, p, n, (int)m, (int)(MODE == 2 ? w : 1), 0, 0, mod};
+        const int rc = mqs_run<MODE>(one, rp, alpha, hs, s);
+        if (rc != kMqsNoFit) return rc;
+    }
+    // rows per workgroup: 4 amortises the Q traffic, but small matrices need the workgroups
     int rb = rp >= 32 ? 2 : 4;
     if (n / rb < 256) rb = rp >= 32 ? 2 : 1;
     size_t lds = (size_t)4 * rb * rp * 4 + (MODE == 2 ? (size_t)rb * w * 4 : 0);
@@ -2215,6 +2313,19 @@ int mq_batch(const ConefPsgdItem* items, int count, float alpha, int32_t a, int3
             members.push_back(j);
             rows += items[j].n;
             done[(size_t)j] = 1;
+        }
+        if (fast) {
+            std::vector<MqsItem> stream_table;
+            for (int j : members) {
+                const ConefPsgdItem& it = items[j];
+                stream_table.push_back(MqsItem{it.x, it.err, it.cs, item_pktab(it), it.q, it.p, it.n, (int)it.m,
+                                               (int)(MODE == 2 ? it.w : 1), 0, 0, conef_make_mod(MODE == 2 ? it.w : 1)});
+            }
+            const int rc = mqs_run<MODE>(stream_table, rp, alpha, hs, s);
+            if (rc != kMqsNoFit) {
+                if (rc != CONEF_OK) return rc;
+                continue;
+            }
         }
         const int rb = mq_rows_per_wg(rows);
         std::vector<MqItem> table;

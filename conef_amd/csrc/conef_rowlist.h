@@ -4,7 +4,8 @@
 // scatters the same way.  A plan built once per sketch lists, per bucket, the columns that fall
 // into it (ascending).  A workgroup then takes a tile of `rb` consecutive rows:
 //
-//   (the bucket lists and their offsets are copied into LDS first: d + w small integers)
+//   (the bucket lists and their offsets, d + w small integers, are requested first and parked in
+//   LDS once the tile is staged)
 //   stage   the values to be sketched are produced in column order with 16-byte accesses and
 //           parked in LDS; whatever the fused step has to do in column order (payload, writing
 //           the decompressed gradient, the low-rank product) happens here;
@@ -295,9 +296,23 @@ conef_rowlist_body(const Front& front, ConefRowlistView plan, const CsT* cs_in, 
     const int64_t row0 = (int64_t)bx * rb;
     const int rows = n - row0 < rb ? (int)(n - row0) : rb;
 
-    // the bucket lists, two entries per load (the table is padded to a multiple of 256 bytes)
-    conef_copy_words_to_lds(reinterpret_cast<uint32_t*>(ent_l), reinterpret_cast<const uint32_t*>(plan.ent), (d + 1) >> 1);
-    conef_copy_words_to_lds(csr_l, plan.csr, w + 1);
+    // The bucket lists (two entries per load; the table is padded to a multiple of 256 bytes) and
+    // their offsets are only needed by the walk: the first words of both are requested now and
+    // parked after the tile has been staged, so that they travel while the tile does.
+    constexpr int kPreE = 8, kPreC = 2;
+    const int ent_words = (d + 1) >> 1, csr_words = w + 1;
+    const uint32_t* ent_src = reinterpret_cast<const uint32_t*>(plan.ent);
+    uint32_t ent_pre[kPreE], csr_pre[kPreC];
+#pragma unroll
+    for (int u = 0; u < kPreE; ++u) {
+        const int i = threadIdx.x + u * kConefRowlistThreads;
+        ent_pre[u] = ent_src[i < ent_words ? i : ent_words - 1];
+    }
+#pragma unroll
+    for (int u = 0; u < kPreC; ++u) {
+        const int i = threadIdx.x + u * kConefRowlistThreads;
+        csr_pre[u] = plan.csr[i < csr_words ? i : csr_words - 1];
+    }
     if (Front::kNeedsCells) {
         const CsT* src = cs_in + row0 * w;
         const int count = rows * w;
@@ -330,6 +345,25 @@ conef_rowlist_body(const Front& front, ConefRowlistView plan, const CsT* cs_in, 
         }
     }
     front.stage(row0, rows, d, w, vals, cells, plan.pk);
+    {
+        uint32_t* ent_w = reinterpret_cast<uint32_t*>(ent_l);
+#pragma unroll
+        for (int u = 0; u < kPreE; ++u) {
+            const int i = threadIdx.x + u * kConefRowlistThreads;
+            if (i < ent_words) ent_w[i] = ent_pre[u];
+        }
+#pragma unroll
+        for (int u = 0; u < kPreC; ++u) {
+            const int i = threadIdx.x + u * kConefRowlistThreads;
+            if (i < csr_words) csr_l[i] = csr_pre[u];
+        }
+        if (ent_words > kPreE * kConefRowlistThreads)
+            conef_copy_words_to_lds(ent_w + kPreE * kConefRowlistThreads, ent_src + kPreE * kConefRowlistThreads,
+                                    ent_words - kPreE * kConefRowlistThreads);
+        if (csr_words > kPreC * kConefRowlistThreads)
+            conef_copy_words_to_lds(csr_l + kPreC * kConefRowlistThreads, plan.csr + kPreC * kConefRowlistThreads,
+                                    csr_words - kPreC * kConefRowlistThreads);
+    }
     if (!Front::kNeedsCells) {
 #pragma unroll
         for (int u = 0; u < kPre; ++u) {
