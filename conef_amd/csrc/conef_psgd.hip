@@ -10,6 +10,7 @@
 // error-feedback add (before the first product) and the residual (after the last) are fused into
 // the passes that touch M anyway.  Sums that cross workgroups meet through a caller-provided
 // workspace in a fixed order: no atomics, results do not change from run to run.
+#include <cstdlib>
 #include <type_traits>
 #include <algorithm>
 #include <atomic>
@@ -409,6 +410,147 @@ psgd_sum_partials_batch_kernel(PsgdBatch<SumItem> b)
     int local;
     const SumItem& it = b.item[psgd_batch_locate(b, &local)];
     psgd_sum_partials_body(it.partial, it.out, it.count, it.slabs, local);
+}
+
+// --------------------------------------- orthogonalisation of P, deferred ----
+// The reference orthogonalises P between the two products (powerSGD_hook.py:516-531): a chain of
+// r column steps over a tall thin matrix, all latency, with the machine idle around it.  Both
+// things it feeds are linear in P: with P' = P T (T the upper triangular matrix of the column
+// steps), Q = M^T P' = (M^T P) T.  So the round computes Q from the raw P at once, and gets T from
+// the Gram matrix P^T P alone (conef_gs_gram.h): the first product leaves each workgroup's share of
+// it, a workgroup per matrix riding in the second product's launch adds the shares and runs the r
+// steps on the r x r matrix, and one short launch then applies T to the rows of P and of the raw Q
+// (adding up Q's row-slab partials on the way, which was a launch of its own before).
+struct GramTask {
+    const double* parts[kPsgdBatchMax];   // [nparts][RP (RP + 1) / 2]
+    int nparts[kPsgdBatchMax];
+    float* tmat[kPsgdBatchMax];           // out: b_ij row-major [RP][RP] (zero unless i < j), then 1 / d_i [RP]
+    int count;
+    float eps;
+};
+
+template <int RP, int T>
+__device__ __forceinline__ void
+gram_solve_body(const double* __restrict__ parts, int nparts, float* __restrict__ tmat, float eps)
+{
+    constexpr int NG = RP * (RP + 1) / 2;
+    constexpr int G = T / NG;                 // groups of NG threads that add shares side by side
+    __shared__ double psum[G][NG];
+    __shared__ double gram[RP][RP + 1];
+    __shared__ __attribute__((aligned(16))) float coef[RP][RP];
+    __shared__ double dinv[RP];
+    __shared__ float dinvf[RP];
+    const int tid = threadIdx.x;
+    const int grp = tid / NG, e = tid - grp * NG;
+    if (grp < G) {
+        double s = 0.;
+#pragma unroll 8
+        for (int p = grp; p < nparts; p += G) s += parts[(size_t)p * NG + e];
+        psum[grp][e] = s;
+    }
+    for (int i = tid; i < RP * RP; i += T) (&coef[0][0])[i] = 0.f;
+    __syncthreads();
+    if (tid < NG) {
+        double s = 0.;
+        for (int g = 0; g < G; ++g) s += psum[g][tid];       // the same order on every run
+        int i, j;
+        gsg_entry(tid, RP, &i, &j);
+        gram[i][j] = s;
+    }
+    __syncthreads();
+    gsg_recurrence<RP, T>(gram, coef, dinv, dinvf, eps, tid);
+    for (int i = tid; i < RP * RP; i += T) tmat[i] = (&coef[0][0])[i];
+    if (tid < RP) tmat[RP * RP + tid] = dinvf[tid];
+}
+
+template <int RP, bool FAST>
+__global__ void __launch_bounds__(kMtpThreads)
+psgd_mtp_gram_batch_kernel(PsgdBatch<MtpItem> b, GramTask g)
+{
+    if ((int)blockIdx.x < g.count) {
+        gram_solve_body<RP, kMtpThreads>(g.parts[blockIdx.x], g.nparts[blockIdx.x], g.tmat[blockIdx.x], g.eps);
+        return;
+    }
+    const int bx = (int)blockIdx.x - g.count;
+    int i = 0;
+    while (i + 1 < b.count && bx >= b.first[i + 1]) ++i;
+    const MtpItem& it = b.item[i];
+    const int local = bx - b.first[i];
+    psgd_mtp_body<RP, FAST>(it.x, it.p, it.out, it.n, it.m, it.r, it.rows_per_slab, local % it.col_tiles,
+                            local / it.col_tiles);
+}
+
+// rows of P and of the raw Q times T, a row a thread: x_k -= b_ik x_i (k > i), x_i *= 1 / d_i for
+// i = 0 .. r - 1, the reference's column steps (powerSGD_hook.py:21-43) with the coefficients known
+struct DeferFixItem {
+    float* p;
+    const float* qsrc;       // [slabs][m][RP] partials of Q = M^T P, or q itself with one slab
+    float* q;
+    const float* tmat;
+    int64_t n, m;
+    int slabs;
+    int pblocks;             // workgroups that take rows of P; the others take rows of Q
+};
+
+template <int RP>
+__global__ void __launch_bounds__(256)
+psgd_defer_fix_batch_kernel(PsgdBatch<DeferFixItem> b)
+{
+    __shared__ float t_l[RP * RP + RP];
+    int local;
+    const DeferFixItem& it = b.item[psgd_batch_locate(b, &local)];
+    const bool is_p = local < it.pblocks;
+    const int64_t rows = is_p ? it.n : it.m;
+    const int64_t row = (int64_t)(is_p ? local : local - it.pblocks) * 256 + threadIdx.x;
+    const int64_t rc = row < rows ? row : rows - 1;
+    const float* src = is_p ? it.p : it.qsrc;
+    const int slabs = is_p ? 1 : it.slabs;
+    const int64_t stride = it.m * RP;
+    float x[RP];
+#pragma unroll
+    for (int c = 0; c < RP; ++c) x[c] = 0.f;
+    int sl = 0;
+    for (; sl + 4 <= slabs; sl += 4) {                      // slabs in ascending order, four requested together
+        float v[4][RP];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float* rp = src + (int64_t)(sl + u) * stride + rc * RP;
+            if (RP >= 4) {
+#pragma unroll
+                for (int c = 0; c < RP; c += 4) ld4(rp + c, &v[u][c]);
+            } else {
+#pragma unroll
+                for (int c = 0; c < RP; ++c) v[u][c] = rp[c];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int c = 0; c < RP; ++c) x[c] += v[u][c];
+    }
+    for (; sl < slabs; ++sl) {
+        const float* rp = src + (int64_t)sl * stride + rc * RP;
+#pragma unroll
+        for (int c = 0; c < RP; ++c) x[c] += rp[c];
+    }
+    if (threadIdx.x < RP * RP + RP) t_l[threadIdx.x] = it.tmat[threadIdx.x];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < RP; ++i) {
+#pragma unroll
+        for (int k = i + 1; k < RP; ++k) x[k] = fmaf(-t_l[i * RP + k], x[i], x[k]);
+        x[i] = __fmul_rn(x[i], t_l[RP * RP + i]);
+    }
+    if (row < rows) {
+        float* dst = (is_p ? it.p : it.q) + row * RP;
+        if (RP >= 4) {
+#pragma unroll
+            for (int c = 0; c < RP; c += 4) st4(dst + c, &x[c]);
+        } else {
+#pragma unroll
+            for (int c = 0; c < RP; ++c) dst[c] = x[c];
+        }
+    }
 }
 
 // ------------------------------------------- matrix-core products, batched ----
@@ -1309,7 +1451,7 @@ constexpr size_t kMfmaMqLdsLimit = 144 * 1024;
 constexpr int kMqsNoFit = -100;
 
 template <int MODE>
-int mqs_run(const std::vector<MqsItem>& table, int rp, float alpha, ConefSeeds hs, hipStream_t s)
+int mqs_run(const std::vector<MqsItem>& table, int rp, float alpha, ConefSeeds hs, hipStream_t s, bool gram = false)
 {
     struct Chunk { size_t k; int nb, T, S; size_t lds; };
     std::vector<Chunk> chunks;
@@ -1317,7 +1459,7 @@ int mqs_run(const std::vector<MqsItem>& table, int rp, float alpha, ConefSeeds h
         Chunk c;
         c.k = k;
         c.nb = (int)std::min(table.size() - k, (size_t)kPsgdBatchMax);
-        if (!mqs_plan_launch(&table[k], c.nb, rp, MODE == 2, &c.T, &c.S, &c.lds)) return kMqsNoFit;
+        if (!mqs_plan_launch(&table[k], c.nb, rp, MODE == 2, &c.T, &c.S, &c.lds, gram)) return kMqsNoFit;
         chunks.push_back(c);
         k += (size_t)c.nb;
     }
@@ -2386,7 +2528,17 @@ inline int64_t mtp_batch_layout(const ConefPsgdItem* items, int count, std::vect
     return off;
 }
 
-int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t workspace_bytes, hipStream_t s)
+// `gram` (deferred orthogonalisation of P): count workgroups in front of the launch solve the
+// matrices' Gram systems, and the row-slab partials are left for the caller's fix launch instead
+// of being added here; outs[k] then says where item k's raw Q is ([slabs][m][r]).  Only for a batch
+// that is one launch of this kernel (one rank below 16, all items 16-byte shaped or none).
+struct MtpRaw {
+    const float* src;
+    int slabs;
+};
+
+int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t workspace_bytes, hipStream_t s,
+              const GramTask* gram = nullptr, std::vector<MtpRaw>* outs = nullptr)
 {
     std::vector<MtpPlan> plans;
     const int64_t floats = mtp_batch_layout(items, count, &plans);
@@ -2460,7 +2612,8 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
             MtpItem t = {it.x, it.p, out, it.n, (int)it.m, it.r, pl.g.rows_per_slab, pl.g.col_tiles};
             table.push_back(t);
             blocks.push_back(pl.g.col_tiles * pl.g.slabs);
-            if (pl.partial_off >= 0) {
+            if (outs) (*outs)[(size_t)j] = MtpRaw{out, pl.partial_off >= 0 ? pl.g.slabs : 1};
+            if (pl.partial_off >= 0 && !gram) {
                 int64_t cnt = it.m * it.r;
                 SumItem si = {out, it.q, cnt, pl.g.slabs};
                 sums.push_back(si);
@@ -2472,7 +2625,11 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
 #define CONEF_MTPB(RP)                                                                                              \
     do {                                                                                                            \
         if (RP >= 16) break;                                                                                        \
-        if (fast) rc = run_batches(table, blocks, [&](const PsgdBatch<MtpItem>& bt, int grid) {                     \
+        if (gram) rc = run_batches(table, blocks, [&](const PsgdBatch<MtpItem>& bt, int grid) {                     \
+            if (fast) hipLaunchKernelGGL((psgd_mtp_gram_batch_kernel<(RP < 16 ? RP : 8), true>), dim3((unsigned)(grid + gram->count)), dim3(kMtpThreads), 0, s, bt, *gram); \
+            else hipLaunchKernelGGL((psgd_mtp_gram_batch_kernel<(RP < 16 ? RP : 8), false>), dim3((unsigned)(grid + gram->count)), dim3(kMtpThreads), 0, s, bt, *gram); \
+        });                                                                                                         \
+        else if (fast) rc = run_batches(table, blocks, [&](const PsgdBatch<MtpItem>& bt, int grid) {                \
             hipLaunchKernelGGL((psgd_mtp_batch_kernel<(RP < 16 ? RP : 8), true>), dim3((unsigned)grid), dim3(kMtpThreads), 0, s, bt); \
         });                                                                                                         \
         else rc = run_batches(table, blocks, [&](const PsgdBatch<MtpItem>& bt, int grid) {                          \
@@ -2490,6 +2647,116 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
         if (rc != CONEF_OK) return rc;
     }
     return CONEF_OK;
+}
+
+// ---- deferred orthogonalisation of P: host side ----
+// The end of a batch workspace holds the Gram shares (a workgroup of the first product each; at
+// most one per four rows) and the solved systems, 512 bytes a matrix.
+constexpr int64_t kDeferTmatBytes = 512;
+
+inline int64_t defer_gram_doubles(const ConefPsgdItem& it)
+{
+    const int rp = rank_bound(it.r);
+    return ((it.n + 3) / 4) * (int64_t)(rp * (rp + 1) / 2);
+}
+
+inline int64_t defer_region_bytes(const ConefPsgdItem* items, int count)
+{
+    int64_t bytes = 0;
+    for (int k = 0; k < count; ++k)
+        if (rank_bound(items[k].r) <= 8) bytes += conef_align256(8 * defer_gram_doubles(items[k])) + kDeferTmatBytes;
+    return bytes;
+}
+
+inline int64_t defer_region_offset(const ConefPsgdItem* items, int count)
+{
+    int64_t single = 256;
+    for (int k = 0; k < count; ++k) {
+        int64_t b = conef_psgd_workspace_bytes(items[k].n, items[k].m, items[k].r);
+        if (b > single) single = b;
+    }
+    return conef_align256(single) + conef_align256(4 * mtp_batch_layout(items, count, nullptr)) +
+           conef_align256(4 * mfma_batch_layout(items, count, nullptr));
+}
+
+// P = X Q (raw) with the Gram shares, Q = X^T P (raw) with the systems solved on the side, then T
+// applied to both.  `mq_items` differ from `items` in q only: the Q the first product reads.
+// kMqsNoFit with nothing launched: the batch is not one this path takes (ranks
+// above 8 or mixed, shapes without 16-byte accesses, a workspace without the region above).
+template <int MODE>
+int round_products_deferred(const ConefPsgdItem* items, const ConefPsgdItem* mq_items, int count, float alpha, float eps,
+                            int32_t a, int32_t b, void* workspace, int64_t workspace_bytes, hipStream_t s)
+{
+    if (count < 1 || count > kPsgdBatchMax || !workspace) return kMqsNoFit;
+    const int rp = rank_bound(items[0].r);
+    if (rp > 8) return kMqsNoFit;
+    const int ng = rp * (rp + 1) / 2;
+    const int64_t region = defer_region_offset(items, count);
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0 || workspace_bytes < region + defer_region_bytes(items, count))
+        return kMqsNoFit;
+    ConefSeeds hs = {a, b, a + 2, b + 3};
+    std::vector<MqsItem> table;
+    std::vector<float*> tmats;
+    char* at = (char*)workspace + region;
+    for (int k = 0; k < count; ++k) {
+        const ConefPsgdItem& it = items[k];
+        const uint32_t* pk = MODE == 2 ? item_pktab(it) : nullptr;
+        const float* q_in = mq_items[k].q;       // the first product's Q (last round's, orthogonalised); it.q receives the new one
+        if (it.r != rp || it.m % 4 != 0 || it.n > 0x7fffffffLL || !aligned16(it.x) || !aligned16(it.q) || !aligned16(it.p) ||
+            !aligned16(q_in) || (MODE == 1 && !aligned16(it.err)) || (pk && !aligned16(pk)))
+            return kMqsNoFit;
+        MqsItem t = {it.x, it.err, it.cs, pk, q_in, it.p, it.n, (int)it.m, (int)(MODE == 2 ? it.w : 1), 0, 0,
+                     conef_make_mod(MODE == 2 ? it.w : 1), (double*)at};
+        table.push_back(t);
+        at += conef_align256(8 * defer_gram_doubles(it));
+        tmats.push_back((float*)at);
+        at += kDeferTmatBytes;
+    }
+    int T, S;
+    size_t lds;
+    if (!mqs_plan_launch(table.data(), count, rp, MODE == 2, &T, &S, &lds, true)) return kMqsNoFit;
+    // the second product must be the 16-byte form of one launch, its partials inside the workspace
+    std::vector<MtpPlan> plans;
+    const int64_t mtp_floats = mtp_batch_layout(items, count, &plans);
+    if (workspace_bytes < 4 * mtp_floats) return kMqsNoFit;
+    for (int k = 0; k < count; ++k) {
+        const float* out = plans[(size_t)k].partial_off >= 0 ? (const float*)workspace + plans[(size_t)k].partial_off : items[k].q;
+        if (!aligned16(out)) return kMqsNoFit;
+    }
+
+    int rc = mqs_run<MODE>(table, rp, alpha, hs, s, true);
+    if (rc != CONEF_OK) return rc;         // mqs_plan_launch above is the same decision: not kMqsNoFit here
+    GramTask gram;
+    gram.count = count;
+    gram.eps = eps;
+    for (int k = 0; k < count; ++k) {
+        const int gw = mqs_group_width(items[k].m, T);
+        gram.parts[k] = table[(size_t)k].gram;
+        gram.nparts[k] = (int)mqs_workgroups(items[k].n, gw, S, T);
+        gram.tmat[k] = tmats[(size_t)k];
+    }
+    std::vector<MtpRaw> raw((size_t)count);
+    rc = mtp_batch(items, count, workspace, workspace_bytes, s, &gram, &raw);
+    if (rc != CONEF_OK) return rc;
+    std::vector<DeferFixItem> fix;
+    std::vector<int> blocks;
+    for (int k = 0; k < count; ++k) {
+        const ConefPsgdItem& it = items[k];
+        const int pb = (int)((it.n + 255) / 256), qb = (int)((it.m + 255) / 256);
+        fix.push_back(DeferFixItem{it.p, raw[(size_t)k].src, it.q, tmats[(size_t)k], it.n, it.m, raw[(size_t)k].slabs, pb});
+        blocks.push_back(pb + qb);
+    }
+    (void)ng;
+#define CONEF_DFX(RP)                                                                                               \
+    do {                                                                                                            \
+        if (RP >= 16) break;                                                                                        \
+        rc = run_batches(fix, blocks, [&](const PsgdBatch<DeferFixItem>& bt, int grid) {                            \
+            hipLaunchKernelGGL((psgd_defer_fix_batch_kernel<(RP < 16 ? RP : 8)>), dim3((unsigned)grid), dim3(256), 0, s, bt); \
+        });                                                                                                         \
+    } while (0)
+    CONEF_RANK_SWITCH(rp, CONEF_DFX)
+#undef CONEF_DFX
+    return rc;
 }
 
 template <int RP, bool FAST>
@@ -2761,7 +3028,7 @@ int64_t conef_psgd_batch_workspace_bytes(const ConefPsgdItem* items, int32_t cou
         if (b > single) single = b;
     }
     return conef_align256(single) + conef_align256(4 * mtp_batch_layout(items, count, nullptr)) +
-           conef_align256(4 * mfma_batch_layout(items, count, nullptr));
+           conef_align256(4 * mfma_batch_layout(items, count, nullptr)) + defer_region_bytes(items, count);
 }
 
 int conef_psgd_mq_batch_f32(const ConefPsgdItem* items, int32_t count, int32_t mode, float alpha, int32_t a, int32_t b,
@@ -2865,6 +3132,38 @@ int conef_psgd_round_ahead_f32(const ConefPsgdItem* items, int32_t count, int32_
         rows[(size_t)k] = items[k].m;
         ranks[(size_t)k] = items[k].r;
     }
+    // P = X Q, P orthogonalised, Q = X^T P: with the orthogonalisation deferred where the batch
+    // allows (round_products_deferred; CONEF_ROUND_DEFER=0 keeps the reference's order of steps,
+    // for comparisons), else as three steps
+    static const bool defer_on = [] {
+        const char* e = getenv("CONEF_ROUND_DEFER");
+        return !(e && e[0] == '0');
+    }();
+    auto products = [&](const ConefPsgdItem* its) -> int {      // its: the items with the Q the first product reads
+        if (mq_mode < 0 || mq_mode > 2) return CONEF_ERR_INVALID;
+        for (int k = 0; k < count; ++k) {
+            const ConefPsgdItem& it = its[k];
+            if ((mq_mode == 1 && !it.err) || (mq_mode == 2 && (!it.cs || it.w < 1 || it.w > (1 << 30)))) return CONEF_ERR_INVALID;
+            if (mq_mode == 2 && it.plan_host && !conef_plan_matches((const ConefPlanHeader*)it.plan_host, it.n, it.m, it.w, a, b))
+                return CONEF_ERR_INVALID;
+        }
+        if (defer_on) {
+            hipStream_t hs = (hipStream_t)stream;
+            const int rd = mq_mode == 0   ? round_products_deferred<0>(items, its, count, 0.f, eps, a, b, workspace, workspace_bytes, hs)
+                           : mq_mode == 1 ? round_products_deferred<1>(items, its, count, 0.f, eps, a, b, workspace, workspace_bytes, hs)
+                                          : round_products_deferred<2>(items, its, count, alpha, eps, a, b, workspace, workspace_bytes, hs);
+            if (rd != kMqsNoFit) return rd;
+        }
+        int rp = conef_psgd_mq_batch_f32(its, count, mq_mode, alpha, a, b, workspace, workspace_bytes, stream);
+        if (rp != CONEF_OK) return rp;
+        for (int k = 0; k < count; ++k) {
+            mats[(size_t)k] = items[k].p;
+            rows[(size_t)k] = items[k].n;
+        }
+        rp = conef_gram_schmidt_batch_f32(mats.data(), rows.data(), ranks.data(), count, eps, workspace, workspace_bytes, stream);
+        if (rp != CONEF_OK) return rp;
+        return conef_psgd_mtp_batch_f32(items, count, workspace, workspace_bytes, stream);
+    };
     int rc = CONEF_OK;
     if (flags & CONEF_ROUND_Q_READY) {
         // q_next holds this round's Q factors, orthogonalised at the end of the bucket's last round
@@ -2873,20 +3172,12 @@ int conef_psgd_round_ahead_f32(const ConefPsgdItem* items, int32_t count, int32_
             if (!q_next[k]) return CONEF_ERR_INVALID;
             with_q[(size_t)k].q = q_next[k];
         }
-        rc = conef_psgd_mq_batch_f32(with_q.data(), count, mq_mode, alpha, a, b, workspace, workspace_bytes, stream);
+        rc = products(with_q.data());
     } else {
         rc = conef_gram_schmidt_batch_f32(mats.data(), rows.data(), ranks.data(), count, eps, workspace, workspace_bytes, stream);
         if (rc != CONEF_OK) return rc;
-        rc = conef_psgd_mq_batch_f32(items, count, mq_mode, alpha, a, b, workspace, workspace_bytes, stream);
+        rc = products(items);
     }
-    if (rc != CONEF_OK) return rc;
-    for (int k = 0; k < count; ++k) {
-        mats[(size_t)k] = items[k].p;
-        rows[(size_t)k] = items[k].n;
-    }
-    rc = conef_gram_schmidt_batch_f32(mats.data(), rows.data(), ranks.data(), count, eps, workspace, workspace_bytes, stream);
-    if (rc != CONEF_OK) return rc;
-    rc = conef_psgd_mtp_batch_f32(items, count, workspace, workspace_bytes, stream);
     if (rc != CONEF_OK) return rc;
     // The new Q factors orthogonalised into q_next by workgroups of the last launch: only where that
     // launch covers the whole bucket (one rank, at most 8) and every Q factor is short.

@@ -38,6 +38,9 @@ struct MqsItem {
     int m, w;
     int gw, S;               // threads of a group, rows of a group (multiple of 4)
     ConefMod mod;
+    // not null: workgroup g of the matrix also leaves the upper triangle of (its rows of P)^T (its
+    // rows of P), RP (RP + 1) / 2 doubles, at gram[g * RP (RP + 1) / 2]: the shares of P^T P
+    double* gram;
 };
 
 // threads of a group for a matrix of m columns in a workgroup of T threads
@@ -62,18 +65,20 @@ inline int64_t mqs_workgroups(int64_t n, int gw, int S, int T)
     return (n + rows - 1) / rows;
 }
 
-inline size_t mqs_lds_bytes(int64_t m, int w, int gw, int S, int T, int rp, bool sketch)
+inline size_t mqs_lds_bytes(int64_t m, int w, int gw, int S, int T, int rp, bool sketch, bool gram = false)
 {
     const int64_t m4 = m >> 2;
     const int64_t niter = (m4 + gw - 1) / gw * (S >> 2);
-    return (size_t)niter * (T / 64) * 4 * rp * 4 + (sketch ? (size_t)(T / gw) * S * w * 4 : 0);
+    return (size_t)niter * (T / 64) * 4 * rp * 4 + (sketch ? (size_t)(T / gw) * S * w * 4 : 0) +
+           (gram ? (size_t)(T / gw) * S * rp * 4 : 0);
 }
 
 // Workgroup size and rows per group for one launch over `count` matrices.  Wide matrices need the
 // threads of a large workgroup side by side; rows per group are as many as still leave the launch
 // enough workgroups, and as the parked sketch rows leave room for in LDS.  False: no geometry fits,
 // or the matrices are too small for this kernel to pay.
-inline bool mqs_plan_launch(const MqsItem* items, int count, int rp, bool sketch, int* T_out, int* S_out, size_t* lds_out)
+inline bool mqs_plan_launch(const MqsItem* items, int count, int rp, bool sketch, int* T_out, int* S_out, size_t* lds_out,
+                            bool gram = false)
 {
     int T = 256;
     for (int k = 0; k < count; ++k)
@@ -85,7 +90,7 @@ inline bool mqs_plan_launch(const MqsItem* items, int count, int rp, bool sketch
         for (int k = 0; k < count; ++k) {
             const int gw = mqs_group_width(items[k].m, T);
             wgs += mqs_workgroups(items[k].n, gw, S, T);
-            const size_t need = mqs_lds_bytes(items[k].m, items[k].w, gw, S, T, rp, sketch);
+            const size_t need = mqs_lds_bytes(items[k].m, items[k].w, gw, S, T, rp, sketch, gram);
             if (need > lds) lds = need;
         }
         if (lds > 64 * 1024) continue;
@@ -238,6 +243,7 @@ psgd_mqs_body(const MqsItem& it, float alpha, ConefSeeds hs, int bx)
     }
     __syncthreads();
     const int wpg = gw >> 6;                               // waves of a group
+    float* prow = cells + (MODE == 2 ? (size_t)groups * S * w : 0);   // [groups * S][RP], only with it.gram
     for (int o = tid; o < rows_here * RP; o += T) {
         const int lr = o / RP, c = o - lr * RP;
         const int gg = lr / S, rr = lr - gg * S;
@@ -248,5 +254,21 @@ psgd_mqs_body(const MqsItem& it, float alpha, ConefSeeds hs, int bx)
             for (int v = 0; v < wpg; ++v) s += base[(size_t)v * NV];
         }
         it.p[(wg_row0 + lr) * RP + c] = s;
+        if (it.gram) prow[o] = s;
+    }
+    if (it.gram) {
+        constexpr int NG = RP * (RP + 1) / 2;
+        __syncthreads();
+        if (tid < NG) {
+            int i = 0, e0 = 0;                             // entry tid of the row-major upper triangle is (i, j)
+            while (tid >= e0 + RP - i) {
+                e0 += RP - i;
+                ++i;
+            }
+            const int j = i + (tid - e0);
+            double s = 0.;
+            for (int lr = 0; lr < rows_here; ++lr) s = fma((double)prow[lr * RP + i], (double)prow[lr * RP + j], s);
+            it.gram[(size_t)bx * NG + tid] = s;
+        }
     }
 }
