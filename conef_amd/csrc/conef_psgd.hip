@@ -429,9 +429,11 @@ struct GramTask {
     float eps;
 };
 
+// adds the shares, runs the r steps, leaves b_ij [RP][RP] and 1 / d_i [RP] in t_l (LDS, RP RP + RP
+// floats), visible to every thread on return; all T threads of the workgroup call this
 template <int RP, int T>
 __device__ __forceinline__ void
-gram_solve_body(const double* __restrict__ parts, int nparts, float* __restrict__ tmat, float eps)
+gram_solve_lds(const double* __restrict__ parts, int nparts, float eps, float* t_l)
 {
     constexpr int NG = RP * (RP + 1) / 2;
     constexpr int G = T / NG;                 // groups of NG threads that add shares side by side
@@ -459,8 +461,80 @@ gram_solve_body(const double* __restrict__ parts, int nparts, float* __restrict_
     }
     __syncthreads();
     gsg_recurrence<RP, T>(gram, coef, dinv, dinvf, eps, tid);
-    for (int i = tid; i < RP * RP; i += T) tmat[i] = (&coef[0][0])[i];
-    if (tid < RP) tmat[RP * RP + tid] = dinvf[tid];
+    for (int i = tid; i < RP * RP; i += T) t_l[i] = (&coef[0][0])[i];
+    if (tid < RP) t_l[RP * RP + tid] = dinvf[tid];
+    __syncthreads();
+}
+
+template <int RP, int T>
+__device__ __forceinline__ void
+gram_solve_body(const double* __restrict__ parts, int nparts, float* __restrict__ tmat, float eps)
+{
+    __shared__ float t_l[RP * RP + RP];
+    gram_solve_lds<RP, T>(parts, nparts, eps, t_l);
+    for (int i = threadIdx.x; i < RP * RP + RP; i += T) tmat[i] = t_l[i];
+}
+
+// x_k -= b_ik x_i (k > i), x_i *= 1 / d_i for i = 0 .. r - 1: the reference's column steps
+// (powerSGD_hook.py:21-43) on one row, coefficients from t_l as gram_solve_lds leaves them
+template <int RP>
+__device__ __forceinline__ void gram_apply_row(float* x, const float* t_l)
+{
+#pragma unroll
+    for (int i = 0; i < RP; ++i) {
+#pragma unroll
+        for (int k = i + 1; k < RP; ++k) x[k] = fmaf(-t_l[i * RP + k], x[i], x[k]);
+        x[i] = __fmul_rn(x[i], t_l[RP * RP + i]);
+    }
+}
+
+template <int RP>
+__device__ __forceinline__ void load_row(const float* p, float* x)
+{
+    if (RP >= 4) {
+#pragma unroll
+        for (int c = 0; c < RP; c += 4) ld4(p + c, x + c);
+    } else {
+#pragma unroll
+        for (int c = 0; c < RP; ++c) x[c] = p[c];
+    }
+}
+
+template <int RP>
+__device__ __forceinline__ void store_row(float* p, const float* x)
+{
+    if (RP >= 4) {
+#pragma unroll
+        for (int c = 0; c < RP; c += 4) st4(p + c, x + c);
+    } else {
+#pragma unroll
+        for (int c = 0; c < RP; ++c) p[c] = x[c];
+    }
+}
+
+// A whole matrix orthogonalised out of place by one workgroup of T threads from the shares of its
+// Gram matrix: solve, then the column steps row by row (four rows a thread in flight).
+template <int RP, int T>
+__device__ __forceinline__ void
+gram_orthogonalise_body(const float* __restrict__ src, float* __restrict__ dst, int rows, const double* parts, int nparts,
+                        float eps)
+{
+    __shared__ float t_l[RP * RP + RP];
+    gram_solve_lds<RP, T>(parts, nparts, eps, t_l);
+    for (int r0 = threadIdx.x; r0 < rows; r0 += 4 * T) {
+        float x[4][RP];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int row = r0 + u * T;
+            load_row<RP>(src + (int64_t)(row < rows ? row : rows - 1) * RP, x[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int row = r0 + u * T;
+            gram_apply_row<RP>(x[u], t_l);
+            if (row < rows) store_row<RP>(dst + (int64_t)row * RP, x[u]);
+        }
+    }
 }
 
 template <int RP, bool FAST>
@@ -487,6 +561,7 @@ struct DeferFixItem {
     const float* qsrc;       // [slabs][m][RP] partials of Q = M^T P, or q itself with one slab
     float* q;
     const float* tmat;
+    double* qgram;           // not null: the workgroups of Q also leave their rows' share of Q^T Q, [m / 256][RP (RP + 1) / 2]
     int64_t n, m;
     int slabs;
     int pblocks;             // workgroups that take rows of P; the others take rows of Q
@@ -496,7 +571,10 @@ template <int RP>
 __global__ void __launch_bounds__(256)
 psgd_defer_fix_batch_kernel(PsgdBatch<DeferFixItem> b)
 {
+    constexpr int NG = RP * (RP + 1) / 2;
     __shared__ float t_l[RP * RP + RP];
+    __shared__ float rows_l[256][RP + 1];
+    __shared__ double part_l[4][NG];
     int local;
     const DeferFixItem& it = b.item[psgd_batch_locate(b, &local)];
     const bool is_p = local < it.pblocks;
@@ -513,43 +591,38 @@ psgd_defer_fix_batch_kernel(PsgdBatch<DeferFixItem> b)
     for (; sl + 4 <= slabs; sl += 4) {                      // slabs in ascending order, four requested together
         float v[4][RP];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const float* rp = src + (int64_t)(sl + u) * stride + rc * RP;
-            if (RP >= 4) {
-#pragma unroll
-                for (int c = 0; c < RP; c += 4) ld4(rp + c, &v[u][c]);
-            } else {
-#pragma unroll
-                for (int c = 0; c < RP; ++c) v[u][c] = rp[c];
-            }
-        }
+        for (int u = 0; u < 4; ++u) load_row<RP>(src + (int64_t)(sl + u) * stride + rc * RP, v[u]);
 #pragma unroll
         for (int u = 0; u < 4; ++u)
 #pragma unroll
             for (int c = 0; c < RP; ++c) x[c] += v[u][c];
     }
     for (; sl < slabs; ++sl) {
-        const float* rp = src + (int64_t)sl * stride + rc * RP;
+        float v[RP];
+        load_row<RP>(src + (int64_t)sl * stride + rc * RP, v);
 #pragma unroll
-        for (int c = 0; c < RP; ++c) x[c] += rp[c];
+        for (int c = 0; c < RP; ++c) x[c] += v[c];
     }
     if (threadIdx.x < RP * RP + RP) t_l[threadIdx.x] = it.tmat[threadIdx.x];
     __syncthreads();
+    gram_apply_row<RP>(x, t_l);
+    if (row < rows) store_row<RP>((is_p ? it.p : it.q) + row * RP, x);
+    if (!is_p && it.qgram) {                                // uniform over the workgroup
 #pragma unroll
-    for (int i = 0; i < RP; ++i) {
-#pragma unroll
-        for (int k = i + 1; k < RP; ++k) x[k] = fmaf(-t_l[i * RP + k], x[i], x[k]);
-        x[i] = __fmul_rn(x[i], t_l[RP * RP + i]);
-    }
-    if (row < rows) {
-        float* dst = (is_p ? it.p : it.q) + row * RP;
-        if (RP >= 4) {
-#pragma unroll
-            for (int c = 0; c < RP; c += 4) st4(dst + c, &x[c]);
-        } else {
-#pragma unroll
-            for (int c = 0; c < RP; ++c) dst[c] = x[c];
+        for (int c = 0; c < RP; ++c) rows_l[threadIdx.x][c] = row < rows ? x[c] : 0.f;
+        __syncthreads();
+        const int e = threadIdx.x >> 2, quarter = threadIdx.x & 3;      // four threads an entry, 64 rows each
+        if (e < NG) {
+            int i, j;
+            gsg_entry(e, RP, &i, &j);
+            double s = 0.;
+            for (int t = quarter * 64; t < quarter * 64 + 64; ++t) s = fma((double)rows_l[t][i], (double)rows_l[t][j], s);
+            part_l[quarter][e] = s;
         }
+        __syncthreads();
+        if (threadIdx.x < NG)
+            it.qgram[(size_t)(local - it.pblocks) * NG + threadIdx.x] =
+                (part_l[0][threadIdx.x] + part_l[1][threadIdx.x]) + (part_l[2][threadIdx.x] + part_l[3][threadIdx.x]);
     }
 }
 
@@ -1158,7 +1231,25 @@ struct GsAhead {
     int rows[kPsgdBatchMax];
     int count, r;
     float eps;
+    // not null: the shares of src^T src are known (nparts of them); the matrix is then
+    // orthogonalised from its Gram matrix, whatever its height (gram_orthogonalise_body)
+    const double* parts[kPsgdBatchMax];
+    int nparts[kPsgdBatchMax];
 };
+
+template <int RP>
+__device__ __forceinline__ void gs_ahead_body(const GsAhead& g, int k)
+{
+    if (g.parts[k]) {
+        gram_orthogonalise_body<RP, kGsRegThreads>(g.src[k], g.dst[k], g.rows[k], g.parts[k], g.nparts[k], g.eps);
+        return;
+    }
+    // at most kGsAheadRowSlots rows a thread: the taller bodies hold over a hundred values in
+    // registers, and the host kernel's allocation is what every workgroup of its launch gets
+    __shared__ float red[2][4][RP];
+    if (g.rows[k] <= kGsRegThreads) gs_reg_body<RP, 1>(g.dst[k], g.rows[k], red, g.r, g.eps, g.src[k]);
+    else gs_reg_body<RP, kGsAheadRowSlots>(g.dst[k], g.rows[k], red, g.r, g.eps, g.src[k]);
+}
 
 // Matrices beyond one workgroup's registers: the same register-resident scheme over up to 128
 // workgroups launched cooperatively (all resident at once).  A column step ends with every
@@ -2660,11 +2751,21 @@ inline int64_t defer_gram_doubles(const ConefPsgdItem& it)
     return ((it.n + 3) / 4) * (int64_t)(rp * (rp + 1) / 2);
 }
 
+// shares of Q^T Q, one per 256 rows of Q (the fix launch leaves them for the workgroups that
+// orthogonalise Q for the bucket's next round)
+inline int64_t defer_qgram_doubles(const ConefPsgdItem& it)
+{
+    const int rp = rank_bound(it.r);
+    return ((it.m + 255) / 256) * (int64_t)(rp * (rp + 1) / 2);
+}
+
 inline int64_t defer_region_bytes(const ConefPsgdItem* items, int count)
 {
     int64_t bytes = 0;
     for (int k = 0; k < count; ++k)
-        if (rank_bound(items[k].r) <= 8) bytes += conef_align256(8 * defer_gram_doubles(items[k])) + kDeferTmatBytes;
+        if (rank_bound(items[k].r) <= 8)
+            bytes += conef_align256(8 * defer_gram_doubles(items[k])) + kDeferTmatBytes +
+                     conef_align256(8 * defer_qgram_doubles(items[k]));
     return bytes;
 }
 
@@ -2681,11 +2782,14 @@ inline int64_t defer_region_offset(const ConefPsgdItem* items, int count)
 
 // P = X Q (raw) with the Gram shares, Q = X^T P (raw) with the systems solved on the side, then T
 // applied to both.  `mq_items` differ from `items` in q only: the Q the first product reads.
+// q_shares (optional): the fix launch also leaves the shares of Q^T Q of the new Q factors; their
+// places are recorded in q_shares->parts / nparts.
 // kMqsNoFit with nothing launched: the batch is not one this path takes (ranks
 // above 8 or mixed, shapes without 16-byte accesses, a workspace without the region above).
 template <int MODE>
 int round_products_deferred(const ConefPsgdItem* items, const ConefPsgdItem* mq_items, int count, float alpha, float eps,
-                            int32_t a, int32_t b, void* workspace, int64_t workspace_bytes, hipStream_t s)
+                            int32_t a, int32_t b, void* workspace, int64_t workspace_bytes, hipStream_t s,
+                            GsAhead* q_shares)
 {
     if (count < 1 || count > kPsgdBatchMax || !workspace) return kMqsNoFit;
     const int rp = rank_bound(items[0].r);
@@ -2697,6 +2801,7 @@ int round_products_deferred(const ConefPsgdItem* items, const ConefPsgdItem* mq_
     ConefSeeds hs = {a, b, a + 2, b + 3};
     std::vector<MqsItem> table;
     std::vector<float*> tmats;
+    std::vector<double*> qgrams;
     char* at = (char*)workspace + region;
     for (int k = 0; k < count; ++k) {
         const ConefPsgdItem& it = items[k];
@@ -2711,6 +2816,8 @@ int round_products_deferred(const ConefPsgdItem* items, const ConefPsgdItem* mq_
         at += conef_align256(8 * defer_gram_doubles(it));
         tmats.push_back((float*)at);
         at += kDeferTmatBytes;
+        qgrams.push_back((double*)at);
+        at += conef_align256(8 * defer_qgram_doubles(it));
     }
     int T, S;
     size_t lds;
@@ -2743,8 +2850,13 @@ int round_products_deferred(const ConefPsgdItem* items, const ConefPsgdItem* mq_
     for (int k = 0; k < count; ++k) {
         const ConefPsgdItem& it = items[k];
         const int pb = (int)((it.n + 255) / 256), qb = (int)((it.m + 255) / 256);
-        fix.push_back(DeferFixItem{it.p, raw[(size_t)k].src, it.q, tmats[(size_t)k], it.n, it.m, raw[(size_t)k].slabs, pb});
+        fix.push_back(DeferFixItem{it.p, raw[(size_t)k].src, it.q, tmats[(size_t)k], q_shares ? qgrams[(size_t)k] : nullptr,
+                                   it.n, it.m, raw[(size_t)k].slabs, pb});
         blocks.push_back(pb + qb);
+        if (q_shares) {
+            q_shares->parts[k] = qgrams[(size_t)k];
+            q_shares->nparts[k] = qb;
+        }
     }
     (void)ng;
 #define CONEF_DFX(RP)                                                                                               \
@@ -2789,13 +2901,7 @@ psgd_residual_rowlist_gs_batch_kernel(PsgdBatch<RowlistResidualItem<RP, FAST>> b
 {
     static_assert(kConefRowlistThreads == kGsRegThreads, "one block size for both kinds of workgroup");
     if ((int)blockIdx.x < g.count) {
-        // at most kGsAheadRowSlots rows a thread: the taller bodies hold over a hundred values in
-        // registers, and this kernel's allocation is what every workgroup of the launch gets
-        __shared__ float red[2][4][RP];
-        if (g.rows[blockIdx.x] <= kGsRegThreads)
-            gs_reg_body<RP, 1>(g.dst[blockIdx.x], g.rows[blockIdx.x], red, g.r, g.eps, g.src[blockIdx.x]);
-        else
-            gs_reg_body<RP, kGsAheadRowSlots>(g.dst[blockIdx.x], g.rows[blockIdx.x], red, g.r, g.eps, g.src[blockIdx.x]);
+        gs_ahead_body<RP>(g, (int)blockIdx.x);
         return;
     }
     const int bx = (int)blockIdx.x - g.count;
@@ -2813,11 +2919,7 @@ psgd_pqt_gs_batch_kernel(PsgdBatch<PqtItem> b, GsAhead g)
 {
     static_assert(kGsRegThreads == 256, "one block size for both kinds of workgroup");
     if ((int)blockIdx.x < g.count) {
-        __shared__ float red[2][4][RP];
-        if (g.rows[blockIdx.x] <= kGsRegThreads)
-            gs_reg_body<RP, 1>(g.dst[blockIdx.x], g.rows[blockIdx.x], red, g.r, g.eps, g.src[blockIdx.x]);
-        else
-            gs_reg_body<RP, kGsAheadRowSlots>(g.dst[blockIdx.x], g.rows[blockIdx.x], red, g.r, g.eps, g.src[blockIdx.x]);
+        gs_ahead_body<RP>(g, (int)blockIdx.x);
         return;
     }
     const int bx = (int)blockIdx.x - g.count;
@@ -3135,10 +3237,20 @@ int conef_psgd_round_ahead_f32(const ConefPsgdItem* items, int32_t count, int32_
     // P = X Q, P orthogonalised, Q = X^T P: with the orthogonalisation deferred where the batch
     // allows (round_products_deferred; CONEF_ROUND_DEFER=0 keeps the reference's order of steps,
     // for comparisons), else as three steps
-    static const bool defer_on = [] {
-        const char* e = getenv("CONEF_ROUND_DEFER");
-        return !(e && e[0] == '0');
-    }();
+    const char* defer_env = getenv("CONEF_ROUND_DEFER");      // read on every call: a test switches it
+    const bool defer_on = !(defer_env && defer_env[0] == '0');
+    GsAhead ahead;
+    ahead.count = 0;
+    for (int k = 0; k < kPsgdBatchMax; ++k) {
+        ahead.parts[k] = nullptr;
+        ahead.nparts[k] = 0;
+    }
+    // the next round's Q factors are wanted in q_next, by workgroups of this round's last launch
+    bool want_next = (flags & CONEF_ROUND_MAKE_NEXT) && pqt_mode <= 2 && count <= kPsgdBatchMax && rank_bound(items[0].r) <= 8;
+    for (int k = 0; k < count && want_next; ++k)
+        want_next = q_next[k] && items[k].r == items[0].r && aligned16(q_next[k]) && aligned16(items[k].q) &&
+                    items[k].m <= 0x7fffffffLL;
+    bool q_shares_made = false;
     auto products = [&](const ConefPsgdItem* its) -> int {      // its: the items with the Q the first product reads
         if (mq_mode < 0 || mq_mode > 2) return CONEF_ERR_INVALID;
         for (int k = 0; k < count; ++k) {
@@ -3149,9 +3261,11 @@ int conef_psgd_round_ahead_f32(const ConefPsgdItem* items, int32_t count, int32_
         }
         if (defer_on) {
             hipStream_t hs = (hipStream_t)stream;
-            const int rd = mq_mode == 0   ? round_products_deferred<0>(items, its, count, 0.f, eps, a, b, workspace, workspace_bytes, hs)
-                           : mq_mode == 1 ? round_products_deferred<1>(items, its, count, 0.f, eps, a, b, workspace, workspace_bytes, hs)
-                                          : round_products_deferred<2>(items, its, count, alpha, eps, a, b, workspace, workspace_bytes, hs);
+            GsAhead* qs = want_next ? &ahead : nullptr;
+            const int rd = mq_mode == 0   ? round_products_deferred<0>(items, its, count, 0.f, eps, a, b, workspace, workspace_bytes, hs, qs)
+                           : mq_mode == 1 ? round_products_deferred<1>(items, its, count, 0.f, eps, a, b, workspace, workspace_bytes, hs, qs)
+                                          : round_products_deferred<2>(items, its, count, alpha, eps, a, b, workspace, workspace_bytes, hs, qs);
+            if (rd == CONEF_OK) q_shares_made = want_next;
             if (rd != kMqsNoFit) return rd;
         }
         int rp = conef_psgd_mq_batch_f32(its, count, mq_mode, alpha, a, b, workspace, workspace_bytes, stream);
@@ -3179,21 +3293,20 @@ int conef_psgd_round_ahead_f32(const ConefPsgdItem* items, int32_t count, int32_
         rc = products(items);
     }
     if (rc != CONEF_OK) return rc;
-    // The new Q factors orthogonalised into q_next by workgroups of the last launch: only where that
-    // launch covers the whole bucket (one rank, at most 8) and every Q factor is short.
-    GsAhead ahead;
-    ahead.count = 0;
-    if ((flags & CONEF_ROUND_MAKE_NEXT) && pqt_mode <= 2 && count <= kPsgdBatchMax && rank_bound(items[0].r) <= 8) {
+    // The new Q factors orthogonalised into q_next by workgroups of the last launch, where that
+    // launch covers the whole bucket (one rank, at most 8): from the shares of Q^T Q when the
+    // products above left them, else by the column steps themselves, which takes a short Q factor.
+    if (want_next) {
         bool ok = true;
-        for (int k = 0; k < count && ok; ++k)
-            ok = q_next[k] && items[k].r == items[0].r && aligned16(q_next[k]) &&
-                 gs_reg_class(items[k].q, items[k].m, items[k].r) >= 0 &&
+        for (int k = 0; k < count && ok && !q_shares_made; ++k)
+            ok = gs_reg_class(items[k].q, items[k].m, items[k].r) >= 0 &&
                  items[k].m <= (int64_t)kGsAheadRowSlots * kGsRegThreads;
         if (ok) {
             for (int k = 0; k < count; ++k) {
                 ahead.src[k] = items[k].q;
                 ahead.dst[k] = q_next[k];
                 ahead.rows[k] = (int)items[k].m;
+                if (!q_shares_made) ahead.parts[k] = nullptr;
             }
             ahead.count = count;
             ahead.r = items[0].r;
