@@ -584,6 +584,7 @@ psgd_defer_fix_batch_kernel(PsgdBatch<DeferFixItem> b)
     const float* src = is_p ? it.p : it.qsrc;
     const int slabs = is_p ? 1 : it.slabs;
     const int64_t stride = it.m * RP;
+    if (threadIdx.x < RP * RP + RP) t_l[threadIdx.x] = it.tmat[threadIdx.x];      // requested first: it travels with the rows
     float x[RP];
 #pragma unroll
     for (int c = 0; c < RP; ++c) x[c] = 0.f;
@@ -603,7 +604,6 @@ psgd_defer_fix_batch_kernel(PsgdBatch<DeferFixItem> b)
 #pragma unroll
         for (int c = 0; c < RP; ++c) x[c] += v[c];
     }
-    if (threadIdx.x < RP * RP + RP) t_l[threadIdx.x] = it.tmat[threadIdx.x];
     __syncthreads();
     gram_apply_row<RP>(x, t_l);
     if (row < rows) store_row<RP>((is_p ? it.p : it.q) + row * RP, x);
@@ -2401,11 +2401,13 @@ inline int64_t mfma_batch_layout(const ConefPsgdItem* items, int count, std::vec
             const int r = items[k].r;
             MfmaMqShape q = mfma_mq_shape(n, m);
             int64_t need = q.splits > 1 ? (int64_t)q.splits * n * r : 0;
-            for (int v = 4; v >= 1; v >>= 1) {
-                MfmaMtpShape t = mfma_mtp_shape(n, m, r, v);
-                int64_t b = t.slabs > 1 ? (int64_t)t.slabs * m * r : 0;
-                if (b > need) need = b;
-            }
+            // The slabs of Q = X^T P depend on how many workgroups the matrix is asked to bring, which
+            // depends on what else is in the launch (a wider lane with more slabs can win there): room
+            // for the most the shape function ever takes.
+            int64_t slabs_most = n / (4 * (int64_t)r);
+            if (slabs_most < 1) slabs_most = 1;
+            if (slabs_most > (n + 7) / 8) slabs_most = (n + 7) / 8;
+            if (slabs_most > 1 && slabs_most * m * r > need) need = slabs_most * m * r;
             at = off;
             off += (need + 63) / 64 * 64;
         }

@@ -312,7 +312,12 @@ def test_round_defers_the_orthogonalisation_of_p(monkeypatch, oracle, mq_mode, e
     buckets = [[(4096, 1024, 8), (1024, 4096, 8), (1024, 1024, 8), (2051, 1024, 8)],
                [(640, 5760, 4), (2048, 768, 4), (5760, 640, 4)],
                [(4096, 512, 2), (3000, 2048, 2)],
-               [(8192, 1024, 1)]]
+               [(8192, 1024, 1)],
+               # ranks on the matrix cores keep the reference's order of steps: the round is the separate
+               # entry points (two matrices whose second products take different lane widths and slab
+               # counts in one bucket: their partial regions must not overlap)
+               [(4096, 1024, 32), (1024, 4096, 32), (1024, 1024, 32)],
+               [(2048, 768, 16), (1024, 1024, 16)]]
     stream = torch.cuda.current_stream().cuda_stream
     for specs in buckets:
         count = len(specs)
@@ -375,10 +380,12 @@ def test_round_defers_the_orthogonalisation_of_p(monkeypatch, oracle, mq_mode, e
             Qn = oracle.mtp(X, P)
             assert_close(Pa, P, rel=rel, what="deferred P against the oracle %s" % (spec,))
             assert_close(Qa, Qn, rel=rel, what="deferred Q against the oracle %s" % (spec,))
+            assert_close(Qb, Qn, rel=rel, what="step-by-step Q against the oracle %s" % (spec,))
             assert_close(Ma, oracle.pqt(P, Qn), rel=rel, what="deferred M against the oracle %s" % (spec,))
             pp = to_np(Pa).astype(np.float64)
             np.testing.assert_allclose(pp.T @ pp, np.eye(spec[2]), atol=1e-2 if (k == 0 and spec[2] > 2) else 2e-5)
-        assert not identical, "the round took the step-by-step path on %s" % (specs,)
+        assert identical == (specs[0][2] > 8), "the round took the %s path on %s" % (
+            "step-by-step" if identical else "deferred", specs)
 
 
 def test_products_with_sketch_on_a_plan(oracle):
