@@ -113,11 +113,11 @@ def UnbiasedRandomBlock_hook(state: UnbiasedRandomBlockState, bucket) -> torch.f
     if tensors:
         rc = lib.conef_randblock_step_batch_f32(items, len(tensors), 0, 0.0, 0.0, 0, 0, stream)
         _lib.check(rc, "conef_randblock_step_batch_f32")
-    spans = list(zip(tensors, starts, blocks, offsets))
 
     if world_size == 1:
         state.maybe_increase_iter(bucket)
         return _bucket.completed_future(input_tensor)
+    spans = list(zip(tensors, starts, blocks, offsets))
 
     # More than one rank (not exercised on the single-GPU boxes this was developed on).
     flat_small = (torch.cat([t.view(-1) for t in uncompressed]) if uncompressed

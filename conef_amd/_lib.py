@@ -132,8 +132,13 @@ def check(code, what):
         raise ConefLibraryError("%s: HIP error %d" % (what, code))
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(tensor):
     """hipStream_t of torch's current stream on the tensor's device, as an integer."""
+    if _raw_stream is not None:       # the handle without building a Stream object: a hook calls this per bucket
+        return _raw_stream(tensor.get_device())
     return torch.cuda.current_stream(tensor.device).cuda_stream
 
 
