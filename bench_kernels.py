@@ -105,10 +105,12 @@ def main():
                                                                     stream), "query"))
         if SketchPlan.applicable(n, d, w):
             plan = SketchPlan(n, d, w, A, B, dev)
-            timeit("cs_query_planned_f32 (buckets and signs from the plan's table) %s [%d,%d] W=%d" % (tag, n, d, w),
+            staging = None if plan.in_place else plan.workspace.data_ptr()
+            timeit("cs_query_planned_f32 (%s) %s [%d,%d] W=%d" % (
+                       "buckets and signs from the plan's table" if plan.in_place else "table, sketch interleaved", tag, n, d, w),
                    8 * n * d + 4 * n * w + 4 * d, make,
-                   lambda s, n=n, d=d, w=w, plan=plan: ck(lib.conef_cs_query_planned_f32(
-                       s[0].data_ptr(), s[1].data_ptr(), plan.host_ptr, plan.device.data_ptr(), n, d, w, 0.1, A, B,
+                   lambda s, n=n, d=d, w=w, plan=plan, staging=staging: ck(lib.conef_cs_query_planned_f32(
+                       s[0].data_ptr(), s[1].data_ptr(), plan.host_ptr, plan.device.data_ptr(), staging, n, d, w, 0.1, A, B,
                        stream), "query planned"))
             timeit("cs_update_planned_f32 (%s) %s [%d,%d] W=%d" % ("row lists" if plan.in_place else "binned", tag, n, d, w),
                    4 * n * d + 8 * n * w, make,

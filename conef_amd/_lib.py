@@ -27,7 +27,7 @@ SIGNATURES = {
     "conef_hash_table_host_i32": [_P, _P, _I64, _I32, _I32, _I32, _I32, _I32],
     "conef_cs_query_f32": [_P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],
     "conef_cs_query_f16": [_P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],
-    "conef_cs_query_planned_f32": [_P, _P, _P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],
+    "conef_cs_query_planned_f32": [_P, _P, _P, _P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],
     "conef_cs_query_planned_f16": [_P, _P, _P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],
     "conef_cs_update_inplace_ok": [_I64, _I64, _I32],
     "conef_cs_update_f32": [_P, _P, _P, _I64, _I64, _I32, _F32, _I32, _I32, _P],

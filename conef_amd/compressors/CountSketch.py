@@ -162,9 +162,11 @@ class DenseCS:
         plan = self.plan()
         if plan is not None:
             # buckets and signs from the plan's table instead of two hashes and modulos per column
+            # (and, for a few long rows, the sketch interleaved into the plan's staging buffer first)
+            staging = None if plan.in_place else plan.workspace.data_ptr()
             rc = self._lib.conef_cs_query_planned_f32(grad_plus_error.data_ptr(), self.cs.data_ptr(), plan.host_ptr,
-                                                      plan.device.data_ptr(), self.N, self.D, self.range, float(alpha),
-                                                      self.a, self.b, _lib.stream_ptr(grad_plus_error))
+                                                      plan.device.data_ptr(), staging, self.N, self.D, self.range,
+                                                      float(alpha), self.a, self.b, _lib.stream_ptr(grad_plus_error))
             _lib.check(rc, "conef_cs_query_planned_f32")
             return
         rc = self._lib.conef_cs_query_f32(grad_plus_error.data_ptr(), self.cs.data_ptr(), self.N, self.D,

@@ -13,6 +13,8 @@ inline bool plan_has_default_sign_seeds(const ConefPlanHeader* hp, int32_t a, in
 }  // namespace
 
 // conef_sketch.hip
+int conef_launch_query_rows8_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha,
+                                 const uint32_t* pktab, float* scratch, hipStream_t stream);
 int conef_launch_query_table_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
                                  int32_t b, const uint32_t* pktab, hipStream_t stream);
 int conef_launch_query_table_f16(float* x, const void* cs_half, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
@@ -95,12 +97,18 @@ int conef_cs_update_planned_f16(const float* vec, const void* cs_in_half, void* 
 
 // DenseCS.query with the buckets and signs of a plan's table instead of hashing (either kind of
 // plan, built for (n, d, w, a, b) with the default sign seeds): same values, bit for bit.
-int conef_cs_query_planned_f32(float* x, const float* cs, const void* plan_host, const void* plan_dev, int64_t n,
-                               int64_t d, int32_t w, float alpha, int32_t a, int32_t b, void* stream)
+int conef_cs_query_planned_f32(float* x, const float* cs, const void* plan_host, const void* plan_dev, void* workspace,
+                               int64_t n, int64_t d, int32_t w, float alpha, int32_t a, int32_t b, void* stream)
 {
     const ConefPlanHeader* hp = (const ConefPlanHeader*)plan_host;
     if (!conef_plan_matches(hp, n, d, w, a, b) || !plan_dev || !plan_has_default_sign_seeds(hp, a, b)) return CONEF_ERR_INVALID;
     const uint32_t* pk = (const uint32_t*)((const char*)plan_dev + hp->off_pk);
+    // A few long rows (the binned plans' shapes) with the plan's workspace at hand: the sketch is
+    // interleaved into it first and a column's cells of all rows come with one gather.
+    if (workspace && hp->kind == kConefPlanBinned && n <= 8 && x && cs && hp->workspace_bytes >= 32 * (int64_t)w) {
+        const int rc = conef_launch_query_rows8_f32(x, cs, n, d, w, alpha, pk, (float*)workspace, (hipStream_t)stream);
+        if (rc != CONEF_ERR_INVALID) return rc;
+    }
     return conef_launch_query_table_f32(x, cs, n, d, w, alpha, a, b, pk, (hipStream_t)stream);
 }
 

@@ -386,6 +386,82 @@ int launch_update(const float* vec, const CsT* cs_in, CsT* cs_out, int64_t n, in
 
 }  // namespace
 
+// ---- the query for a few long rows (at most 8 rows, a sketch row far beyond LDS) ----
+// Every row of the tensor uses the same bucket for a column, so with the sketch transposed to
+// [w][8] (32 bytes a bucket, rows past n zero) a column's cells of ALL rows are one 32-byte gather
+// instead of one 4-byte gather per row, each of which drags a cache line from L2: five times fewer
+// lines for the flat 25 MB bucket, whose query was bound by exactly that.
+namespace {
+
+__global__ void __launch_bounds__(256)
+cs_interleave8_kernel(const float* __restrict__ cs, float* __restrict__ inter, int n, int w)
+{
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= w) return;
+    float v[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) v[r] = r < n ? cs[(int64_t)r * w + j] : 0.f;
+    float4* dst = reinterpret_cast<float4*>(inter + (int64_t)j * 8);
+    dst[0] = make_float4(v[0], v[1], v[2], v[3]);
+    dst[1] = make_float4(v[4], v[5], v[6], v[7]);
+}
+
+// a thread owns a column quad of all rows; d % 4 == 0, x and the table 16-byte aligned
+template <int NR>
+__global__ void __launch_bounds__(256)
+cs_query_rows8_kernel(float* __restrict__ x, const float* __restrict__ inter, int64_t d, float alpha,
+                      const uint32_t* __restrict__ pktab)
+{
+    const int64_t c0 = (blockIdx.x * (int64_t)blockDim.x + threadIdx.x) * 4;
+    if (c0 >= d) return;
+    const uint4 t = *reinterpret_cast<const uint4*>(pktab + c0);
+    const uint32_t pk[4] = {t.x, t.y, t.z, t.w};
+    float4 v[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) v[r] = *reinterpret_cast<const float4*>(x + (int64_t)r * d + c0);
+    float cell[4][8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float4* src = reinterpret_cast<const float4*>(inter + (int64_t)(pk[k] & 0x7fffffffu) * 8);
+        const float4 lo = src[0];
+        cell[k][0] = lo.x; cell[k][1] = lo.y; cell[k][2] = lo.z; cell[k][3] = lo.w;
+        if (NR > 4) {
+            const float4 hi = src[1];
+            cell[k][4] = hi.x; cell[k][5] = hi.y; cell[k][6] = hi.z; cell[k][7] = hi.w;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        float4 o;
+        o.x = __fadd_rn(v[r].x, conef_query_term(cell[0][r], pk[0], alpha));
+        o.y = __fadd_rn(v[r].y, conef_query_term(cell[1][r], pk[1], alpha));
+        o.z = __fadd_rn(v[r].z, conef_query_term(cell[2][r], pk[2], alpha));
+        o.w = __fadd_rn(v[r].w, conef_query_term(cell[3][r], pk[3], alpha));
+        *reinterpret_cast<float4*>(x + (int64_t)r * d + c0) = o;
+    }
+}
+
+}  // namespace
+
+// scratch: at least 32 w bytes, 16-byte aligned.  Returns CONEF_ERR_INVALID for shapes this form
+// does not take (more than 8 rows, d % 4 != 0, unaligned x or table); the caller then takes the
+// general query.
+int conef_launch_query_rows8_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha,
+                                 const uint32_t* pktab, float* scratch, hipStream_t stream)
+{
+    if (n < 1 || n > 8 || d < 4 || d % 4 != 0 || !aligned16(x) || !aligned16(pktab) || !aligned16(scratch)) return CONEF_ERR_INVALID;
+    hipLaunchKernelGGL(cs_interleave8_kernel, dim3((unsigned)((w + 255) / 256)), dim3(256), 0, stream, cs, scratch, (int)n, (int)w);
+    const dim3 grid((unsigned)((d / 4 + 255) / 256));
+    switch ((int)n) {
+#define CONEF_ROWS8(NR) \
+    case NR: hipLaunchKernelGGL(cs_query_rows8_kernel<NR>, grid, dim3(256), 0, stream, x, scratch, d, alpha, pktab); break
+        CONEF_ROWS8(1); CONEF_ROWS8(2); CONEF_ROWS8(3); CONEF_ROWS8(4);
+        CONEF_ROWS8(5); CONEF_ROWS8(6); CONEF_ROWS8(7); CONEF_ROWS8(8);
+#undef CONEF_ROWS8
+    }
+    return (int)hipGetLastError();
+}
+
 // The query with buckets and signs read from a table (uint32[d]: bucket | sign bit << 31, the `pk`
 // table of a plan); called by conef_cs_query_planned_f32 / _f16 in conef_plan.hip.
 int conef_launch_query_table_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,

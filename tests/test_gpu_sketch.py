@@ -62,11 +62,13 @@ def test_query_bit_exact(oracle, n, d, ss):
     np.testing.assert_array_equal(to_np(xd), x)
 
 
-@pytest.mark.parametrize("n,d,ss", [(5, 130_000, 0.1), (40, 650, 0.1), (640, 5760, 0.2), (3, 17, 0.3), (7, 4099, 0.25)])
+@pytest.mark.parametrize("n,d,ss", [(5, 130_000, 0.1), (40, 650, 0.1), (640, 5760, 0.2), (3, 17, 0.3), (7, 4099, 0.25),
+                                    (8, 40_000, 0.1), (3, 100_000, 0.2), (1, 65_536, 0.1), (6, 30_002, 0.3)])
 def test_query_hashed_and_table_entry_points_agree(oracle, n, d, ss):
     """conef_cs_query_f32 hashes every column, conef_cs_query_planned_f32 reads bucket and sign from the
-    plan's table (binned and row-list plans): both must give the oracle's bits; a plan built for other
-    seeds is refused."""
+    plan's table (binned and row-list plans) and, given a binned plan's workspace, gathers the cells of
+    all (at most 8) rows of a column at once from an interleaved copy of the sketch: all must give the
+    oracle's bits; a plan built for other seeds is refused."""
     from conef_amd import _lib
     from conef_amd._plan import SketchPlan
     lib = _lib.load()
@@ -81,15 +83,20 @@ def test_query_hashed_and_table_entry_points_agree(oracle, n, d, ss):
     hashed, table = dev(x), dev(x)
     assert lib.conef_cs_query_f32(hashed.data_ptr(), csd.data_ptr(), n, d, w, 0.1, a, b, 0) == 0
     plan = SketchPlan.shared(n, d, w, a, b, torch.device("cuda", 0))
-    assert lib.conef_cs_query_planned_f32(table.data_ptr(), csd.data_ptr(), plan.host_ptr, plan.device.data_ptr(), n, d,
-                                          w, 0.1, a, b, 0) == 0
+    assert lib.conef_cs_query_planned_f32(table.data_ptr(), csd.data_ptr(), plan.host_ptr, plan.device.data_ptr(), None,
+                                          n, d, w, 0.1, a, b, 0) == 0
     np.testing.assert_array_equal(to_np(hashed), want)
     np.testing.assert_array_equal(to_np(table), want)
+    if not plan.in_place:                      # a binned plan has a workspace: the interleaved form where the shape allows
+        inter = dev(x)
+        assert lib.conef_cs_query_planned_f32(inter.data_ptr(), csd.data_ptr(), plan.host_ptr, plan.device.data_ptr(),
+                                              plan.workspace.data_ptr(), n, d, w, 0.1, a, b, 0) == 0
+        np.testing.assert_array_equal(to_np(inter), want)
     other = SketchPlan.shared(n, d, w, a, b, torch.device("cuda", 0), sign_seeds=(a + 4, b + 5))
-    assert lib.conef_cs_query_planned_f32(table.data_ptr(), csd.data_ptr(), other.host_ptr, other.device.data_ptr(), n,
-                                          d, w, 0.1, a, b, 0) == -1
-    assert lib.conef_cs_query_planned_f32(table.data_ptr(), csd.data_ptr(), plan.host_ptr, plan.device.data_ptr(), n, d,
-                                          w + 1, 0.1, a, b, 0) == -1
+    assert lib.conef_cs_query_planned_f32(table.data_ptr(), csd.data_ptr(), other.host_ptr, other.device.data_ptr(), None,
+                                          n, d, w, 0.1, a, b, 0) == -1
+    assert lib.conef_cs_query_planned_f32(table.data_ptr(), csd.data_ptr(), plan.host_ptr, plan.device.data_ptr(), None,
+                                          n, d, w + 1, 0.1, a, b, 0) == -1
 
 
 @pytest.mark.parametrize("n,d,ss", SHAPES)
