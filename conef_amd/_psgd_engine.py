@@ -106,7 +106,7 @@ class _RoundPlan:
     and layout, so that a step costs a handful of foreign calls however many tensors it has."""
     __slots__ = ("key", "shapes", "work", "passthrough", "before", "after", "total_ps", "total_qs", "arena_key", "ps",
                  "qs", "items", "count", "sketches", "fused_sketch", "batched_update", "residual_offsets",
-                 "topk_table", "q_next", "q_next_ptrs", "q_next_ready", "made")
+                 "topk_table", "q_next", "q_next_ptrs", "q_next_ready", "made", "q_next_views", "items_next", "q_next_event")
 
 
 def _build_round(state, grads, shapes, key, error_mode):
@@ -319,7 +319,17 @@ def _run_round(state, bucket, error_mode):
         mode3 = 3 if error_mode == "conef" and plan.batched_update else 1
     else:
         mode3 = 0
-    if (mode3 in (0, 1, 2) and state.matrix_approximation_rank <= 8 and state.warm_start and count and count <= 24
+    if (state.matrix_approximation_rank > 8 and state.warm_start and count
+            and int(getattr(state, "hook_streams", 1) or 1) <= 1 and os.environ.get("CONEF_ROUND_AHEAD", "1") != "0"):
+        # Ranks on the matrix cores: the round as its separate launches, with the Gram-Schmidt of the new
+        # Q factors (which the reference runs at the start of the bucket's next round,
+        # powerSGD_hook.py:496-497: 27-35 us of dependent steps on a few workgroups) on a side stream,
+        # out of place, while this stream goes on with M = P Q^T and the sketch update.  The next round
+        # of this bucket waits for it.  CONEF_ROUND_AHEAD=0 keeps everything on one stream; so does
+        # hook_streams > 1, where buckets already run side by side (measured: the two together are slower).
+        _round_with_q_on_the_side(state, plan, lib, items, count, mode1, mode3, alpha, eps, ws_ptr, ws_len, stream,
+                                  device, q_mem, qs)
+    elif (mode3 in (0, 1, 2) and state.matrix_approximation_rank <= 8 and state.warm_start and count and count <= 24
             and os.environ.get("CONEF_ROUND_AHEAD", "1") != "0"):
         # The bucket's next round starts by orthogonalising the Q factors this round leaves
         # (powerSGD_hook.py:496-497): a few workgroups and an idle machine.  Workgroups of this
@@ -359,6 +369,53 @@ def _run_round(state, bucket, error_mode):
 
     state.maybe_increase_iter(bucket)
     return _bucket.completed_future(input_tensor)
+
+
+def _round_with_q_on_the_side(state, plan, lib, items, count, mode1, mode3, alpha, eps, ws_ptr, ws_len, stream, device,
+                              q_mem, qs):
+    import ctypes
+    main = torch.cuda.current_stream(device)
+    if plan.q_next is None:
+        plan.q_next = torch.empty_like(q_mem)
+        plan.q_next_views, off = [], 0
+        for q in qs:
+            plan.q_next_views.append(plan.q_next[off: off + q.numel()].view(q.shape))
+            off += q.numel()
+        plan.items_next = (type(items[0]) * count)()      # the same table with the first product reading the second buffer
+        plan.q_next_event = torch.cuda.Event()
+        plan.q_next_ready = False
+    if plan.q_next_ready:
+        for k in range(count):                              # pointers of the table can move between steps (err, cs)
+            ctypes.memmove(ctypes.byref(plan.items_next[k]), ctypes.byref(items[k]), ctypes.sizeof(items[k]))
+            plan.items_next[k].q = plan.q_next_views[k].data_ptr()
+        main.wait_event(plan.q_next_event)
+        first = plan.items_next
+    else:
+        orthogonalize_all(qs, eps, ws_ptr, ws_len, stream)
+        first = items
+    rc = lib.conef_psgd_mq_batch_f32(first, count, mode1, float(alpha), HASH_A, HASH_B, ws_ptr, ws_len, stream)
+    _lib.check(rc, "conef_psgd_mq_batch_f32")
+    orthogonalize_all(plan.ps, eps, ws_ptr, ws_len, stream)
+    rc = lib.conef_psgd_mtp_batch_f32(items, count, ws_ptr, ws_len, stream)
+    _lib.check(rc, "conef_psgd_mtp_batch_f32")
+    # the new Q is final: orthogonalise a copy of it on the side
+    q_final = torch.cuda.Event()
+    q_final.record(main)
+    side = _pools.side_stream(device, 0, 1)
+    side.wait_event(q_final)
+    with torch.cuda.stream(side):
+        plan.q_next.copy_(q_mem, non_blocking=True)
+        side_ws = _workspace(device, side.cuda_stream, max(ws_len, 256))
+        orthogonalize_all(plan.q_next_views, eps, side_ws.data_ptr(), side_ws.numel(), side.cuda_stream)
+        plan.q_next_event.record(side)
+    plan.q_next_ready = True
+    beta = float(state.beta) if mode3 in (2, 3) else 0.0
+    rc = lib.conef_psgd_pqt_batch_f32(items, count, 1 if mode3 == 3 else mode3, beta if mode3 == 2 else 0.0, HASH_A, HASH_B,
+                                      stream)
+    _lib.check(rc, "conef_psgd_pqt_batch_f32")
+    if mode3 == 3:
+        rc = lib.conef_psgd_sketch_update_batch_f32(items, count, beta, HASH_A, HASH_B, stream)
+        _lib.check(rc, "conef_psgd_sketch_update_batch_f32")
 
 
 def run_batched_round(state, bucket):

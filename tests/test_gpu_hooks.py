@@ -803,6 +803,58 @@ def test_q_factors_orthogonalised_by_the_last_launch(monkeypatch, oracle, rank, 
             same(x, z)
 
 
+@pytest.mark.parametrize("rank,mode", [(32, "conef"), (16, "ef"), (12, "plain")])
+def test_high_rank_rounds_orthogonalise_q_on_a_side_stream(monkeypatch, rank, mode):
+    """Above rank 8 the new Q factors of a bucket are orthogonalised for its next round on a side stream
+    while the round goes on (a copy of Q, the same kernels): bucket, P, Q and error state must equal
+    the one-stream order bit for bit, step after step, over buckets with tall and short factors."""
+    from conef_amd.powerSGD_hook import PowerSGDState, powerSGD_hook
+    buckets = [[(1024, 256), (256,), (256, 1024), (640, 768)], [(4096, 128), (128, 4096)], [(64, 576), (40, 64), (33, 40)]]
+
+    def make():
+        st = PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, use_error_feedback=mode != "plain",
+                           use_error_compression=mode == "conef", sketch_size=0.1, beta=0.9)
+        st.iter = 2
+        return st
+
+    def steps(st, count):
+        outs = []
+        for step in range(count):
+            gen = torch.Generator().manual_seed(500 + step)
+            flats = [(torch.randn(numel_of(b), generator=gen) * 1e-3).cuda() for b in buckets]
+            futs = [powerSGD_hook(st, FakeGradBucket(f, b, index=i, is_last=i == len(buckets) - 1))
+                    for i, (f, b) in enumerate(zip(flats, buckets))]
+            outs.append([to_np(f.wait()) for f in futs])
+        torch.cuda.synchronize()
+        return outs
+
+    def snapshot(st):
+        keep = []
+        for i in range(len(buckets)):
+            keep += [to_np(st.p_memory_dict[i]), to_np(st.q_memory_dict[i])]
+            err = st.error_dict.get(i)
+            if isinstance(err, dict):
+                keep += [to_np(e.cs) for e in err.values()]
+            elif err is not None:
+                keep.append(to_np(err))
+        return keep
+
+    monkeypatch.setenv("CONEF_ROUND_AHEAD", "0")
+    plain = make()
+    outs_plain = steps(plain, 5)
+    monkeypatch.setenv("CONEF_ROUND_AHEAD", "1")
+    side = make()
+    outs_side = steps(side, 5)
+    compressing = [i for i in range(len(buckets)) if side.round_cache[i].count]       # a bucket may hold nothing worth compressing
+    assert compressing and all(side.round_cache[i].q_next_ready for i in compressing)
+    assert not any(plain.round_cache[i].q_next_ready for i in range(len(buckets)))
+    for a, b in zip(outs_plain, outs_side):
+        for x, y in zip(a, b):
+            np.testing.assert_array_equal(x, y)
+    for x, y in zip(snapshot(plain), snapshot(side)):
+        np.testing.assert_array_equal(x, y)
+
+
 def test_powersgd_state_errors_and_warmup():
     from conef_amd.powerSGD_hook import PowerSGDState, _should_compress, powerSGD_hook
     with pytest.raises(ValueError, match="Expect `start_powerSGD_iter` > 1"):
