@@ -61,7 +61,15 @@ class Checkpointable:
     __slots__ = ()
     CHECKPOINT_FIELDS = ()
 
+    def settle(self):
+        """Work the hooks left on a side stream that touches this state's tensors is ordered before
+        the current stream's next operation (a no-op for the states that leave none)."""
+        if hasattr(self, "round_cache"):
+            from ._psgd_engine import settle
+            settle(self)
+
     def state_dict(self):
+        self.settle()
         return {"class": type(self).__name__, "fields": {f: pack(getattr(self, f)) for f in self.CHECKPOINT_FIELDS}}
 
     def load_state_dict(self, state, device=None):

@@ -106,7 +106,8 @@ class _RoundPlan:
     and layout, so that a step costs a handful of foreign calls however many tensors it has."""
     __slots__ = ("key", "shapes", "work", "passthrough", "before", "after", "total_ps", "total_qs", "arena_key", "ps",
                  "qs", "items", "count", "sketches", "fused_sketch", "batched_update", "residual_offsets",
-                 "topk_table", "q_next", "q_next_ptrs", "q_next_ready", "made", "q_next_views", "items_next", "q_next_event")
+                 "topk_table", "q_next", "q_next_ptrs", "q_next_ready", "made", "q_next_views", "items_next", "q_next_event",
+                 "topk_event")
 
 
 def _build_round(state, grads, shapes, key, error_mode):
@@ -138,6 +139,7 @@ def _build_round(state, grads, shapes, key, error_mode):
     plan.fused_sketch = False
     plan.batched_update = False
     plan.topk_table = None
+    plan.topk_event = None          # the side stream's top-k of this bucket's errors, to be waited for by its next round
     # Second buffer for the Q factors, orthogonalised at the end of a round for the bucket's next
     # round (conef_psgd_round_ahead_f32).  Derived data: q_memory_dict keeps what the reference
     # keeps, and the flag falls with the plan whenever the state is replaced.
@@ -154,6 +156,16 @@ def _build_round(state, grads, shapes, key, error_mode):
 
 
 _side_stream = _pools.side_stream
+
+
+def settle(state):
+    """Orders torch's current stream after whatever the rounds of ``state`` left running on a side
+    stream that touches the state's own tensors (the top-k of the error tensors): to be called
+    before those tensors are read or written from outside the hooks."""
+    for plan in getattr(state, "round_cache", {}).values():
+        event = getattr(plan, "topk_event", None)
+        if event is not None:
+            torch.cuda.current_stream().wait_event(event)
 
 
 def run_round(state, bucket, error_mode):
@@ -276,6 +288,10 @@ def _run_round(state, bucket, error_mode):
             if cnt not in errs:
                 errs[cnt] = DenseCS(m, n, state.sketch_size, device=device)
 
+    if plan.topk_event is not None:
+        # the errors this round adds are still being sparsified on the side stream
+        torch.cuda.current_stream(device).wait_event(plan.topk_event)
+        plan.topk_event = None
     eps = float(state.orthogonalization_epsilon)
     ws = _workspace(device, stream, max(lib.conef_psgd_batch_workspace_bytes(items, count), 256))
     ws_ptr, ws_len = ws.data_ptr(), ws.numel()
@@ -357,7 +373,29 @@ def _run_round(state, bucket, error_mode):
                                       eps, HASH_A, HASH_B, ws_ptr, ws_len, stream)
         _lib.check(rc, "conef_psgd_round_f32")
     if error_mode == "topk":
-        plan.topk_table = topk_sparsify_all([errs[cnt] for cnt in range(count)], state.topk_ratio, plan.topk_table)
+        if (count and int(getattr(state, "hook_streams", 1) or 1) <= 1
+                and os.environ.get("CONEF_ROUND_AHEAD", "1") != "0"):
+            # The sparsification only touches the error tensors, which nobody reads before this bucket's
+            # next round: it runs on a side stream while this stream goes on with the next bucket (five
+            # streaming passes next to launches that are mostly latency).  Same kernels, same values.
+            main = torch.cuda.current_stream(device)
+            done = torch.cuda.Event()
+            done.record(main)
+            side = _pools.side_stream(device, 0, 1)
+            side.wait_event(done)
+            with torch.cuda.stream(side):
+                fresh = plan.topk_table is None
+                plan.topk_table = topk_sparsify_all([errs[cnt] for cnt in range(count)], state.topk_ratio, plan.topk_table)
+                if fresh:
+                    # memory the side stream works on must not go back to the allocator under it
+                    for cnt in range(count):
+                        errs[cnt].record_stream(side)
+                    plan.topk_table[4].record_stream(side)
+                if plan.topk_event is None:
+                    plan.topk_event = torch.cuda.Event()
+                plan.topk_event.record(side)
+        else:
+            plan.topk_table = topk_sparsify_all([errs[cnt] for cnt in range(count)], state.topk_ratio, plan.topk_table)
     elif residual is not None and mode3 != 3:
         for cnt, (matrix, n, m, rank) in enumerate(work):
             res = residual[plan.residual_offsets[cnt]: plan.residual_offsets[cnt + 1]]
@@ -375,7 +413,8 @@ def _round_with_q_on_the_side(state, plan, lib, items, count, mode1, mode3, alph
                               q_mem, qs):
     import ctypes
     main = torch.cuda.current_stream(device)
-    if plan.q_next is None:
+    fresh_q_next = plan.q_next is None
+    if fresh_q_next:
         plan.q_next = torch.empty_like(q_mem)
         plan.q_next_views, off = [], 0
         for q in qs:
@@ -403,6 +442,8 @@ def _round_with_q_on_the_side(state, plan, lib, items, count, mode1, mode3, alph
     q_final.record(main)
     side = _pools.side_stream(device, 0, 1)
     side.wait_event(q_final)
+    if fresh_q_next:
+        plan.q_next.record_stream(side)       # memory the side stream works on must not go back to the allocator under it
     with torch.cuda.stream(side):
         plan.q_next.copy_(q_mem, non_blocking=True)
         side_ws = _workspace(device, side.cuda_stream, max(ws_len, 256))

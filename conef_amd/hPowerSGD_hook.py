@@ -107,6 +107,7 @@ class hPowerSGDState(Checkpointable):
     def clean_error(self):
         """Zeroes the kept errors.  (The reference calls ``.clean(0)`` on dense tensors here,
         :267-271, which would raise; zeroing is what that call means.)"""
+        self.settle()
         if self.use_error_feedback:
             for per_bucket in self.error_dict.values():
                 if isinstance(per_bucket, dict):
