@@ -157,16 +157,18 @@ topk_hist_body(const float* __restrict__ x, int64_t numel, TopkState* st, int pa
     const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
     const int64_t stride = (int64_t)gx * blockDim.x;
     if (vec) {
-        // four 16-byte loads in flight per thread
-        for (int64_t q0 = bx * (int64_t)blockDim.x + threadIdx.x; q0 < quads; q0 += 4 * stride) {
-            float4 v[4];
+        // eight 16-byte loads in flight per thread: a thread's share is sixteen quads or so, and every
+        // round of loads is a trip to memory
+        constexpr int U = 8;
+        for (int64_t q0 = bx * (int64_t)blockDim.x + threadIdx.x; q0 < quads; q0 += U * stride) {
+            float4 v[U];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < U; ++u) {
                 const int64_t q = q0 + u * stride;
                 v[u] = reinterpret_cast<const float4*>(x)[q < quads ? q : q0];
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < U; ++u) {
                 if (q0 + u * stride >= quads) break;
                 const uint32_t key[4] = {mag_key(v[u].x), mag_key(v[u].y), mag_key(v[u].z), mag_key(v[u].w)};
 #pragma unroll
@@ -268,16 +270,30 @@ topk_filter_body(float* __restrict__ x, int64_t numel, TopkState* st, int bx, in
     const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
     const int64_t stride = (int64_t)gx * blockDim.x;
     if (vec) {
-        for (int64_t q = bx * (int64_t)blockDim.x + threadIdx.x; q < quads; q += stride) {
-            float4 v = reinterpret_cast<float4*>(x)[q];
-            const uint32_t key[4] = {mag_key(v.x), mag_key(v.y), mag_key(v.z), mag_key(v.w)};
-            bool k0 = key[0] >= thr, k1 = key[1] >= thr, k2 = key[2] >= thr, k3 = key[3] >= thr;
-            if (!(k0 && k1 && k2 && k3))
-                reinterpret_cast<float4*>(x)[q] = make_float4(k0 ? v.x : 0.f, k1 ? v.y : 0.f, k2 ? v.z : 0.f, k3 ? v.w : 0.f);
-            if (listed) {
+        // eight quads requested before the first is used (a load behind a store to the same array is
+        // not moved up by the compiler: one quad a trip otherwise)
+        constexpr int U = 8;
+        for (int64_t q0 = bx * (int64_t)blockDim.x + threadIdx.x; q0 < quads; q0 += U * stride) {
+            float4 vv[U];
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (key[e] == thr) note(4 * q + e);
+            for (int u = 0; u < U; ++u) {
+                const int64_t q = q0 + u * stride;
+                vv[u] = reinterpret_cast<const float4*>(x)[q < quads ? q : q0];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t q = q0 + u * stride;
+                if (q >= quads) break;
+                const float4 v = vv[u];
+                const uint32_t key[4] = {mag_key(v.x), mag_key(v.y), mag_key(v.z), mag_key(v.w)};
+                bool k0 = key[0] >= thr, k1 = key[1] >= thr, k2 = key[2] >= thr, k3 = key[3] >= thr;
+                if (!(k0 && k1 && k2 && k3))
+                    reinterpret_cast<float4*>(x)[q] = make_float4(k0 ? v.x : 0.f, k1 ? v.y : 0.f, k2 ? v.z : 0.f, k3 ? v.w : 0.f);
+                if (listed) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (key[e] == thr) note(4 * q + e);
+                }
             }
         }
     }
