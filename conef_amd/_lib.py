@@ -51,6 +51,7 @@ SIGNATURES = {
     "conef_psgd_workspace_bytes": [_I64, _I64, _I32],
     "conef_psgd_batch_workspace_bytes": [_P, _I32],
     "conef_psgd_mq_batch_f32": [_P, _I32, _I32, _F32, _I32, _I32, _P, _I64, _P],
+    "conef_psgd_products_f32": [_P, _P, _I32, _I32, _F32, _F32, _I32, _I32, _P, _I64, _P],
     "conef_psgd_mtp_batch_f32": [_P, _I32, _P, _I64, _P],
     "conef_psgd_pqt_batch_f32": [_P, _I32, _I32, _F32, _I32, _I32, _P],
     "conef_psgd_sketch_update_batch_f32": [_P, _I32, _F32, _I32, _I32, _P],

@@ -431,12 +431,10 @@ def _round_with_q_on_the_side(state, plan, lib, items, count, mode1, mode3, alph
         first = plan.items_next
     else:
         orthogonalize_all(qs, eps, ws_ptr, ws_len, stream)
-        first = items
-    rc = lib.conef_psgd_mq_batch_f32(first, count, mode1, float(alpha), HASH_A, HASH_B, ws_ptr, ws_len, stream)
-    _lib.check(rc, "conef_psgd_mq_batch_f32")
-    orthogonalize_all(plan.ps, eps, ws_ptr, ws_len, stream)
-    rc = lib.conef_psgd_mtp_batch_f32(items, count, ws_ptr, ws_len, stream)
-    _lib.check(rc, "conef_psgd_mtp_batch_f32")
+        first = None
+    # P = M Q, P orthogonalised, Q = M^T P
+    rc = lib.conef_psgd_products_f32(items, first, count, mode1, float(alpha), eps, HASH_A, HASH_B, ws_ptr, ws_len, stream)
+    _lib.check(rc, "conef_psgd_products_f32")
     # the new Q is final: orthogonalise a copy of it on the side
     q_final = torch.cuda.Event()
     q_final.record(main)

@@ -94,6 +94,87 @@ __device__ __forceinline__ void gsg_entry(int e, int rp, int* pi, int* pj)
     *pj = i + (e - (i * rp - (i * (i - 1)) / 2));
 }
 
+// A workgroup's share of G = A^T A over rows [r0, r1) of the row-major [*, RP] matrix a, on the matrix
+// cores in double: per-wave partial tiles into `tiles` ([waves][NT][256], [i][j] row-major inside a
+// 16 x 16 tile; tiles in the order (0,0), (0,1), (1,1)).  All kGsgThreads threads call this; a
+// barrier must follow before the tiles are read (gsg_tiles_entry).
+template <int RP>
+__device__ __forceinline__ void
+gsg_gram_tiles(const float* __restrict__ a, int r0, int r1, double (*tiles)[(RP >= 16 ? (RP / 16) * (RP / 16 + 1) / 2 : 1)][256])
+{
+    constexpr int NW = kGsgThreads / 64;
+    constexpr int NC = RP >= 16 ? RP / 16 : 1;
+    constexpr int NT = NC * (NC + 1) / 2;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // a wave takes blocks of four rows, lane = (row l / 16,
+    // column l % 16 of each column group); D[i][j] += sum_k A[k][i] A[k][j] over the block's rows.
+    // At rank 8 lanes 8..15 of a row group take the same columns of the NEXT four rows: the two
+    // diagonal 8 x 8 blocks of the product are then two partial sums of G (the off-diagonal blocks
+    // mix the row blocks and are dropped).  Sixteen blocks' loads are in flight per wave: the
+    // phase is a few trips to memory, not arithmetic.
+    constexpr int U = 16;
+    constexpr int RPB = RP == 8 ? 8 : 4;                    // rows a block covers
+    gsg_v4d acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = (gsg_v4d){0., 0., 0., 0.};
+    const int lr = lane >> 4, lc = lane & 15;
+    const int nblk = (r1 - r0 + RPB - 1) / RPB;
+    for (int b0 = wave; b0 < nblk; b0 += U * NW) {
+        float x[U][NC];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int blk = b0 + u * NW;
+            const int row = r0 + blk * RPB + (RP == 8 ? (lc >> 3) * 4 : 0) + lr;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const int col = RP == 8 ? (lc & 7) : c * 16 + lc;
+                const bool in = blk < nblk && row < r1;
+                x[u][c] = in ? a[(int64_t)row * RP + col] : 0.f;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            double d[NC];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) d[c] = (double)x[u][c];
+            int t = 0;
+#pragma unroll
+            for (int ci = 0; ci < NC; ++ci) {
+#pragma unroll
+                for (int cj = ci; cj < NC; ++cj) {
+                    acc[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(d[ci], d[cj], acc[t], 0, 0, 0);
+                    ++t;
+                }
+            }
+        }
+    }
+    // result register v of lane l is element (4 v + l / 16, l % 16) of the tile
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) tiles[wave][t][(4 * v + lr) * 16 + lc] = acc[t][v];
+    }
+}
+
+// entry (i, j), i <= j, of the share: the waves' partial tiles added in wave order
+template <int RP>
+__device__ __forceinline__ double
+gsg_tiles_entry(const double (*tiles)[(RP >= 16 ? (RP / 16) * (RP / 16 + 1) / 2 : 1)][256], int i, int j)
+{
+    constexpr int NW = kGsgThreads / 64;
+    constexpr int NC = RP >= 16 ? RP / 16 : 1;
+    const int ci = i >> 4, cj = j >> 4;
+    const int t = NC == 1 ? 0 : (ci == 0 ? cj : 2);
+    const int at = (i & 15) * 16 + (j & 15);
+    double s = 0.;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        s += tiles[w][t][at];
+        if (RP == 8) s += tiles[w][t][at + 8 * 16 + 8];   // the second row block's partial sum
+    }
+    return s;
+}
+
 // The r column steps on the upper triangle of the r x r Gram matrix in LDS (all T threads of the
 // workgroup call this; `gram` must be complete and visible).  Leaves b_ij in coef[i][j] (i < j) and
 // 1 / d_i in dinvf[i]; `dinv` is scratch.
@@ -233,54 +314,8 @@ gsg_kernel(GsgBatch batch, int count, float eps, GsgWs* ws, unsigned tag)
     if (tid == 0) failed = 0;
     GSG_STAMP(0);
 
-    // ---- 1. this workgroup's share of G: a wave takes blocks of four rows, lane = (row l / 16,
-    // column l % 16 of each column group); D[i][j] += sum_k A[k][i] A[k][j] over the block's rows.
-    // At rank 8 lanes 8..15 of a row group take the same columns of the NEXT four rows: the two
-    // diagonal 8 x 8 blocks of the product are then two partial sums of G (the off-diagonal blocks
-    // mix the row blocks and are dropped).  Sixteen blocks' loads are in flight per wave: the
-    // phase is a few trips to memory, not arithmetic.
-    constexpr int U = 16;
-    constexpr int RPB = RP == 8 ? 8 : 4;                    // rows a block covers
-    gsg_v4d acc[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) acc[t] = (gsg_v4d){0., 0., 0., 0.};
-    const int lr = lane >> 4, lc = lane & 15;
-    const int nblk = (r1 - r0 + RPB - 1) / RPB;
-    for (int b0 = wave; b0 < nblk; b0 += U * NW) {
-        float x[U][NC];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int blk = b0 + u * NW;
-            const int row = r0 + blk * RPB + (RP == 8 ? (lc >> 3) * 4 : 0) + lr;
-#pragma unroll
-            for (int c = 0; c < NC; ++c) {
-                const int col = RP == 8 ? (lc & 7) : c * 16 + lc;
-                const bool in = blk < nblk && row < r1;
-                x[u][c] = in ? a[(int64_t)row * RP + col] : 0.f;
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            double d[NC];
-#pragma unroll
-            for (int c = 0; c < NC; ++c) d[c] = (double)x[u][c];
-            int t = 0;
-#pragma unroll
-            for (int ci = 0; ci < NC; ++ci) {
-#pragma unroll
-                for (int cj = ci; cj < NC; ++cj) {
-                    acc[t] = __builtin_amdgcn_mfma_f64_16x16x4f64(d[ci], d[cj], acc[t], 0, 0, 0);
-                    ++t;
-                }
-            }
-        }
-    }
-    // result register v of lane l is element (4 v + l / 16, l % 16) of the tile
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-#pragma unroll
-        for (int v = 0; v < 4; ++v) tiles[wave][t][(4 * v + lr) * 16 + lc] = acc[t][v];
-    }
+    // ---- 1. this workgroup's share of G on the matrix cores
+    gsg_gram_tiles<RP>(a, r0, r1, tiles);
     __syncthreads();
     GSG_STAMP(1);
 
@@ -288,15 +323,7 @@ gsg_kernel(GsgBatch batch, int count, float eps, GsgWs* ws, unsigned tag)
     for (int e = tid; e < NG; e += T) {
         int i, j;
         gsg_entry(e, RP, &i, &j);
-        const int ci = i >> 4, cj = j >> 4;
-        const int t = NC == 1 ? 0 : (ci == 0 ? cj : 2);     // tiles in the order (0,0), (0,1), (1,1)
-        const int at = (i & 15) * 16 + (j & 15);
-        double s = 0.;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) {
-            s += tiles[w][t][at];
-            if (RP == 8) s += tiles[w][t][at + 8 * 16 + 8];   // the second row block's partial sum
-        }
+        const double s = gsg_tiles_entry<RP>(tiles, i, j);
         if (nwg > 1) {
             const unsigned long long bits = (unsigned long long)__double_as_longlong(s);
             const unsigned long long hi = ((unsigned long long)tag << 32) | (bits >> 32);

@@ -436,43 +436,47 @@ __device__ __forceinline__ void
 gram_solve_lds(const double* __restrict__ parts, int nparts, float eps, float* t_l)
 {
     constexpr int NG = RP * (RP + 1) / 2;
-    constexpr int G = T / NG;                 // groups of NG threads that add shares side by side
-    __shared__ double psum[G][NG];
+    constexpr bool kSideBySide = 2 * NG <= T;      // ranks up to 8: groups of NG threads add shares side by side
+    constexpr int G = kSideBySide ? T / NG : 1;
+    __shared__ double psum[G][kSideBySide ? NG : 1];
     __shared__ double gram[RP][RP + 1];
     __shared__ __attribute__((aligned(16))) float coef[RP][RP];
     __shared__ double dinv[RP];
     __shared__ float dinvf[RP];
     const int tid = threadIdx.x;
-    const int grp = tid / NG, e = tid - grp * NG;
-    if (grp < G) {
-        double s = 0.;
-#pragma unroll 8
-        for (int p = grp; p < nparts; p += G) s += parts[(size_t)p * NG + e];
-        psum[grp][e] = s;
-    }
     for (int i = tid; i < RP * RP; i += T) (&coef[0][0])[i] = 0.f;
-    __syncthreads();
-    if (tid < NG) {
-        double s = 0.;
-        for (int g = 0; g < G; ++g) s += psum[g][tid];       // the same order on every run
-        int i, j;
-        gsg_entry(tid, RP, &i, &j);
-        gram[i][j] = s;
+    if constexpr (kSideBySide) {
+        const int grp = tid / NG, e = tid - grp * NG;
+        if (grp < G) {
+            double s = 0.;
+#pragma unroll 8
+            for (int p = grp; p < nparts; p += G) s += parts[(size_t)p * NG + e];
+            psum[grp][e] = s;
+        }
+        __syncthreads();
+        if (tid < NG) {
+            double s = 0.;
+            for (int g = 0; g < G; ++g) s += psum[g][tid];       // the same order on every run
+            int i, j;
+            gsg_entry(tid, RP, &i, &j);
+            gram[i][j] = s;
+        }
+    } else {
+        // more entries than threads to share them out: a thread adds all shares of its entries, in order
+        for (int e = tid; e < NG; e += T) {
+            double s = 0.;
+#pragma unroll 4
+            for (int p = 0; p < nparts; ++p) s += parts[(size_t)p * NG + e];
+            int i, j;
+            gsg_entry(e, RP, &i, &j);
+            gram[i][j] = s;
+        }
     }
     __syncthreads();
     gsg_recurrence<RP, T>(gram, coef, dinv, dinvf, eps, tid);
     for (int i = tid; i < RP * RP; i += T) t_l[i] = (&coef[0][0])[i];
     if (tid < RP) t_l[RP * RP + tid] = dinvf[tid];
     __syncthreads();
-}
-
-template <int RP, int T>
-__device__ __forceinline__ void
-gram_solve_body(const double* __restrict__ parts, int nparts, float* __restrict__ tmat, float eps)
-{
-    __shared__ float t_l[RP * RP + RP];
-    gram_solve_lds<RP, T>(parts, nparts, eps, t_l);
-    for (int i = threadIdx.x; i < RP * RP + RP; i += T) tmat[i] = t_l[i];
 }
 
 // x_k -= b_ik x_i (k > i), x_i *= 1 / d_i for i = 0 .. r - 1: the reference's column steps
@@ -485,6 +489,30 @@ __device__ __forceinline__ void gram_apply_row(float* x, const float* t_l)
 #pragma unroll
         for (int k = i + 1; k < RP; ++k) x[k] = fmaf(-t_l[i * RP + k], x[i], x[k]);
         x[i] = __fmul_rn(x[i], t_l[RP * RP + i]);
+    }
+}
+
+// tmat receives the steps themselves (b_ij, 1 / d_i) or, EXPLICIT, their product: the upper
+// triangular matrix T with orth(A) = A T, row-major [RP][RP] (row i is what the steps make of the
+// unit vector e_i).  A row times T is RP independent multiply-adds a column where the steps are a
+// chain of RP dependent exchanges, which is what the wide fix launch needs.
+template <int RP, int T, bool EXPLICIT = false>
+__device__ __forceinline__ void
+gram_solve_body(const double* __restrict__ parts, int nparts, float* __restrict__ tmat, float eps)
+{
+    __shared__ float t_l[RP * RP + RP];
+    gram_solve_lds<RP, T>(parts, nparts, eps, t_l);
+    if (!EXPLICIT) {
+        for (int i = threadIdx.x; i < RP * RP + RP; i += T) tmat[i] = t_l[i];
+        return;
+    }
+    if ((int)threadIdx.x < RP) {
+        float x[RP];
+#pragma unroll
+        for (int k = 0; k < RP; ++k) x[k] = k == (int)threadIdx.x ? 1.f : 0.f;
+        gram_apply_row<RP>(x, t_l);
+#pragma unroll
+        for (int k = 0; k < RP; ++k) tmat[threadIdx.x * RP + k] = x[k];
     }
 }
 
@@ -626,6 +654,104 @@ psgd_defer_fix_batch_kernel(PsgdBatch<DeferFixItem> b)
     }
 }
 
+// ---- ranks 16 and 32 ----
+// The shares of P^T P of a finished P (the matrix-core product leaves P in column splits that a
+// second kernel adds, so they cannot come out of the product itself): a workgroup per 256 rows,
+// on the matrix cores in double (the first phase of gsg_kernel).
+struct GramShareItem {
+    const float* a;
+    int64_t rows;
+    double* parts;           // [ceil(rows / 256)][RP (RP + 1) / 2]
+};
+
+template <int RP>
+__global__ void __launch_bounds__(kGsgThreads)
+psgd_gram_shares_batch_kernel(PsgdBatch<GramShareItem> b)
+{
+    constexpr int NC = RP / 16, NT = NC * (NC + 1) / 2, NG = RP * (RP + 1) / 2;
+    __shared__ double tiles[kGsgThreads / 64][NT][256];
+    int local;
+    const GramShareItem& it = b.item[psgd_batch_locate(b, &local)];
+    const int r0 = local * 256;
+    const int r1 = (int64_t)r0 + 256 < it.rows ? r0 + 256 : (int)it.rows;
+    gsg_gram_tiles<RP>(it.a, r0, r1, tiles);
+    __syncthreads();
+    for (int e = threadIdx.x; e < NG; e += kGsgThreads) {
+        int i, j;
+        gsg_entry(e, RP, &i, &j);
+        it.parts[(size_t)local * NG + e] = gsg_tiles_entry<RP>(tiles, i, j);
+    }
+}
+
+// P <- P T and Q <- (sum of the slab partials of the raw Q) T at ranks 16 and 32.  A workgroup
+// takes 32 rows; a thread adds the slabs of one 16-byte piece of a row (eight slabs requested
+// together: a matrix-core Q has up to 32 of them), the rows meet in LDS, and a wave then forms
+// row times T for a few rows at a time, a lane per column.
+template <int RP>
+__global__ void __launch_bounds__(256)
+psgd_defer_fix_wide_batch_kernel(PsgdBatch<DeferFixItem> b)
+{
+    constexpr int QPR = RP / 4;                 // 16-byte pieces of a row
+    constexpr int ROWS = 256 / QPR;             // rows a workgroup takes: 64 at rank 16, 32 at rank 32
+    __shared__ float t_l[RP * RP + RP];
+    __shared__ float rows_l[ROWS][RP + 1];
+    int local;
+    const DeferFixItem& it = b.item[psgd_batch_locate(b, &local)];
+    const bool is_p = local < it.pblocks;
+    const int64_t rows = is_p ? it.n : it.m;
+    const int lrow = threadIdx.x / QPR, piece = threadIdx.x - lrow * QPR;
+    const int64_t row = (int64_t)(is_p ? local : local - it.pblocks) * ROWS + lrow;
+    const int64_t rc = row < rows ? row : rows - 1;
+    const float* src = (is_p ? it.p : it.qsrc) + rc * RP + 4 * piece;
+    const int slabs = is_p ? 1 : it.slabs;
+    const int64_t stride = it.m * RP;
+    for (int i = threadIdx.x; i < RP * RP; i += 256) t_l[i] = it.tmat[i];      // T itself here (gram_solve_body, EXPLICIT)
+    float x[4] = {0.f, 0.f, 0.f, 0.f};
+    int sl = 0;
+    for (; sl + 8 <= slabs; sl += 8) {          // slabs in ascending order
+        float v[8][4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) ld4(src + (int64_t)(sl + u) * stride, v[u]);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) x[c] += v[u][c];
+    }
+    for (; sl < slabs; ++sl) {
+        float v[4];
+        ld4(src + (int64_t)sl * stride, v);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) x[c] += v[c];
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) rows_l[lrow][4 * piece + c] = x[c];
+    __syncthreads();
+    // row times T: a wave takes 64 / RP rows at a time, a lane per column, RP independent multiply-adds
+    // in ascending order of the row's entries
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int RPW = 64 / RP;                // rows a wave holds at once: 4 or 2
+    const int col = lane % RP, sub = lane / RP;
+    float out[ROWS / (4 * RPW)];
+#pragma unroll
+    for (int u = 0; u < ROWS / (4 * RPW); ++u) {
+        const int lr = wave * RPW + u * 4 * RPW + sub;
+        float acc = 0.f;
+#pragma unroll 8
+        for (int i = 0; i < RP; ++i) acc = fmaf(rows_l[lr][i], t_l[i * RP + col], acc);      // T is zero below the diagonal
+        out[u] = acc;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < ROWS / (4 * RPW); ++u) rows_l[wave * RPW + u * 4 * RPW + sub][col] = out[u];
+    __syncthreads();
+    if (row < rows) {
+        float o[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) o[c] = rows_l[lrow][4 * piece + c];
+        st4((is_p ? it.p : it.q) + row * RP + 4 * piece, o);
+    }
+}
+
 // ------------------------------------------- matrix-core products, batched ----
 // The MFMA kernels of conef_psgd_mfma.h over the matrices of a bucket: workgroup `local` of an
 // item is workgroup (local % its first grid dimension, local / it) of the single-matrix launch.
@@ -665,6 +791,24 @@ psgd_mfma_mtp_batch_kernel(PsgdBatch<MfmaMtpItem> b)
 {
     int local;
     const MfmaMtpItem& it = b.item[psgd_batch_locate(b, &local)];
+    psgd_mfma_mtp_body<V>(it.x, it.p, it.out, it.n, it.m, it.r, it.rows_per_slab, local % it.col_tiles, local / it.col_tiles);
+}
+
+// the same launch with the workgroups in front that solve the matrices' Gram systems (deferred
+// orthogonalisation of P at ranks 16 and 32)
+template <int V, int RP>
+__global__ void __launch_bounds__(kMfmaThreads)
+psgd_mfma_mtp_gram_batch_kernel(PsgdBatch<MfmaMtpItem> b, GramTask g)
+{
+    if ((int)blockIdx.x < g.count) {
+        gram_solve_body<RP, kMfmaThreads, true>(g.parts[blockIdx.x], g.nparts[blockIdx.x], g.tmat[blockIdx.x], g.eps);
+        return;
+    }
+    const int bx = (int)blockIdx.x - g.count;
+    int i = 0;
+    while (i + 1 < b.count && bx >= b.first[i + 1]) ++i;
+    const MfmaMtpItem& it = b.item[i];
+    const int local = bx - b.first[i];
     psgd_mfma_mtp_body<V>(it.x, it.p, it.out, it.n, it.m, it.r, it.rows_per_slab, local % it.col_tiles, local / it.col_tiles);
 }
 
@@ -2644,6 +2788,7 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
     std::vector<char> done((size_t)count, 0);
     std::vector<SumItem> sums;
     std::vector<int> sum_blocks;
+    bool riders_done = false;
     // matrix-core items: one launch per vector width (4, 2 or 1 floats a lane, by the alignment of x
     // and by how many workgroups the matrix has to bring to a launch it shares)
     int mfma_items = 0;
@@ -2663,7 +2808,8 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
             MfmaMtpItem mi = {it.x, it.p, out, it.n, (int)it.m, it.r, t.rows_per_slab, t.col_tiles};
             table.push_back(mi);
             blocks.push_back(t.col_tiles * t.slabs);
-            if (t.slabs > 1) {
+            if (outs) (*outs)[(size_t)k] = MtpRaw{out, t.slabs > 1 ? t.slabs : 1};
+            if (t.slabs > 1 && !gram) {
                 const int64_t cnt = it.m * it.r;
                 SumItem si = {out, it.q, cnt, t.slabs};
                 sums.push_back(si);
@@ -2672,6 +2818,25 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
             done[(size_t)k] = 1;
         }
         if (table.empty()) continue;
+        if (gram && !riders_done) {
+            // the Gram systems ride in the first of these launches
+            riders_done = true;
+            const int rp = rank_bound(items[0].r);
+            int rc = run_batches(table, blocks, [&](const PsgdBatch<MfmaMtpItem>& bt, int grid) {
+                const dim3 g3((unsigned)(grid + gram->count)), b3(kMfmaThreads);
+#define CONEF_MMG(V)                                                                                              \
+    do {                                                                                                          \
+        if (rp == 32) hipLaunchKernelGGL((psgd_mfma_mtp_gram_batch_kernel<V, 32>), g3, b3, 0, s, bt, *gram);       \
+        else hipLaunchKernelGGL((psgd_mfma_mtp_gram_batch_kernel<V, 16>), g3, b3, 0, s, bt, *gram);                \
+    } while (0)
+                if (v == 4) CONEF_MMG(4);
+                else if (v == 2) CONEF_MMG(2);
+                else CONEF_MMG(1);
+#undef CONEF_MMG
+            });
+            if (rc != CONEF_OK) return rc;
+            continue;
+        }
         int rc = run_batches(table, blocks, [&](const PsgdBatch<MfmaMtpItem>& bt, int grid) {
             if (v == 4) hipLaunchKernelGGL(psgd_mfma_mtp_batch_kernel<4>, dim3((unsigned)grid), dim3(kMfmaThreads), 0, s, bt);
             else if (v == 2) hipLaunchKernelGGL(psgd_mfma_mtp_batch_kernel<2>, dim3((unsigned)grid), dim3(kMfmaThreads), 0, s, bt);
@@ -2743,14 +2908,16 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
 }
 
 // ---- deferred orthogonalisation of P: host side ----
-// The end of a batch workspace holds the Gram shares (a workgroup of the first product each; at
-// most one per four rows) and the solved systems, 512 bytes a matrix.
-constexpr int64_t kDeferTmatBytes = 512;
+// The end of a batch workspace holds, per matrix, the shares of P^T P (ranks up to 8: one per
+// workgroup of the first product, at most one per four rows; ranks 16 and 32: one per 256 rows),
+// the solved system (b_ij and 1 / d_i) and, at ranks up to 8, the shares of Q^T Q (one per 256
+// rows of Q).
+inline int64_t defer_tmat_bytes(int rp) { return conef_align256((int64_t)(rp * rp + rp) * 4); }
 
 inline int64_t defer_gram_doubles(const ConefPsgdItem& it)
 {
     const int rp = rank_bound(it.r);
-    return ((it.n + 3) / 4) * (int64_t)(rp * (rp + 1) / 2);
+    return (rp <= 8 ? (it.n + 3) / 4 : (it.n + 255) / 256) * (int64_t)(rp * (rp + 1) / 2);
 }
 
 // shares of Q^T Q, one per 256 rows of Q (the fix launch leaves them for the workgroups that
@@ -2758,16 +2925,15 @@ inline int64_t defer_gram_doubles(const ConefPsgdItem& it)
 inline int64_t defer_qgram_doubles(const ConefPsgdItem& it)
 {
     const int rp = rank_bound(it.r);
-    return ((it.m + 255) / 256) * (int64_t)(rp * (rp + 1) / 2);
+    return rp <= 8 ? ((it.m + 255) / 256) * (int64_t)(rp * (rp + 1) / 2) : 0;
 }
 
 inline int64_t defer_region_bytes(const ConefPsgdItem* items, int count)
 {
     int64_t bytes = 0;
     for (int k = 0; k < count; ++k)
-        if (rank_bound(items[k].r) <= 8)
-            bytes += conef_align256(8 * defer_gram_doubles(items[k])) + kDeferTmatBytes +
-                     conef_align256(8 * defer_qgram_doubles(items[k]));
+        bytes += conef_align256(8 * defer_gram_doubles(items[k])) + defer_tmat_bytes(rank_bound(items[k].r)) +
+                 conef_align256(8 * defer_qgram_doubles(items[k]));
     return bytes;
 }
 
@@ -2817,7 +2983,7 @@ int round_products_deferred(const ConefPsgdItem* items, const ConefPsgdItem* mq_
         table.push_back(t);
         at += conef_align256(8 * defer_gram_doubles(it));
         tmats.push_back((float*)at);
-        at += kDeferTmatBytes;
+        at += defer_tmat_bytes(rp);
         qgrams.push_back((double*)at);
         at += conef_align256(8 * defer_qgram_doubles(it));
     }
@@ -2871,6 +3037,73 @@ int round_products_deferred(const ConefPsgdItem* items, const ConefPsgdItem* mq_
     CONEF_RANK_SWITCH(rp, CONEF_DFX)
 #undef CONEF_DFX
     return rc;
+}
+
+// The same for ranks 16 and 32, whose products run on the matrix cores: the shares of P^T P come
+// from a short launch of their own over the finished P, the systems ride in the second product's
+// first launch, and the fix launch is the wide form.  `mq_mode` as in conef_psgd_mq_batch_f32.
+int round_products_deferred_mfma(const ConefPsgdItem* items, const ConefPsgdItem* mq_items, int count, int mq_mode,
+                                 float alpha, float eps, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
+                                 hipStream_t s)
+{
+    if (count < 1 || count > kPsgdBatchMax || !workspace) return kMqsNoFit;
+    const int rp = items[0].r;
+    if (rp != 16 && rp != 32) return kMqsNoFit;
+    const int64_t region = defer_region_offset(items, count);
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0 || workspace_bytes < region + defer_region_bytes(items, count))
+        return kMqsNoFit;
+    for (int k = 0; k < count; ++k) {
+        const ConefPsgdItem& it = items[k];
+        if (it.r != rp || it.m % 4 != 0 || it.n > 0x7fffffffLL || !aligned16(it.x) || !aligned16(it.q) || !aligned16(it.p) ||
+            !aligned16(mq_items[k].q) || (mq_mode == 1 && !aligned16(it.err)))
+            return kMqsNoFit;
+    }
+    // the second product must run as matrix-core launches (the systems ride in the first of them)
+    // with their slabs inside the workspace
+    std::vector<int64_t> offs;
+    if (!mfma_partial_base(items, count, workspace, workspace_bytes, &offs)) return kMqsNoFit;
+    int rc = conef_psgd_mq_batch_f32(mq_items, count, mq_mode, alpha, a, b, workspace, workspace_bytes, (void*)s);
+    if (rc != CONEF_OK) return rc;
+    std::vector<GramShareItem> shares;
+    std::vector<int> share_blocks;
+    std::vector<float*> tmats;
+    GramTask gram;
+    gram.count = count;
+    gram.eps = eps;
+    char* at = (char*)workspace + region;
+    for (int k = 0; k < count; ++k) {
+        const ConefPsgdItem& it = items[k];
+        const int nb = (int)((it.n + 255) / 256);
+        shares.push_back(GramShareItem{it.p, it.n, (double*)at});
+        share_blocks.push_back(nb);
+        gram.parts[k] = (const double*)at;
+        gram.nparts[k] = nb;
+        at += conef_align256(8 * defer_gram_doubles(it));
+        tmats.push_back((float*)at);
+        gram.tmat[k] = (float*)at;
+        at += defer_tmat_bytes(rp) + conef_align256(8 * defer_qgram_doubles(it));
+    }
+    rc = run_batches(shares, share_blocks, [&](const PsgdBatch<GramShareItem>& bt, int grid) {
+        if (rp == 32) hipLaunchKernelGGL(psgd_gram_shares_batch_kernel<32>, dim3((unsigned)grid), dim3(kGsgThreads), 0, s, bt);
+        else hipLaunchKernelGGL(psgd_gram_shares_batch_kernel<16>, dim3((unsigned)grid), dim3(kGsgThreads), 0, s, bt);
+    });
+    if (rc != CONEF_OK) return rc;
+    std::vector<MtpRaw> raw((size_t)count);
+    rc = mtp_batch(items, count, workspace, workspace_bytes, s, &gram, &raw);
+    if (rc != CONEF_OK) return rc;
+    std::vector<DeferFixItem> fix;
+    std::vector<int> blocks;
+    const int rows_per_wg = 256 / (rp / 4);
+    for (int k = 0; k < count; ++k) {
+        const ConefPsgdItem& it = items[k];
+        const int pb = (int)((it.n + rows_per_wg - 1) / rows_per_wg), qb = (int)((it.m + rows_per_wg - 1) / rows_per_wg);
+        fix.push_back(DeferFixItem{it.p, raw[(size_t)k].src, it.q, tmats[(size_t)k], nullptr, it.n, it.m, raw[(size_t)k].slabs, pb});
+        blocks.push_back(pb + qb);
+    }
+    return run_batches(fix, blocks, [&](const PsgdBatch<DeferFixItem>& bt, int grid) {
+        if (rp == 32) hipLaunchKernelGGL(psgd_defer_fix_wide_batch_kernel<32>, dim3((unsigned)grid), dim3(256), 0, s, bt);
+        else hipLaunchKernelGGL(psgd_defer_fix_wide_batch_kernel<16>, dim3((unsigned)grid), dim3(256), 0, s, bt);
+    });
 }
 
 template <int RP, bool FAST>
@@ -3269,6 +3502,8 @@ int conef_psgd_round_ahead_f32(const ConefPsgdItem* items, int32_t count, int32_
                                           : round_products_deferred<2>(items, its, count, alpha, eps, a, b, workspace, workspace_bytes, hs, qs);
             if (rd == CONEF_OK) q_shares_made = want_next;
             if (rd != kMqsNoFit) return rd;
+            const int rm = round_products_deferred_mfma(items, its, count, mq_mode, alpha, eps, a, b, workspace, workspace_bytes, hs);
+            if (rm != kMqsNoFit) return rm;
         }
         int rp = conef_psgd_mq_batch_f32(its, count, mq_mode, alpha, a, b, workspace, workspace_bytes, stream);
         if (rp != CONEF_OK) return rp;
@@ -3332,6 +3567,51 @@ int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_m
 {
     return conef_psgd_round_ahead_f32(items, count, mq_mode, pqt_mode, alpha, beta, eps, a, b, nullptr, 0, nullptr,
                                       workspace, workspace_bytes, stream);
+}
+
+// The middle of a round as a call of its own, for a caller that splits the round (the hooks at
+// ranks above 8 do, to run the Gram-Schmidt of the new Q on a side stream): P = X Q with the Q of
+// `first` (items whose q may point elsewhere, or null for items' own), P orthogonalised,
+// Q = X^T P into items[k].q - deferred where the batch allows, as in conef_psgd_round_f32.
+int conef_psgd_products_f32(const ConefPsgdItem* items, const ConefPsgdItem* first, int32_t count, int32_t mq_mode,
+                            float alpha, float eps, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
+                            void* stream)
+{
+    if (count < 0 || (count > 0 && !items) || mq_mode < 0 || mq_mode > 2) return CONEF_ERR_INVALID;
+    if (count == 0) return CONEF_OK;
+    const ConefPsgdItem* its = first ? first : items;
+    for (int k = 0; k < count; ++k) {
+        const ConefPsgdItem& it = its[k];
+        if (!item_ok(items[k]) || !item_ok(it) || it.n != items[k].n || it.m != items[k].m || it.r != items[k].r ||
+            it.x != items[k].x || it.p != items[k].p)
+            return CONEF_ERR_INVALID;
+        if ((mq_mode == 1 && !it.err) || (mq_mode == 2 && (!it.cs || it.w < 1 || it.w > (1 << 30)))) return CONEF_ERR_INVALID;
+        if (mq_mode == 2 && it.plan_host && !conef_plan_matches((const ConefPlanHeader*)it.plan_host, it.n, it.m, it.w, a, b))
+            return CONEF_ERR_INVALID;
+    }
+    const char* defer_env = getenv("CONEF_ROUND_DEFER");
+    if (!(defer_env && defer_env[0] == '0')) {
+        hipStream_t hs = (hipStream_t)stream;
+        const int rd = mq_mode == 0   ? round_products_deferred<0>(items, its, count, 0.f, eps, a, b, workspace, workspace_bytes, hs, nullptr)
+                       : mq_mode == 1 ? round_products_deferred<1>(items, its, count, 0.f, eps, a, b, workspace, workspace_bytes, hs, nullptr)
+                                      : round_products_deferred<2>(items, its, count, alpha, eps, a, b, workspace, workspace_bytes, hs, nullptr);
+        if (rd != kMqsNoFit) return rd;
+        const int rm = round_products_deferred_mfma(items, its, count, mq_mode, alpha, eps, a, b, workspace, workspace_bytes, hs);
+        if (rm != kMqsNoFit) return rm;
+    }
+    int rc = conef_psgd_mq_batch_f32(its, count, mq_mode, alpha, a, b, workspace, workspace_bytes, stream);
+    if (rc != CONEF_OK) return rc;
+    std::vector<float*> mats((size_t)count);
+    std::vector<int64_t> rows((size_t)count);
+    std::vector<int32_t> ranks((size_t)count);
+    for (int k = 0; k < count; ++k) {
+        mats[(size_t)k] = items[k].p;
+        rows[(size_t)k] = items[k].n;
+        ranks[(size_t)k] = items[k].r;
+    }
+    rc = conef_gram_schmidt_batch_f32(mats.data(), rows.data(), ranks.data(), count, eps, workspace, workspace_bytes, stream);
+    if (rc != CONEF_OK) return rc;
+    return conef_psgd_mtp_batch_f32(items, count, workspace, workspace_bytes, stream);
 }
 
 // dense error feedback on the parts of a bucket that are not compressed: x += e; e = 0

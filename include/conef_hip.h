@@ -334,6 +334,15 @@ int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_m
                          float beta, float eps, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
                          void* stream);
 
+/* The middle of that round as a call of its own, for a caller that splits the round (the hooks above
+ * rank 8 do, to orthogonalise the new Q on a side stream meanwhile): P = X Q with the Q factors of
+ * `first` (a copy of `items` whose q may point elsewhere; null: items' own), P orthogonalised
+ * (powerSGD_hook.py:516-531), Q = X^T P into items[k].q.  Deferred orthogonalisation of P where the
+ * batch allows, as in conef_psgd_round_f32 (ranks 1, 2, 4, 8, 16, 32 of 16-byte shaped matrices). */
+int conef_psgd_products_f32(const ConefPsgdItem* items, const ConefPsgdItem* first, int32_t count, int32_t mq_mode,
+                            float alpha, float eps, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
+                            void* stream);
+
 /* The same round for callers that keep a second buffer per Q factor (q_next[k], [m,r] like items[k].q).
  * The reference orthogonalises a bucket's Q factors at the start of the bucket's next round
  * (powerSGD_hook.py:496-497), a launch of a few workgroups with the machine idle around it.  Here
