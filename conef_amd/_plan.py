@@ -70,9 +70,10 @@ class SketchPlan:
         """Decoded header fields (for tests and diagnostics)."""
         h = self.host
         i32 = h[:128].view(np.int32)
-        i64 = h[:128].view(np.int64)
+        i64 = h[:136].view(np.int64)
         return {"n": int(i64[1]), "d": int(i64[2]), "w": int(i32[6]), "a": int(i32[7]), "b": int(i32[8]),
                 "chunk_cols": int(i32[9]), "nchunks": int(i32[10]), "bin_buckets": int(i32[11]),
                 "nbins": int(i32[12]), "max_bin_records": int(i32[13]), "off_pos": int(i64[7]),
                 "off_seg": int(i64[8]), "off_csr": int(i64[9]), "off_ent": int(i64[10]), "off_pk": int(i64[11]),
-                "total_bytes": int(i64[12]), "workspace_bytes": int(i64[13]), "kind": int(i64[14])}
+                "total_bytes": int(i64[12]), "workspace_bytes": int(i64[13]), "kind": int(i64[14]),
+                "off_order": int(i64[16])}

@@ -374,7 +374,7 @@ def _run_round(state, bucket, error_mode):
         _lib.check(rc, "conef_psgd_round_f32")
     if error_mode == "topk":
         if (count and int(getattr(state, "hook_streams", 1) or 1) <= 1
-                and os.environ.get("CONEF_ROUND_AHEAD", "1") != "0"):
+                and os.environ.get("CONEF_ROUND_AHEAD", "1") != "0" and os.environ.get("CONEF_TOPK_SIDE", "1") != "0"):
             # The sparsification only touches the error tensors, which nobody reads before this bucket's
             # next round: it runs on a side stream while this stream goes on with the next bucket (five
             # streaming passes next to launches that are mostly latency).  Same kernels, same values.

@@ -310,7 +310,7 @@ gsg_kernel(GsgBatch batch, int count, float eps, GsgWs* ws, unsigned tag)
     const int r1 = r0 + slab < rows ? r0 + slab : rows;
     float* __restrict__ a = batch.a[it];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x;
     if (tid == 0) failed = 0;
     GSG_STAMP(0);
 

@@ -22,6 +22,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <vector>
 
 #include "conef_device.h"
@@ -55,7 +56,8 @@ struct ConefPlanHeader {
     int64_t total_bytes;
     int64_t workspace_bytes;   // staging buffer: n * d floats, rounded up (binned plans only)
     int64_t kind;              // kConefPlanBinned or kConefPlanRowlist
-    int64_t reserved[2];
+    int64_t seeds;             // sign-hash seeds the tables were built with, sa << 32 | sb
+    int64_t off_order;         // row lists: uint16[w], the buckets by falling list length (ties: by index)
 };
 
 inline int64_t conef_align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
@@ -81,6 +83,8 @@ inline bool conef_plan_shape(int64_t n, int64_t d, int32_t w, int32_t hint_chunk
         off += conef_align256(2 * d);
         h->off_pk = off;
         off += conef_align256(4 * d);
+        h->off_order = off;
+        off += conef_align256(2 * (int64_t)w);
         h->total_bytes = off;
         h->workspace_bytes = 0;
         return true;
@@ -136,7 +140,7 @@ inline bool conef_plan_fill(void* buf, const ConefPlanHeader& shape, int32_t a, 
     ConefPlanHeader h = shape;
     h.a = a;
     h.b = b;
-    h.reserved[0] = ((int64_t)(uint32_t)sa << 32) | (uint32_t)sb;      // sign-hash seeds the tables were built with
+    h.seeds = ((int64_t)(uint32_t)sa << 32) | (uint32_t)sb;
     const int64_t d = h.d;
     if (h.kind == kConefPlanRowlist) {
         char* rbase = (char*)buf;
@@ -154,6 +158,15 @@ inline bool conef_plan_fill(void* buf, const ConefPlanHeader& shape, int32_t a, 
         std::vector<uint32_t> cur(rcsr, rcsr + h.w);
         for (int64_t i = 0; i < d; ++i)       // ascending columns inside every bucket
             rent[cur[rpk[i] & 0x7fffffffu]++] = (uint16_t)((uint32_t)i | ((rpk[i] >> 31) << 15));
+        // The walk gives neighbouring lanes neighbouring entries of this order, so that the lanes of
+        // a wave walk lists of about the same length.
+        uint16_t* rord = (uint16_t*)(rbase + h.off_order);
+        std::vector<uint32_t> by_len((size_t)h.w);
+        for (int32_t j = 0; j < h.w; ++j) by_len[(size_t)j] = (uint32_t)j;
+        std::stable_sort(by_len.begin(), by_len.end(), [&](uint32_t x, uint32_t y) {
+            return rcsr[x + 1] - rcsr[x] > rcsr[y + 1] - rcsr[y];
+        });
+        for (int32_t j = 0; j < h.w; ++j) rord[j] = (uint16_t)by_len[(size_t)j];
         memcpy(rbase, &h, sizeof(h));
         return true;
     }
@@ -233,7 +246,7 @@ inline ConefRowlistView conef_rowlist_view(const ConefPlanHeader* host, const vo
 {
     const char* b = (const char*)dev;
     ConefRowlistView v = {(const uint32_t*)(b + host->off_csr), (const uint16_t*)(b + host->off_ent),
-                          (const uint32_t*)(b + host->off_pk)};
+                          (const uint32_t*)(b + host->off_pk), (const uint16_t*)(b + host->off_order)};
     return v;
 }
 

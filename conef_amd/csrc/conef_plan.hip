@@ -8,7 +8,7 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // the sign-hash seeds a plan's tables were built with
 inline bool plan_has_default_sign_seeds(const ConefPlanHeader* hp, int32_t a, int32_t b)
 {
-    return hp->reserved[0] == (((int64_t)(uint32_t)(a + 2) << 32) | (uint32_t)(b + 3));
+    return hp->seeds == (((int64_t)(uint32_t)(a + 2) << 32) | (uint32_t)(b + 3));
 }
 }  // namespace
 
@@ -142,7 +142,7 @@ int conef_randblock_conef_step_planned_f32(float* x, const float* cs_in, float* 
     if (!(start >= 0 && start < numel && block >= 1 && block <= numel)) return CONEF_ERR_INVALID;
     ConefBlock blk = conef_make_block(numel, start, block);
     if (hp->kind == kConefPlanRowlist) {
-        ConefListRandBlock front = {x, payload, blk, alpha, aligned16(x) && m % 4 == 0};
+        ConefListRandBlock front = {x, payload, blk, alpha};
         return conef_launch_rowlist(front, conef_rowlist_view(hp, plan_dev), cs_in, cs_out, n, m, w, beta,
                                     (hipStream_t)stream);
     }

@@ -1012,6 +1012,7 @@ struct ListPsgdResidual {
     const float* q;
     int r;
     static constexpr bool kNeedsCells = false;
+    struct Regs {};
     __device__ __forceinline__ void stage(int64_t row0, int rows, int d, int, float* vals, const float*,
                                           const uint32_t*) const
     {

@@ -70,6 +70,7 @@ struct ListItem {
     float* cs_out;
     int64_t n;
     int d, w, rb;
+    bool pk_lds;
 };
 
 __global__ void __launch_bounds__(kConefRowlistThreads)
@@ -78,7 +79,7 @@ randblock_rowlist_batch_kernel(RbBatch<ListItem> b, double one_minus_beta)
     int local, width;
     const ListItem& it = b.item[rb_locate(b, &local, &width)];
     conef_rowlist_body<float, ConefListRandBlock>(it.front, it.plan, it.cs_in, it.cs_out, it.n, it.d, it.w, it.rb,
-                                                  one_minus_beta, local);
+                                                  one_minus_beta, local, it.pk_lds);
 }
 
 template <typename Item, typename Go>
@@ -164,9 +165,8 @@ int conef_randblock_step_batch_f32(const ConefRandBlockItem* items, int32_t coun
         if (!hp || hp->kind != kConefPlanRowlist) continue;
         ConefRowlistShape shape;
         if (!conef_rowlist_shape(it.n, it.m, it.w, ConefListRandBlock::kNeedsCells, &shape)) return CONEF_ERR_INVALID;
-        ListItem t = {{it.x, it.payload, conef_make_block(it.n * it.m, it.start, it.block), alpha,
-                       aligned16(it.x) && it.m % 4 == 0},
-                      conef_rowlist_view(hp, it.plan_dev), it.cs_in, it.cs_out, it.n, (int)it.m, it.w, shape.rb};
+        ListItem t = {{it.x, it.payload, conef_make_block(it.n * it.m, it.start, it.block), alpha},
+                      conef_rowlist_view(hp, it.plan_dev), it.cs_in, it.cs_out, it.n, (int)it.m, it.w, shape.rb, shape.pk_lds};
         table.push_back(t);
         blocks.push_back((int)shape.tiles);
         if (shape.lds > lds) lds = shape.lds;

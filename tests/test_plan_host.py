@@ -105,10 +105,14 @@ def build_rowlist(n, d, w):
     assert lib.conef_plan_build_host(buf.ctypes.data, nb, n, d, w, A, B, 0, 0) == 0
     assert lib.conef_plan_kind(buf.ctypes.data) == 1
     assert lib.conef_plan_workspace_bytes(buf.ctypes.data) == 0
-    i64 = buf[:128].view(np.int64)
+    i64 = buf[:136].view(np.int64)
     csr = buf[int(i64[9]):int(i64[9]) + 4 * (w + 1)].view(np.uint32)
     ent = buf[int(i64[10]):int(i64[10]) + 2 * d].view(np.uint16)
     pk = buf[int(i64[11]):int(i64[11]) + 4 * d].view(np.uint32)
+    order = buf[int(i64[16]):int(i64[16]) + 2 * w].view(np.uint16)
+    # the walk's bucket order: every bucket once, longest list first, equal lengths by index
+    lengths = np.diff(csr.astype(np.int64))
+    np.testing.assert_array_equal(order.astype(np.int64), np.argsort(-lengths, kind="stable"))
     return csr, ent, pk
 
 
