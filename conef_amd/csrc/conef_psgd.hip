@@ -462,14 +462,36 @@ gram_solve_lds(const double* __restrict__ parts, int nparts, float eps, float* t
             gram[i][j] = s;
         }
     } else {
-        // more entries than threads to share them out: a thread adds all shares of its entries, in order
-        for (int e = tid; e < NG; e += T) {
-            double s = 0.;
-#pragma unroll 4
-            for (int p = 0; p < nparts; ++p) s += parts[(size_t)p * NG + e];
-            int i, j;
-            gsg_entry(e, RP, &i, &j);
-            gram[i][j] = s;
+        // more entries than threads to share them out: a thread adds all shares of its entries, in
+        // order, eight shares of each entry requested at a time (a share a trip otherwise: the sums
+        // of a 16-share rank-32 matrix were most of what this workgroup spent)
+        constexpr int EPT = (NG + T - 1) / T, kAhead = 8;
+        double s[EPT];
+#pragma unroll
+        for (int u = 0; u < EPT; ++u) s[u] = 0.;
+        for (int p0 = 0; p0 < nparts; p0 += kAhead) {
+            double v[EPT][kAhead];
+#pragma unroll
+            for (int u = 0; u < EPT; ++u) {
+                const int e = tid + u * T < NG ? tid + u * T : NG - 1;
+#pragma unroll
+                for (int q = 0; q < kAhead; ++q)
+                    v[u][q] = parts[(size_t)(p0 + q < nparts ? p0 + q : nparts - 1) * NG + e];
+            }
+#pragma unroll
+            for (int u = 0; u < EPT; ++u)
+#pragma unroll
+                for (int q = 0; q < kAhead; ++q)
+                    if (p0 + q < nparts) s[u] += v[u][q];
+        }
+#pragma unroll
+        for (int u = 0; u < EPT; ++u) {
+            const int e = tid + u * T;
+            if (e < NG) {
+                int i, j;
+                gsg_entry(e, RP, &i, &j);
+                gram[i][j] = s[u];
+            }
         }
     }
     __syncthreads();
@@ -506,7 +528,29 @@ gram_solve_body(const double* __restrict__ parts, int nparts, float* __restrict_
         for (int i = threadIdx.x; i < RP * RP + RP; i += T) tmat[i] = t_l[i];
         return;
     }
-    if ((int)threadIdx.x < RP) {
+    if constexpr (RP % 8 == 0 && RP * 8 <= T) {
+        // eight lanes a row of T, lane c holding columns c, c + 8, ...: step j takes x_j from the lane
+        // that holds it, the same multiply-adds in the same order as gram_apply_row on e_i
+        constexpr int M = RP / 8;
+        const int i = threadIdx.x >> 3, c = threadIdx.x & 7, lane = threadIdx.x & 63;
+        if (i < RP) {
+            float x[M];
+#pragma unroll
+            for (int m = 0; m < M; ++m) x[m] = c + 8 * m == i ? 1.f : 0.f;
+#pragma unroll
+            for (int j = 0; j < RP; ++j) {
+                const float xj = __shfl(x[j >> 3], (lane & ~7) | (j & 7), 64);
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    const int k = c + 8 * m;
+                    if (k > j) x[m] = fmaf(-t_l[j * RP + k], xj, x[m]);
+                    else if (k == j) x[m] = __fmul_rn(x[m], t_l[RP * RP + j]);
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < M; ++m) tmat[i * RP + c + 8 * m] = x[m];
+        }
+    } else if ((int)threadIdx.x < RP) {
         float x[RP];
 #pragma unroll
         for (int k = 0; k < RP; ++k) x[k] = k == (int)threadIdx.x ? 1.f : 0.f;
@@ -783,6 +827,7 @@ struct MfmaMtpItem {
     float* out;
     int64_t n;
     int m, r, rows_per_slab, col_tiles;
+    int v;              // floats a lane loads at a time (4, 2, 1): read by the launch that takes every width
 };
 
 template <int V>
@@ -794,9 +839,11 @@ psgd_mfma_mtp_batch_kernel(PsgdBatch<MfmaMtpItem> b)
     psgd_mfma_mtp_body<V>(it.x, it.p, it.out, it.n, it.m, it.r, it.rows_per_slab, local % it.col_tiles, local / it.col_tiles);
 }
 
-// the same launch with the workgroups in front that solve the matrices' Gram systems (deferred
-// orthogonalisation of P at ranks 16 and 32)
-template <int V, int RP>
+// the same with the workgroups in front that solve the matrices' Gram systems (deferred
+// orthogonalisation of P at ranks 16 and 32), and one launch for the matrices of every vector
+// width: the solving workgroups outlast the products of one width, and a launch per width would
+// each wait for its slowest workgroup
+template <int RP>
 __global__ void __launch_bounds__(kMfmaThreads)
 psgd_mfma_mtp_gram_batch_kernel(PsgdBatch<MfmaMtpItem> b, GramTask g)
 {
@@ -809,7 +856,10 @@ psgd_mfma_mtp_gram_batch_kernel(PsgdBatch<MfmaMtpItem> b, GramTask g)
     while (i + 1 < b.count && bx >= b.first[i + 1]) ++i;
     const MfmaMtpItem& it = b.item[i];
     const int local = bx - b.first[i];
-    psgd_mfma_mtp_body<V>(it.x, it.p, it.out, it.n, it.m, it.r, it.rows_per_slab, local % it.col_tiles, local / it.col_tiles);
+    const int ct = local % it.col_tiles, slab = local / it.col_tiles;
+    if (it.v == 4) psgd_mfma_mtp_body<4>(it.x, it.p, it.out, it.n, it.m, it.r, it.rows_per_slab, ct, slab);
+    else if (it.v == 2) psgd_mfma_mtp_body<2>(it.x, it.p, it.out, it.n, it.m, it.r, it.rows_per_slab, ct, slab);
+    else psgd_mfma_mtp_body<1>(it.x, it.p, it.out, it.n, it.m, it.r, it.rows_per_slab, ct, slab);
 }
 
 struct MfmaPqtItem {
@@ -2795,7 +2845,9 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
     int mfma_items = 0;
     for (int k = 0; k < count; ++k) mfma_items += rank_bound(items[k].r) >= 16;
     const int64_t want_wgs = mfma_items > 0 && 768 / mfma_items > 96 ? 768 / mfma_items : 96;
-    for (int v = 4; v >= 1 && mfma_partials; v >>= 1) {
+    // with riders: every width in the one launch they ride in (v = 0 below stands for "any")
+    for (int pass = 0; pass < (gram ? 1 : 3) && mfma_partials; ++pass) {
+        const int v = gram ? 0 : 4 >> pass;
         std::vector<MfmaMtpItem> table;
         std::vector<int> blocks;
         for (int k = 0; k < count; ++k) {
@@ -2804,9 +2856,9 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
             const uintptr_t xa = reinterpret_cast<uintptr_t>(it.x);
             const int vmax = (it.m % 4 == 0 && (xa & 15u) == 0) ? 4 : (it.m % 2 == 0 && (xa & 7u) == 0) ? 2 : 1;
             MfmaMtpShape t = mfma_mtp_shape(it.n, it.m, it.r, vmax, want_wgs < 512 ? want_wgs : 512);
-            if (t.v != v) continue;
+            if (v != 0 && t.v != v) continue;
             float* out = t.slabs > 1 ? mfma_partials + mfma_offs[(size_t)k] : it.q;
-            MfmaMtpItem mi = {it.x, it.p, out, it.n, (int)it.m, it.r, t.rows_per_slab, t.col_tiles};
+            MfmaMtpItem mi = {it.x, it.p, out, it.n, (int)it.m, it.r, t.rows_per_slab, t.col_tiles, t.v};
             table.push_back(mi);
             blocks.push_back(t.col_tiles * t.slabs);
             if (outs) (*outs)[(size_t)k] = MtpRaw{out, t.slabs > 1 ? t.slabs : 1};
@@ -2819,21 +2871,15 @@ int mtp_batch(const ConefPsgdItem* items, int count, void* workspace, int64_t wo
             done[(size_t)k] = 1;
         }
         if (table.empty()) continue;
-        if (gram && !riders_done) {
-            // the Gram systems ride in the first of these launches
+        if (gram) {
+            // the Gram systems ride in this launch (the caller has checked that the batch is one launch)
+            if (riders_done) return CONEF_ERR_INVALID;
             riders_done = true;
             const int rp = rank_bound(items[0].r);
             int rc = run_batches(table, blocks, [&](const PsgdBatch<MfmaMtpItem>& bt, int grid) {
                 const dim3 g3((unsigned)(grid + gram->count)), b3(kMfmaThreads);
-#define CONEF_MMG(V)                                                                                              \
-    do {                                                                                                          \
-        if (rp == 32) hipLaunchKernelGGL((psgd_mfma_mtp_gram_batch_kernel<V, 32>), g3, b3, 0, s, bt, *gram);       \
-        else hipLaunchKernelGGL((psgd_mfma_mtp_gram_batch_kernel<V, 16>), g3, b3, 0, s, bt, *gram);                \
-    } while (0)
-                if (v == 4) CONEF_MMG(4);
-                else if (v == 2) CONEF_MMG(2);
-                else CONEF_MMG(1);
-#undef CONEF_MMG
+                if (rp == 32) hipLaunchKernelGGL(psgd_mfma_mtp_gram_batch_kernel<32>, g3, b3, 0, s, bt, *gram);
+                else hipLaunchKernelGGL(psgd_mfma_mtp_gram_batch_kernel<16>, g3, b3, 0, s, bt, *gram);
             });
             if (rc != CONEF_OK) return rc;
             continue;
