@@ -455,15 +455,23 @@ def hook_steps(args, results):
         torch.cuda.synchronize()
         wall = (time.perf_counter() - t0) / reps * 1e3
         gpu = e0.elapsed_time(e1) / reps
+        # what the host spends on issuing one step, with nothing queued in front of it
+        issued = 1e9
+        for _ in range(3):
+            t1 = time.perf_counter()
+            step()
+            issued = min(issued, (time.perf_counter() - t1) * 1e3)
+            torch.cuda.synchronize()
         rec = {"case": name, "ms_per_step_wall": round(wall, 3), "ms_per_step_gpu_events": round(gpu, 3),
+               "ms_per_step_host_issue": round(issued, 3),
                "gradient_MB": round(4 * total / 1e6, 1), "buckets": len(buckets),
                "gradient_GBs": round(4 * total / 1e6 / max(wall, gpu), 1)}
         results.append(rec)
         if args.json:
             print(json.dumps(rec), flush=True)
         else:
-            print("%-58s %8.3f ms/step wall  %8.3f ms gpu  %8.1f MB gradient in %2d buckets  %7.1f GB/s of gradient" % (
-                name, wall, gpu, rec["gradient_MB"], len(buckets), rec["gradient_GBs"]), flush=True)
+            print("%-58s %8.3f ms/step wall  %8.3f ms gpu  %8.3f ms host  %8.1f MB gradient in %2d buckets  %7.1f GB/s of gradient" % (
+                name, wall, gpu, issued, rec["gradient_MB"], len(buckets), rec["gradient_GBs"]), flush=True)
         del state, hook, fakes, grads, step        # the case's device state goes before the next case (and before exit)
 
 

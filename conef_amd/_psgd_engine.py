@@ -38,18 +38,24 @@ def orthogonalize(matrix, epsilon=0, workspace=None):
     return workspace
 
 
-def orthogonalize_all(matrices, epsilon, ws_ptr, ws_len, stream):
+def orthogonalize_all(matrices, epsilon, ws_ptr, ws_len, stream, table=None):
     """Gram-Schmidt of independent [rows, r] device matrices, side by side in as few launches as
-    their shapes allow."""
+    their shapes allow.  ``table``: what an earlier call over the same matrices returned (the host
+    arrays are reused while the matrices stay where they are); returns the table."""
     import ctypes
     count = len(matrices)
     if count == 0:
-        return
-    ptrs = (ctypes.c_void_p * count)(*[m.data_ptr() for m in matrices])
-    rows = (ctypes.c_int64 * count)(*[m.shape[0] for m in matrices])
-    ranks = (ctypes.c_int32 * count)(*[m.shape[1] for m in matrices])
+        return None
+    key = tuple(m.data_ptr() for m in matrices)
+    if table is None or table[0] != key:
+        ptrs = (ctypes.c_void_p * count)(*key)
+        rows = (ctypes.c_int64 * count)(*[m.shape[0] for m in matrices])
+        ranks = (ctypes.c_int32 * count)(*[m.shape[1] for m in matrices])
+        table = (key, ptrs, rows, ranks)
+    _, ptrs, rows, ranks = table
     rc = _lib.load().conef_gram_schmidt_batch_f32(ptrs, rows, ranks, count, float(epsilon), ws_ptr, ws_len, stream)
     _lib.check(rc, "conef_gram_schmidt_batch_f32")
+    return table
 
 
 # one buffer per (device, stream), grown on demand; held and released by conef_amd._pools
@@ -73,10 +79,11 @@ def topk_sparsify(err, topk_ratio, workspace=None):
     return workspace
 
 
-def topk_sparsify_all(tensors, topk_ratio, table=None):
+def topk_sparsify_all(tensors, topk_ratio, table=None, stream=None):
     """``topk_sparsify`` of every tensor of a list (one stream, one device) with each pass a
     single launch over all of them.  ``table`` is what an earlier call over the same tensors
-    returned: the host arrays and the workspace are reused while the tensors stay where they are."""
+    returned: the host arrays and the workspace are reused while the tensors stay where they are.
+    ``stream``: the raw stream to launch on (torch's current one if None)."""
     import ctypes
     count = len(tensors)
     if count == 0:
@@ -94,7 +101,8 @@ def topk_sparsify_all(tensors, topk_ratio, table=None):
     elif table[5] != topk_ratio:
         return topk_sparsify_all(tensors, topk_ratio, None)
     _, ptrs, numels, ks, ws, _ = table
-    rc = lib.conef_topk_sparsify_batch_f32(ptrs, numels, ks, count, ws.data_ptr(), ws.numel(), _lib.stream_ptr(tensors[0]))
+    rc = lib.conef_topk_sparsify_batch_f32(ptrs, numels, ks, count, ws.data_ptr(), ws.numel(),
+                                           _lib.stream_ptr(tensors[0]) if stream is None else stream)
     _lib.check(rc, "conef_topk_sparsify_batch_f32")
     return table
 
@@ -107,7 +115,7 @@ class _RoundPlan:
     __slots__ = ("key", "shapes", "work", "passthrough", "before", "after", "total_ps", "total_qs", "arena_key", "ps",
                  "qs", "items", "count", "sketches", "fused_sketch", "batched_update", "residual_offsets",
                  "topk_table", "q_next", "q_next_ptrs", "q_next_ready", "made", "q_next_views", "items_next", "q_next_event",
-                 "topk_event")
+                 "topk_event", "ws_need", "handoff_event", "gs_table", "topk_number", "q_next_number")
 
 
 def _build_round(state, grads, shapes, key, error_mode):
@@ -140,6 +148,11 @@ def _build_round(state, grads, shapes, key, error_mode):
     plan.batched_update = False
     plan.topk_table = None
     plan.topk_event = None          # the side stream's top-k of this bucket's errors, to be waited for by its next round
+    plan.topk_number = None         # the side stream's running number of that top-k (None: nothing to wait for)
+    plan.q_next_number = None       # likewise for the Gram-Schmidt of the next round's Q factors
+    plan.ws_need = None             # bytes of workspace the batch entry points ask for (a function of the table's shapes)
+    plan.handoff_event = None       # recorded on the hook's stream where the side stream may start (one event, reused)
+    plan.gs_table = None            # host arrays of the side stream's Gram-Schmidt call
     # Second buffer for the Q factors, orthogonalised at the end of a round for the bucket's next
     # round (conef_psgd_round_ahead_f32).  Derived data: q_memory_dict keeps what the reference
     # keeps, and the flag falls with the plan whenever the state is replaced.
@@ -288,12 +301,14 @@ def _run_round(state, bucket, error_mode):
             if cnt not in errs:
                 errs[cnt] = DenseCS(m, n, state.sketch_size, device=device)
 
-    if plan.topk_event is not None:
-        # the errors this round adds are still being sparsified on the side stream
-        torch.cuda.current_stream(device).wait_event(plan.topk_event)
-        plan.topk_event = None
+    if plan.topk_number is not None:
+        # the errors this round adds to may still be being sparsified on the side stream
+        _pools.side_wait(device, _lib.current_stream(device), plan.topk_number)
+        plan.topk_number = None
     eps = float(state.orthogonalization_epsilon)
-    ws = _workspace(device, stream, max(lib.conef_psgd_batch_workspace_bytes(items, count), 256))
+    if plan.ws_need is None:
+        plan.ws_need = max(lib.conef_psgd_batch_workspace_bytes(items, count), 256)
+    ws = _workspace(device, stream, plan.ws_need)
     ws_ptr, ws_len = ws.data_ptr(), ws.numel()
     if need_randomize_qs:
         # same seeded CPU draws as the reference so every replica starts from the same Q (:479-494)
@@ -378,22 +393,26 @@ def _run_round(state, bucket, error_mode):
             # The sparsification only touches the error tensors, which nobody reads before this bucket's
             # next round: it runs on a side stream while this stream goes on with the next bucket (five
             # streaming passes next to launches that are mostly latency).  Same kernels, same values.
-            main = torch.cuda.current_stream(device)
-            done = torch.cuda.Event()
-            done.record(main)
+            if plan.handoff_event is None:
+                plan.handoff_event = torch.cuda.Event()
+            plan.handoff_event.record(_lib.current_stream(device))
             side = _pools.side_stream(device, 0, 1)
-            side.wait_event(done)
-            with torch.cuda.stream(side):
-                fresh = plan.topk_table is None
-                plan.topk_table = topk_sparsify_all([errs[cnt] for cnt in range(count)], state.topk_ratio, plan.topk_table)
-                if fresh:
-                    # memory the side stream works on must not go back to the allocator under it
-                    for cnt in range(count):
-                        errs[cnt].record_stream(side)
-                    plan.topk_table[4].record_stream(side)
-                if plan.topk_event is None:
-                    plan.topk_event = torch.cuda.Event()
-                plan.topk_event.record(side)
+            side.wait_event(plan.handoff_event)
+            fresh = plan.topk_table is None
+            if fresh:
+                with _lib.on_stream(side):          # the table's workspace is allocated on the stream that uses it
+                    plan.topk_table = topk_sparsify_all([errs[cnt] for cnt in range(count)], state.topk_ratio, None)
+                # memory the side stream works on must not go back to the allocator under it
+                for cnt in range(count):
+                    errs[cnt].record_stream(side)
+                plan.topk_table[4].record_stream(side)
+            else:
+                plan.topk_table = topk_sparsify_all([errs[cnt] for cnt in range(count)], state.topk_ratio, plan.topk_table,
+                                                    side.cuda_stream)
+            if plan.topk_event is None:
+                plan.topk_event = torch.cuda.Event()
+            plan.topk_event.record(side)
+            plan.topk_number = _pools.side_recorded(device, plan.topk_event)
         else:
             plan.topk_table = topk_sparsify_all([errs[cnt] for cnt in range(count)], state.topk_ratio, plan.topk_table)
     elif residual is not None and mode3 != 3:
@@ -412,7 +431,7 @@ def _run_round(state, bucket, error_mode):
 def _round_with_q_on_the_side(state, plan, lib, items, count, mode1, mode3, alpha, eps, ws_ptr, ws_len, stream, device,
                               q_mem, qs):
     import ctypes
-    main = torch.cuda.current_stream(device)
+    main = _lib.current_stream(device)
     fresh_q_next = plan.q_next is None
     if fresh_q_next:
         plan.q_next = torch.empty_like(q_mem)
@@ -427,7 +446,7 @@ def _round_with_q_on_the_side(state, plan, lib, items, count, mode1, mode3, alph
         for k in range(count):                              # pointers of the table can move between steps (err, cs)
             ctypes.memmove(ctypes.byref(plan.items_next[k]), ctypes.byref(items[k]), ctypes.sizeof(items[k]))
             plan.items_next[k].q = plan.q_next_views[k].data_ptr()
-        main.wait_event(plan.q_next_event)
+        _pools.side_wait(device, main, plan.q_next_number)
         first = plan.items_next
     else:
         orthogonalize_all(qs, eps, ws_ptr, ws_len, stream)
@@ -436,17 +455,20 @@ def _round_with_q_on_the_side(state, plan, lib, items, count, mode1, mode3, alph
     rc = lib.conef_psgd_products_f32(items, first, count, mode1, float(alpha), eps, HASH_A, HASH_B, ws_ptr, ws_len, stream)
     _lib.check(rc, "conef_psgd_products_f32")
     # the new Q is final: orthogonalise a copy of it on the side
-    q_final = torch.cuda.Event()
-    q_final.record(main)
+    if plan.handoff_event is None:
+        plan.handoff_event = torch.cuda.Event()
+    plan.handoff_event.record(main)
     side = _pools.side_stream(device, 0, 1)
-    side.wait_event(q_final)
+    side.wait_event(plan.handoff_event)
     if fresh_q_next:
         plan.q_next.record_stream(side)       # memory the side stream works on must not go back to the allocator under it
-    with torch.cuda.stream(side):
+    with _lib.on_stream(side):
         plan.q_next.copy_(q_mem, non_blocking=True)
         side_ws = _workspace(device, side.cuda_stream, max(ws_len, 256))
-        orthogonalize_all(plan.q_next_views, eps, side_ws.data_ptr(), side_ws.numel(), side.cuda_stream)
-        plan.q_next_event.record(side)
+    plan.gs_table = orthogonalize_all(plan.q_next_views, eps, side_ws.data_ptr(), side_ws.numel(), side.cuda_stream,
+                                      plan.gs_table)
+    plan.q_next_event.record(side)
+    plan.q_next_number = _pools.side_recorded(device, plan.q_next_event)
     plan.q_next_ready = True
     beta = float(state.beta) if mode3 in (2, 3) else 0.0
     rc = lib.conef_psgd_pqt_batch_f32(items, count, 1 if mode3 == 3 else mode3, beta if mode3 == 2 else 0.0, HASH_A, HASH_B,
