@@ -79,6 +79,7 @@ SIGNATURES = {
     "conef_topk_sparsify_f32": [_P, _I64, _I64, _P, _I64, _P],
     "conef_topk_batch_workspace_bytes": [_P, _I32],
     "conef_topk_sparsify_batch_f32": [_P, _P, _P, _I32, _P, _I64, _P],
+    "conef_topk_sparsify_batch_kept_f32": [_P, _P, _P, _I32, _P, _I64, _P],
     "conef_topk_sparsify_noalloc_f32": [_P, _I64, _I64, _P],
     "conef_randblock_step_batch_f32": [_P, _I32, _I32, _F32, _F32, _I32, _I32, _P],
 }

@@ -96,14 +96,16 @@ def topk_sparsify_all(tensors, topk_ratio, table=None, stream=None):
         ptrs = (ctypes.c_void_p * count)(*key)
         numels = (ctypes.c_int64 * count)(*[t.numel() for t in tensors])
         ks = (ctypes.c_int64 * count)(*[max(1, int(0.5 * topk_ratio * t.numel())) for t in tensors])
-        ws = torch.empty(lib.conef_topk_batch_workspace_bytes(numels, count), dtype=torch.uint8, device=tensors[0].device)
+        # zero-filled once: the table keeps this workspace with these tensors, and the passes clear the
+        # selection state behind themselves (conef_topk_sparsify_batch_kept_f32)
+        ws = torch.zeros(lib.conef_topk_batch_workspace_bytes(numels, count), dtype=torch.uint8, device=tensors[0].device)
         table = (key, ptrs, numels, ks, ws, topk_ratio)
     elif table[5] != topk_ratio:
         return topk_sparsify_all(tensors, topk_ratio, None)
     _, ptrs, numels, ks, ws, _ = table
-    rc = lib.conef_topk_sparsify_batch_f32(ptrs, numels, ks, count, ws.data_ptr(), ws.numel(),
-                                           _lib.stream_ptr(tensors[0]) if stream is None else stream)
-    _lib.check(rc, "conef_topk_sparsify_batch_f32")
+    rc = lib.conef_topk_sparsify_batch_kept_f32(ptrs, numels, ks, count, ws.data_ptr(), ws.numel(),
+                                                _lib.stream_ptr(tensors[0]) if stream is None else stream)
+    _lib.check(rc, "conef_topk_sparsify_batch_kept_f32")
     return table
 
 

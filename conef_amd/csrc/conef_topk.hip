@@ -140,13 +140,25 @@ __device__ __forceinline__ void topk_resolve(TopkState* st, int p, uint32_t* pre
 // REP copies of every bin, copy = lane % REP, laid out [bin][copy]: the keys of a gradient crowd
 // into a few dozen bins of the first digit (one exponent and three mantissa bits), and lanes of a
 // wave that meet in a bin then add to different LDS banks instead of queueing on one address.
+// `kept` (a state that stays with its tensor from call to call, zero-filled before the first): no
+// launch clears the state; the first workgroup of pass 0 clears what the later passes count into,
+// and the filter's clears what pass 0 of the next call counts into (topk_filter_body).
 template <int REP>
 __device__ __forceinline__ void
-topk_hist_body(const float* __restrict__ x, int64_t numel, TopkState* st, int pass, int bx, int gx)
+topk_hist_body(const float* __restrict__ x, int64_t numel, TopkState* st, int pass, int bx, int gx, bool kept = false,
+               uint32_t k = 0)
 {
     __shared__ uint32_t bins[kBins * REP];
     uint32_t prefix = 0, remaining = 0, ties = 0;
     if (pass > 0) topk_resolve(st, pass - 1, &prefix, &remaining, &ties, bx);
+    if (kept && pass == 0 && bx == 0) {
+        for (int i = threadIdx.x; i < (kPasses - 1) * kBins; i += 256) (&st->hist[1][0])[i] = 0u;
+        if (threadIdx.x == 0) {
+            st->k = k;
+            st->done = 0u;
+            st->tie_count = 0u;
+        }
+    }
     const int nb = 1 << kDigitBits[pass];
     for (int i = threadIdx.x; i < nb * REP; i += 256) bins[i] = 0u;
     __syncthreads();
@@ -199,11 +211,11 @@ topk_hist_kernel(const float* __restrict__ x, int64_t numel, TopkState* st, int 
 }
 
 __global__ void __launch_bounds__(256)
-topk_hist_batch_kernel(TopkBatch b, int pass)
+topk_hist_batch_kernel(TopkBatch b, int pass, bool kept)
 {
     int local, width;
     const TopkItem& it = b.item[topk_locate(b.first, b.count, &local, &width)];
-    if (pass == 0) topk_hist_body<4>(it.x, it.numel, it.st, 0, local, width);
+    if (pass == 0) topk_hist_body<4>(it.x, it.numel, it.st, 0, local, width, kept, it.k);
     else topk_hist_body<1>(it.x, it.numel, it.st, pass, local, width);
 }
 
@@ -254,12 +266,14 @@ __device__ __forceinline__ void topk_order_ties(float* __restrict__ x, int64_t n
 
 // keep key >= threshold, zero the rest, settle surplus ties on the threshold by index
 __device__ __forceinline__ void
-topk_filter_body(float* __restrict__ x, int64_t numel, TopkState* st, int bx, int gx)
+topk_filter_body(float* __restrict__ x, int64_t numel, TopkState* st, int bx, int gx, bool kept = false)
 {
     __shared__ uint32_t ticket;
     __shared__ uint32_t idx_l[kTieMax];
     uint32_t thr, keep_ties, ties;
     topk_resolve(st, kPasses - 1, &thr, &keep_ties, &ties, bx);
+    if (kept && bx == 0)       // nobody reads the first digit's counters any more: ready for the next call
+        for (int i = threadIdx.x; i < kBins; i += 256) st->hist[0][i] = 0u;
     const bool surplus = ties != keep_ties && thr != 0u;      // a zero threshold has only zeros for ties
     const bool listed = surplus && ties <= (uint32_t)kTieMax;
     auto note = [&](int64_t i) {
@@ -335,11 +349,11 @@ topk_filter_kernel(float* __restrict__ x, int64_t numel, TopkState* st)
 }
 
 __global__ void __launch_bounds__(256)
-topk_filter_batch_kernel(TopkBatch b)
+topk_filter_batch_kernel(TopkBatch b, bool kept)
 {
     int local, width;
     const TopkItem& it = b.item[topk_locate(b.first, b.count, &local, &width)];
-    topk_filter_body(it.x, it.numel, it.st, local, width);
+    topk_filter_body(it.x, it.numel, it.st, local, width, kept);
 }
 
 
@@ -433,8 +447,9 @@ int64_t conef_topk_batch_workspace_bytes(const int64_t* numels, int32_t count)
     return total > 256 ? total : 256;
 }
 
-int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const int64_t* ks, int32_t count,
-                                  void* workspace, int64_t workspace_bytes, void* stream)
+namespace {
+int topk_sparsify_batch(float* const* xs, const int64_t* numels, const int64_t* ks, int32_t count, void* workspace,
+                        int64_t workspace_bytes, void* stream, bool kept)
 {
     if (count < 0 || (count > 0 && (!xs || !numels || !ks))) return CONEF_ERR_INVALID;
     for (int i = 0; i < count; ++i)
@@ -464,12 +479,29 @@ int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const
         if (nb == 0) continue;
         b.first[nb] = wgs;
         b.count = nb;
-        hipLaunchKernelGGL(topk_init_batch_kernel, dim3((unsigned)nb), dim3(256), 0, s, b);
+        if (!kept) hipLaunchKernelGGL(topk_init_batch_kernel, dim3((unsigned)nb), dim3(256), 0, s, b);
         for (int pass = 0; pass < kPasses; ++pass)
-            hipLaunchKernelGGL(topk_hist_batch_kernel, dim3((unsigned)wgs), dim3(256), 0, s, b, pass);
-        hipLaunchKernelGGL(topk_filter_batch_kernel, dim3((unsigned)wgs), dim3(256), 0, s, b);
+            hipLaunchKernelGGL(topk_hist_batch_kernel, dim3((unsigned)wgs), dim3(256), 0, s, b, pass, kept);
+        hipLaunchKernelGGL(topk_filter_batch_kernel, dim3((unsigned)wgs), dim3(256), 0, s, b, kept);
     }
     return (int)hipGetLastError();
+}
+}  // namespace
+
+int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const int64_t* ks, int32_t count,
+                                  void* workspace, int64_t workspace_bytes, void* stream)
+{
+    return topk_sparsify_batch(xs, numels, ks, count, workspace, workspace_bytes, stream, false);
+}
+
+// The same for a workspace that stays with its tensors: zero-filled by the caller before its first
+// use and passed to nothing but this entry point, with the same xs / numels / count, afterwards.
+// No launch clears the selection state then (the passes clear behind themselves): four launches a
+// call instead of five.
+int conef_topk_sparsify_batch_kept_f32(float* const* xs, const int64_t* numels, const int64_t* ks, int32_t count,
+                                       void* workspace, int64_t workspace_bytes, void* stream)
+{
+    return topk_sparsify_batch(xs, numels, ks, count, workspace, workspace_bytes, stream, true);
 }
 
 

@@ -382,6 +382,13 @@ int conef_topk_sparsify_f32(float* x, int64_t numel, int64_t k, void* workspace,
 int64_t conef_topk_batch_workspace_bytes(const int64_t* numels, int32_t count);
 int conef_topk_sparsify_batch_f32(float* const* xs, const int64_t* numels, const int64_t* ks, int32_t count,
                                   void* workspace, int64_t workspace_bytes, void* stream);
+/* The same call (hPowerSGD_hook.py:554, every matrix of a bucket) for a workspace that stays with
+ * its tensors from step to step: the caller zero-fills it once, before its first use, and passes
+ * it to nothing but this entry point, with the same xs / numels / count, afterwards.  The passes
+ * then clear the selection state behind themselves and the launch that clears it is left out (four
+ * launches a call instead of five).  Same results, bit for bit. */
+int conef_topk_sparsify_batch_kept_f32(float* const* xs, const int64_t* numels, const int64_t* ks, int32_t count,
+                                       void* workspace, int64_t workspace_bytes, void* stream);
 
 /* conef_topk_sparsify_f32 without a workspace argument and without any allocation.  No counterpart
  * in the reference: it is for callers that cannot allocate device memory - code under HIP graph

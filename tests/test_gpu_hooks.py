@@ -659,13 +659,30 @@ def test_topk_batch_exact(oracle):
             oracle.topk_sparsify(want, ratio)
             np.testing.assert_array_equal(to_np(d), want)
         assert float(arena[off:].abs().max()) == 0.0
-        # the cached table serves a second round over the same tensors
+        # the cached table serves the next rounds over the same tensors: its workspace is never
+        # cleared by a launch, the passes leave the selection state ready for the next call
+        for again in range(2):
+            for h, d in zip(host, dev):
+                d.copy_(h if again == 0 else -h)
+            assert topk_sparsify_all(dev, ratio, table) is table
+            for h, d in zip(host, dev):
+                want = (h if again == 0 else -h).numpy().copy()
+                oracle.topk_sparsify(want, ratio)
+                np.testing.assert_array_equal(to_np(d), want)
+        # the entry point that clears the state itself, on a workspace full of anything
+        import ctypes
+        from conef_amd import _lib
+        lib = _lib.load()
+        _, ptrs, numels, ks, ws, _ = table
+        junk = torch.full((ws.numel(),), 0xA5, dtype=torch.uint8, device="cuda")
         for h, d in zip(host, dev):
             d.copy_(h)
-        assert topk_sparsify_all(dev, ratio, table) is table
-        want = host[2].numpy().copy()
-        oracle.topk_sparsify(want, ratio)
-        np.testing.assert_array_equal(to_np(dev[2]), want)
+        _lib.check(lib.conef_topk_sparsify_batch_f32(ptrs, numels, ks, len(dev), junk.data_ptr(), junk.numel(),
+                                                     _lib.stream_ptr(arena)), "conef_topk_sparsify_batch_f32")
+        for h, d in zip(host, dev):
+            want = h.numpy().copy()
+            oracle.topk_sparsify(want, ratio)
+            np.testing.assert_array_equal(to_np(d), want)
 
 
 @pytest.mark.parametrize("mode", ["conef", "ef", "topk"])
