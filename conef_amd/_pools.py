@@ -78,6 +78,18 @@ def side_stream(device, bucket_index, count):
     return pool[bucket_index % count]
 
 
+_SIDE_EVENTS = {}
+
+
+def side_event(device, bucket_index, count):
+    """The event by which ``side_stream(device, bucket_index, count)`` is told where to start."""
+    key = (device, count, bucket_index % count)
+    event = _SIDE_EVENTS.get(key)
+    if event is None:
+        event = _SIDE_EVENTS[key] = torch.cuda.Event()
+    return event
+
+
 class _SideOrder:
     __slots__ = ("issued", "latest", "waited")
 
@@ -136,7 +148,7 @@ def release():
                     torch.cuda.synchronize(dev)
                 except Exception:      # a device that is already gone has nothing left to wait for
                     pass
-        for pool in (_PLANS, _STAGING, _WORKSPACES, _SCRATCH, _SIDE_STREAMS, _SIDE_ORDER):
+        for pool in (_PLANS, _STAGING, _WORKSPACES, _SCRATCH, _SIDE_STREAMS, _SIDE_ORDER, _SIDE_EVENTS):
             pool.clear()
 
 

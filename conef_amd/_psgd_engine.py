@@ -196,10 +196,16 @@ def run_round(state, bucket, error_mode):
     input_tensor = _bucket.buffer(bucket)
     if streams <= 1 or not input_tensor.is_cuda or state.iter < state.start_powerSGD_iter:
         return _run_round(state, bucket, error_mode)
-    side = _side_stream(input_tensor.device, _bucket.index(bucket), streams)
-    side.wait_stream(torch.cuda.current_stream(input_tensor.device))
+    device = input_tensor.device
+    index = _bucket.index(bucket)
+    side = _side_stream(device, index, streams)
+    # the side stream starts where the hook's stream is now (one event per side stream, recorded again
+    # for every bucket: a wait takes the event as it is when the wait is enqueued)
+    event = _pools.side_event(device, index, streams)
+    event.record(_lib.current_stream(device))
+    side.wait_event(event)
     input_tensor.record_stream(side)
-    with torch.cuda.stream(side):
+    with _lib.on_stream(side):
         return _run_round(state, bucket, error_mode)
 
 
