@@ -387,7 +387,7 @@ def hook_steps(args, results):
 
     ns = max(1, args.hook_streams)
 
-    def psgd(rank, ss, streams=1):
+    def psgd(rank, ss, streams=None):      # None: the state's own choice (two streams above rank 8)
         return lambda: (PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2,
                                       use_error_compression=True, sketch_size=ss, beta=0.9, hook_streams=streams),
                         powerSGD_hook)

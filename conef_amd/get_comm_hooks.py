@@ -27,7 +27,7 @@ def _lowrank(args):
 def _lowrank_eps(args):
     # hook_streams is not a flag of the reference's drivers: taken when the namespace has it
     return dict(_lowrank(args), orthogonalization_epsilon=args.orthogonalization_epsilon,
-                hook_streams=getattr(args, "hook_streams", 1))
+                hook_streams=getattr(args, "hook_streams", None))
 
 
 def _sketch(args):

@@ -685,7 +685,7 @@ def test_topk_batch_exact(oracle):
             np.testing.assert_array_equal(to_np(d), want)
 
 
-@pytest.mark.parametrize("mode", ["conef", "ef", "topk"])
+@pytest.mark.parametrize("mode", ["conef", "ef", "topk", "conef32"])
 def test_powersgd_rounds_on_side_streams(mode):
     """hook_streams > 1: the buckets of a step run on side streams and only the Futures order the
     caller after them.  Same kernels, same order per bucket: every result must equal the
@@ -701,9 +701,12 @@ def test_powersgd_rounds_on_side_streams(mode):
                                 topk_ratio=0.4, hook_streams=streams)
             hook = hpowerSGD_hook
         else:
-            st = PowerSGDState(None, matrix_approximation_rank=8, start_powerSGD_iter=2, use_error_feedback=True,
-                               use_error_compression=mode == "conef", sketch_size=0.1, beta=0.9, hook_streams=streams)
+            # rank 32 takes two streams when the state is not told otherwise (None)
+            st = PowerSGDState(None, matrix_approximation_rank=32 if mode == "conef32" else 8, start_powerSGD_iter=2,
+                               use_error_feedback=True, use_error_compression=mode.startswith("conef"), sketch_size=0.1,
+                               beta=0.9, hook_streams=None if mode == "conef32" and streams == 3 else streams)
             hook = powerSGD_hook
+            assert st.hook_streams == (2 if mode == "conef32" and streams == 3 else streams)
         st.iter = 2
         outs = []
         for step in range(4):
@@ -829,7 +832,7 @@ def test_high_rank_rounds_orthogonalise_q_on_a_side_stream(monkeypatch, rank, mo
 
     def make():
         st = PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, use_error_feedback=mode != "plain",
-                           use_error_compression=mode == "conef", sketch_size=0.1, beta=0.9)
+                           use_error_compression=mode == "conef", sketch_size=0.1, beta=0.9, hook_streams=1)
         st.iter = 2
         return st
 
