@@ -66,7 +66,12 @@ def test_randomblock_dense_ef_bit_exact(oracle, shapes, ratio):
                                              ([(2, 50_000)], 1.0, 0.2),
                                              # tensors that start 4, 8 and 12 bytes past a 16-byte boundary
                                              ([(1,), (21, 650), (2,), (33, 1023), (64, 576)], 0.2, 0.1),
-                                             ([(3,), (40, 650), (2,), (64, 576), (7, 333)], 0.3, 0.1)])
+                                             ([(3,), (40, 650), (2,), (64, 576), (7, 333)], 0.3, 0.1),
+                                             # row lists at their edges: rows of one to three columns (a quad of the
+                                             # flat run crosses several rows), one-row tiles of long rows (the column
+                                             # table stays in global memory), tiles taller than a thread's first quads
+                                             ([(2, 20_000), (50, 3), (9, 2), (300, 1), (3, 16_000), (5,)], 0.3, 0.25),
+                                             ([(1,), (700, 2), (130, 70), (16, 1100), (2, 24_576)], 0.6, 0.5)])
 @pytest.mark.parametrize("bucket_cls", [FakeGradBucket, OldApiGradBucket])
 def test_randomblock_conef_parity(oracle, shapes, ratio, ss, bucket_cls):
     from conef_amd.RandomBlock_hook import RandomBlock_hook, RandomBlockState
