@@ -49,7 +49,9 @@ class SketchPlan:
         """Staging buffer of a binned plan for work on torch's current stream: one buffer per
         (device, stream), shared by every sketch, live only inside a call."""
         dev = self.device.device
-        return _pools.staging(dev, torch.cuda.current_stream(dev).cuda_stream, max(self.workspace_bytes, 16))
+        stream = (_lib._raw_stream(dev.index if dev.index is not None else torch.cuda.current_device())
+                  if _lib._raw_stream is not None else torch.cuda.current_stream(dev).cuda_stream)
+        return _pools.staging(dev, stream, max(self.workspace_bytes, 16))
 
     @property
     def host_ptr(self):
