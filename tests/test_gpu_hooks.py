@@ -733,6 +733,38 @@ def test_powersgd_rounds_on_side_streams(mode):
         np.testing.assert_array_equal(x, y)
 
 
+def test_stream_helpers_fall_back_to_the_public_calls(monkeypatch):
+    """The hooks take the current stream and switch streams through two private torch calls where
+    they exist (no device lookups); without them the public calls must do the same job: an
+    hPowerSGD run on two hook streams with the top-k on its side stream, bit for bit."""
+    from conef_amd import _lib
+    from conef_amd.hPowerSGD_hook import hPowerSGDState, hpowerSGD_hook
+    buckets = [[(512, 256), (256,), (256, 512)], [(300, 300), (33, 40)]]
+
+    def run():
+        st = hPowerSGDState(None, matrix_approximation_rank=4, start_powerSGD_iter=2, use_error_compression=True,
+                            topk_ratio=0.4, hook_streams=2)
+        st.iter = 2
+        outs = []
+        for step in range(3):
+            gen = torch.Generator().manual_seed(70 + step)
+            flats = [(torch.randn(numel_of(b), generator=gen) * 1e-3).cuda() for b in buckets]
+            futs = [hpowerSGD_hook(st, FakeGradBucket(f, b, index=i, is_last=i == len(buckets) - 1))
+                    for i, (f, b) in enumerate(zip(flats, buckets))]
+            outs.append([to_np(f.wait()) for f in futs])
+        torch.cuda.synchronize()
+        return outs
+
+    fast = run()
+    assert _lib._current_stream_ids is not None and _lib._set_stream_ids is not None      # this torch has them
+    monkeypatch.setattr(_lib, "_current_stream_ids", None)
+    monkeypatch.setattr(_lib, "_set_stream_ids", None)
+    slow = run()
+    for a, b in zip(fast, slow):
+        for x, y in zip(a, b):
+            np.testing.assert_array_equal(x, y)
+
+
 @pytest.mark.parametrize("defer", ["0", "1"])
 @pytest.mark.parametrize("rank,ss,mode", [(8, 0.1, "conef"), (4, 0.2, "conef"), (2, 0.5, "conef"), (8, 0.1, "ef"),
                                           (4, 0.1, "topk"), (8, 0.1, "plain")])
