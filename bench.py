@@ -190,7 +190,16 @@ def main():
     plans = [cs.plan() for cs in sketches]
     planned = plans[0] is not None
     entry = "conef_randblock_conef_step_planned_f32" if planned else "conef_randblock_conef_step_f32"
+    # Everything the rotating states will ever allocate exists, and has been written once, before the
+    # first step: the second sketch buffer the step writes into, the payloads, the shared staging
+    # buffer.  A short run (a handful of warm-up steps for twelve states) then times steady-state
+    # steps, not first touches of fresh memory.
+    for cs, payload in zip(sketches, payloads):
+        (cs.spare_buffer() if planned else cs.next_buffer()).zero_()
+        payload.zero_()
     staging_ptr = plans[0].workspace.data_ptr() if planned else 0
+    if planned:
+        plans[0].workspace.zero_()
     plan_host_ptr, plan_dev_ptr = (plans[0].host_ptr, plans[0].device.data_ptr()) if planned else (0, 0)
 
     def one_step(i, g, b):

@@ -16,6 +16,7 @@ import torch.distributed as dist
 
 from . import _bucket
 from . import _lib
+from . import _pools
 from ._checkpoint import Checkpointable
 from .compressors.CountSketch import HASH_A, HASH_B, DenseCS
 
@@ -179,6 +180,15 @@ def RandomBlock_hook(state: RandomBlockState, bucket) -> torch.futures.Future[to
     starts = []
     randint = state.rng.randint     # RandomState.choice(n) of an int n draws randint(0, n): same stream (:218)
     written = []
+    staging = None
+    if state.use_error_compression:
+        # One staging buffer serves every binned sketch of the bucket (the launches run one after the
+        # other on this stream): it is sized for the largest of them before any pointer is taken, since
+        # the pool replaces its buffer when it has to grow.
+        need = max((p.workspace_bytes for p in (errors[cnt].plan() for cnt in range(count))
+                    if p is not None and not p.in_place), default=0)
+        if need:
+            staging = _pools.staging(device, stream, need).data_ptr()
     for cnt in range(count):
         it = items[cnt]
         start = int(randint(0, table.numels[cnt]))             # one draw per tensor, in bucket order (:218)
@@ -193,7 +203,7 @@ def RandomBlock_hook(state: RandomBlockState, bucket) -> torch.futures.Future[to
                 # the binned step reads the old sketch while it writes the new one
                 out = error.cs if plan.in_place else error.spare_buffer()
                 it.plan_host, it.plan_dev = plan.host_ptr, plan.device.data_ptr()
-                it.staging = None if plan.in_place else plan.workspace.data_ptr()
+                it.staging = None if plan.in_place else staging
             else:
                 out = error.next_buffer()
                 it.plan_host = it.plan_dev = it.staging = None

@@ -64,6 +64,7 @@ SIGNATURES = {
     "conef_psgd_pqt_conef_planned_f32": [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I32, _I32, _F32, _I32, _I32, _P],
     "conef_gram_schmidt_f32": [_P, _I64, _I32, _F32, _P, _I64, _P],
     "conef_gram_schmidt_batch_f32": [_P, _P, _P, _I32, _F32, _P, _I64, _P],
+    "conef_gram_schmidt_give_ups": [_P],
     "conef_ef_passthrough_f32": [_P, _P, _I64, _P],
     "conef_plan_bytes": [_I64, _I64, _I32, _I32, _I32],
     "conef_plan_build_host": [_P, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32],

@@ -58,6 +58,19 @@ def orthogonalize_all(matrices, epsilon, ws_ptr, ws_len, stream, table=None):
     return table
 
 
+def gram_schmidt_give_ups():
+    """How many Gram-Schmidt workgroups on the current device have run out their bounded wait for a
+    neighbouring workgroup since the library was loaded (each leaves NaN in its rows of the factor).
+    The kernels that spread one factor over several workgroups rely on those workgroups being
+    resident together; with several hook streams busy that is an assumption, and this is where its
+    failure shows before the NaN reaches a gradient.  Waits for the device.  With CONEF_CHECK_GS=1
+    every hook call ends with this check and raises."""
+    import ctypes
+    count = ctypes.c_int64(0)
+    _lib.check(_lib.load().conef_gram_schmidt_give_ups(ctypes.byref(count)), "conef_gram_schmidt_give_ups")
+    return count.value
+
+
 # one buffer per (device, stream), grown on demand; held and released by conef_amd._pools
 _workspace = _pools.workspace
 _scratch_f32 = _pools.scratch_f32
@@ -101,7 +114,7 @@ def topk_sparsify_all(tensors, topk_ratio, table=None, stream=None):
         ws = torch.zeros(lib.conef_topk_batch_workspace_bytes(numels, count), dtype=torch.uint8, device=tensors[0].device)
         table = (key, ptrs, numels, ks, ws, topk_ratio)
     elif table[5] != topk_ratio:
-        return topk_sparsify_all(tensors, topk_ratio, None)
+        return topk_sparsify_all(tensors, topk_ratio, None, stream)
     _, ptrs, numels, ks, ws, _ = table
     rc = lib.conef_topk_sparsify_batch_kept_f32(ptrs, numels, ks, count, ws.data_ptr(), ws.numel(),
                                                 _lib.stream_ptr(tensors[0]) if stream is None else stream)
@@ -171,6 +184,38 @@ def _build_round(state, grads, shapes, key, error_mode):
 
 
 _side_stream = _pools.side_stream
+
+
+def topk_table_is_stale(table, tensors, topk_ratio):
+    """Whether ``topk_sparsify_all`` would build a new table (and allocate its workspace) for these tensors."""
+    return table is None or table[0] != tuple(t.data_ptr() for t in tensors) or table[5] != topk_ratio
+
+
+def plan_for(state, bucket_index, grads, shapes, key, error_mode, device, stream_now):
+    """The bucket's cached round plan, rebuilt when its buffer or layout changed.  What the
+    replaced plan's last round left running on the side stream works on tensors that outlive the
+    plan (the error tensors in ``state.error_dict``, the Q arena): the pending top-k is handed on
+    to the new plan, whose round waits for it before it touches the errors, and the stream the
+    round is about to run on (``stream_now()``) is ordered after a pending copy of the Q arena
+    here, since the new plan no longer knows of it."""
+    plan = state.round_cache.get(bucket_index)
+    if plan is None or plan.key != key or plan.shapes != shapes:
+        old = plan
+        plan = _build_round(state, grads, shapes, key, error_mode)
+        if old is not None:
+            plan.topk_number, plan.topk_event = old.topk_number, old.topk_event
+            if old.q_next_number is not None:
+                _pools.side_wait(device, stream_now(), old.q_next_number)
+        state.round_cache[bucket_index] = plan
+    return plan
+
+
+def wait_for_side_topk(plan, device, stream_now):
+    """Orders the stream a round is about to run on after the side stream's top-k of the bucket's
+    error tensors from its previous round, if one may still be running."""
+    if plan.topk_number is not None:
+        _pools.side_wait(device, stream_now(), plan.topk_number)
+        plan.topk_number = None
 
 
 def settle(state):
@@ -244,10 +289,7 @@ def _run_round(state, bucket, error_mode):
     shapes = [t.shape for t in grads]
     key = (base_ptr, total_length, error_mode, state.matrix_approximation_rank, state.min_compression_rate,
            getattr(state, "sketch_size", None), dense_err.data_ptr() if dense_err is not None else 0)
-    plan = state.round_cache.get(bucket_index)
-    if plan is None or plan.key != key or plan.shapes != shapes:
-        plan = _build_round(state, grads, shapes, key, error_mode)
-        state.round_cache[bucket_index] = plan
+    plan = plan_for(state, bucket_index, grads, shapes, key, error_mode, device, lambda: _lib.current_stream(device))
     work, items, count = plan.work, plan.items, plan.count
     state.total_numel_before_compression += plan.before
     state.total_numel_after_compression += plan.after
@@ -309,10 +351,8 @@ def _run_round(state, bucket, error_mode):
             if cnt not in errs:
                 errs[cnt] = DenseCS(m, n, state.sketch_size, device=device)
 
-    if plan.topk_number is not None:
-        # the errors this round adds to may still be being sparsified on the side stream
-        _pools.side_wait(device, _lib.current_stream(device), plan.topk_number)
-        plan.topk_number = None
+    # the errors this round adds to may still be being sparsified on the side stream
+    wait_for_side_topk(plan, device, lambda: _lib.current_stream(device))
     eps = float(state.orthogonalization_epsilon)
     if plan.ws_need is None:
         plan.ws_need = max(lib.conef_psgd_batch_workspace_bytes(items, count), 256)
@@ -406,17 +446,18 @@ def _run_round(state, bucket, error_mode):
             plan.handoff_event.record(_lib.current_stream(device))
             side = _pools.side_stream(device, 0, 1)
             side.wait_event(plan.handoff_event)
-            fresh = plan.topk_table is None
-            if fresh:
-                with _lib.on_stream(side):          # the table's workspace is allocated on the stream that uses it
-                    plan.topk_table = topk_sparsify_all([errs[cnt] for cnt in range(count)], state.topk_ratio, None)
+            tensors = [errs[cnt] for cnt in range(count)]
+            # a table that no longer fits (an error tensor was replaced, another ratio) is a new one: its
+            # workspace has to be allocated and zero-filled on the stream whose kernels rely on the zeros
+            if topk_table_is_stale(plan.topk_table, tensors, state.topk_ratio):
+                with _lib.on_stream(side):
+                    plan.topk_table = topk_sparsify_all(tensors, state.topk_ratio, None)
                 # memory the side stream works on must not go back to the allocator under it
-                for cnt in range(count):
-                    errs[cnt].record_stream(side)
+                for t in tensors:
+                    t.record_stream(side)
                 plan.topk_table[4].record_stream(side)
             else:
-                plan.topk_table = topk_sparsify_all([errs[cnt] for cnt in range(count)], state.topk_ratio, plan.topk_table,
-                                                    side.cuda_stream)
+                plan.topk_table = topk_sparsify_all(tensors, state.topk_ratio, plan.topk_table, side.cuda_stream)
             if plan.topk_event is None:
                 plan.topk_event = torch.cuda.Event()
             plan.topk_event.record(side)
@@ -432,6 +473,9 @@ def _run_round(state, bucket, error_mode):
         state.p_memory_dict.clear()
         state.q_memory_dict.clear()
 
+    if os.environ.get("CONEF_CHECK_GS", "0") == "1" and gram_schmidt_give_ups():
+        raise RuntimeError("a Gram-Schmidt workgroup gave up waiting for its neighbours: the factors of bucket %d hold NaN"
+                           % bucket_index)
     state.maybe_increase_iter(bucket)
     return _bucket.completed_future(input_tensor)
 

@@ -26,6 +26,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "conef_gs_lanes.h"      // gs_count_give_up
+
 constexpr int kGsgThreads = 256;
 constexpr int kGsgMaxItems = 24;            // matrices per launch
 constexpr int kGsgMaxWgs = 128;             // workgroups per launch
@@ -177,12 +179,24 @@ gsg_tiles_entry(const double (*tiles)[(RP >= 16 ? (RP / 16) * (RP / 16 + 1) / 2 
 
 // The r column steps on the upper triangle of the r x r Gram matrix in LDS (all T threads of the
 // workgroup call this; `gram` must be complete and visible).  Leaves b_ij in coef[i][j] (i < j) and
-// 1 / d_i in dinvf[i]; `dinv` is scratch.
+// 1 / d_i in dinvf[i]; `dinv` and `diag0` (RP doubles each) are scratch.
+//
+// Columns that depend on earlier ones.  The squared norm a column has left when its turn comes is
+// G_ii minus what the earlier steps took away, and for a column that lies in the span of the earlier
+// ones that difference is rounding noise around zero, of either sign.  The reference
+// (powerSGD_hook.py:21-43) meets the same case in fp32: what its subtractions leave of such a column
+// is their own rounding residue, about 2^-23 of the column's original norm, which it then scales to
+// unit length - finite numbers that mean nothing.  A pivot below that residue, (2^-23)^2 of the
+// column's original G_ii, is therefore raised to it: the column comes out finite, as in the
+// reference, and no result above the reference's own noise changes.  A column that was zero to begin
+// with keeps its pivot of zero and gives NaN (eps = 0) or zeros (eps != 0), as in the reference.
 template <int RP, int T>
 __device__ __forceinline__ void gsg_recurrence(double (*gram)[RP + 1], float (*coef)[RP], double* dinv, float* dinvf,
-                                               float eps, int tid)
+                                               double* diag0, float eps, int tid)
 {
     constexpr int NG = RP * (RP + 1) / 2;
+    if (tid < RP) diag0[tid] = gram[tid][tid] * 0x1p-46;
+    __syncthreads();
     // Thread (j, part) owns
     // entries (j, k), k = j + part, j + part + parts, ...  Step i reads row i (final since the
     // barrier of step i - 1) and rewrites the rows below it; its coefficients go to `coef`, which
@@ -232,7 +246,8 @@ __device__ __forceinline__ void gsg_recurrence(double (*gram)[RP + 1], float (*c
             // 1 / d^2: hardware estimate and two Newton steps (exact to the last bits of a double)
             // instead of a division.  With eps = 0, d^2 is the pivot itself and the square root
             // for 1 / d waits until after the loop.
-            const double piv = P[a2][a2];
+            const double least = diag0[i0 + a2];
+            const double piv = P[a2][a2] < least ? least : P[a2][a2];
             double dd = piv;
             if (eps != 0.f) {
                 double y = __builtin_amdgcn_rsq(piv);
@@ -297,6 +312,7 @@ gsg_kernel(GsgBatch batch, int count, float eps, GsgWs* ws, unsigned tag)
     __shared__ double gram[RP][RP + 1];                     // upper triangle of the current Gram matrix
     __shared__ __attribute__((aligned(16))) float coef[RP][RP];       // b_ij for i < j, rounded once for step 4
     __shared__ double dinv[RP];                             // the pivots G_ii, then 1 / d_i
+    __shared__ double diag0[RP];                            // the least pivot each column may end up with
     __shared__ float dinvf[RP];
     __shared__ int failed;
 
@@ -378,13 +394,14 @@ gsg_kernel(GsgBatch batch, int count, float eps, GsgWs* ws, unsigned tag)
     __syncthreads();
     GSG_STAMP(2);
     if (failed) {
+        if (tid == 0) gs_count_give_up();
         // a half-orthogonalised matrix would pass for a result: leave one that cannot
         for (int e = tid; e < (r1 - r0) * RP; e += T) a[(int64_t)r0 * RP + e] = __builtin_nanf("");
         return;
     }
 
     // ---- 3. the r column steps on the r x r matrix
-    gsg_recurrence<RP, T>(gram, coef, dinv, dinvf, eps, tid);
+    gsg_recurrence<RP, T>(gram, coef, dinv, dinvf, diag0, eps, tid);
     GSG_STAMP(4);
 
     // ---- 4. the same steps on this workgroup's rows, a row per thread: the reference's column

@@ -30,6 +30,18 @@ constexpr int kGslMaxItems = 24;          // matrices per launch
 constexpr int kGslMaxWgs = 128;           // workgroups per launch
 constexpr unsigned kGslSpinLimit = 1u << 22;
 
+// Workgroups of the Gram-Schmidt kernels that exchange sums between workgroups inside one launch
+// (this file, conef_gs_gram.h, gram_schmidt_grid_kernel) wait for each other with a bounded spin.
+// One that runs out its wait leaves NaN in its rows and counts itself here, per GPU, since the
+// library was loaded: the host reads the count with conef_gram_schmidt_give_ups.  A diagnostic
+// only: nothing in the kernels reads it.
+static __device__ unsigned long long g_gs_give_ups;
+
+__device__ __forceinline__ void gs_count_give_up()
+{
+    __hip_atomic_fetch_add(&g_gs_give_ups, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Workspace of the kernel.  slot[i & 1][g][c]: workgroup g's sum for column c at step i, low word
 // the float, high word i + 1.
 struct GslWs {
@@ -151,6 +163,7 @@ gsl_kernel(GslBatch batch, int count, float eps, GslWs* ws)
         }
         __syncthreads();
         if (failed) {
+            if (tid == 0) gs_count_give_up();
             // a half-orthogonalised matrix would pass for a result: leave one that cannot
 #pragma unroll
             for (int t = 0; t < RPT; ++t) {

@@ -442,6 +442,7 @@ gram_solve_lds(const double* __restrict__ parts, int nparts, float eps, float* t
     __shared__ double gram[RP][RP + 1];
     __shared__ __attribute__((aligned(16))) float coef[RP][RP];
     __shared__ double dinv[RP];
+    __shared__ double diag0[RP];
     __shared__ float dinvf[RP];
     const int tid = threadIdx.x;
     for (int i = tid; i < RP * RP; i += T) (&coef[0][0])[i] = 0.f;
@@ -495,7 +496,7 @@ gram_solve_lds(const double* __restrict__ parts, int nparts, float eps, float* t
         }
     }
     __syncthreads();
-    gsg_recurrence<RP, T>(gram, coef, dinv, dinvf, eps, tid);
+    gsg_recurrence<RP, T>(gram, coef, dinv, dinvf, diag0, eps, tid);
     for (int i = tid; i < RP * RP; i += T) t_l[i] = (&coef[0][0])[i];
     if (tid < RP) t_l[RP * RP + tid] = dinvf[tid];
     __syncthreads();
@@ -1503,6 +1504,7 @@ __device__ __forceinline__ bool gs_grid_step(float (&v)[RPT][RP], float (&red)[4
             if (++spins > kGsSpinLimit || __hip_atomic_load(&ws->gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
                 ok = false;
                 __hip_atomic_store(&ws->gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                gs_count_give_up();
                 break;
             }
         }
@@ -2420,6 +2422,21 @@ int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* w
 #undef CONEF_GSS
     }
     return (int)hipGetLastError();
+}
+
+// Diagnostic: how many Gram-Schmidt workgroups on the current device have run out their bounded wait
+// for another workgroup (and left NaN in their rows) since the library was loaded.  Waits for the
+// device, then reads the library's per-GPU counter.
+int conef_gram_schmidt_give_ups(int64_t* count)
+{
+    if (!count) return CONEF_ERR_INVALID;
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) return (int)e;
+    unsigned long long v = 0;
+    e = hipMemcpyFromSymbol(&v, HIP_SYMBOL(g_gs_give_ups), sizeof(v), 0, hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return (int)e;
+    *count = (int64_t)v;
+    return CONEF_OK;
 }
 
 // Gram-Schmidt of `count` independent matrices (matrix k: mats[k], [rows[k], ranks[k]] row-major,

@@ -371,8 +371,8 @@ inline int64_t topk_hist_groups(int64_t numel)
 // ---- selection state of the entry point that allocates nothing ------------------------------
 // One TopkState per GPU, inside the code object: every GPU the library runs on holds its own
 // copy at its own address until the process ends.  `scratch` is only a host-side handle of the
-// symbol; device code and hipMemsetAsync need the address hipGetSymbolAddress returns for the
-// device that is current, looked up once per device and kept.
+// symbol; kernels (topk_init_kernel clears the state at the start of every call) need the address
+// hipGetSymbolAddress returns for the device that is current, looked up once per device and kept.
 constexpr size_t kScratchBytes = (sizeof(TopkState) + 255) / 256 * 256;      // 29 184 bytes
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 

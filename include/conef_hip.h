@@ -242,6 +242,14 @@ int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* w
 int conef_gram_schmidt_batch_f32(float* const* mats, const int64_t* rows, const int32_t* ranks, int32_t count,
                                  float eps, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Diagnostic, with no counterpart in the reference: *count = the number of Gram-Schmidt workgroups
+ * on the current device that ran out their bounded wait for a neighbouring workgroup of the same
+ * launch (about a second; they leave NaN in their rows) since the library was loaded.  The kernels
+ * that spread one matrix over several workgroups assume those workgroups are resident together (at
+ * most 128 of 256 threads); a count above zero says that assumption failed.  Unlike every other
+ * entry point this one waits for the device (HOST pointer, no stream). */
+int conef_gram_schmidt_give_ups(int64_t* count);
+
 /* Bytes of device workspace conef_gram_schmidt_f32 (matrices too large for LDS), conef_psgd_mtp_f32
  * (sums across row slabs) and the conef_psgd_mq_* family (sums across column splits at rank >= 16)
  * may need for an [n,m] matrix at rank r.  The sums meet in a fixed order: no atomics, results do

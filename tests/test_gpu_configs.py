@@ -215,12 +215,15 @@ def test_bert_large_powersgd_sketch10(rank):
     assert not _should_compress(2, 1024, 2, 2)[0]
 
 
-def test_bert_large_hpowersgd_topk_one_bucket():
+@pytest.mark.parametrize("rank", [8, 32])
+def test_bert_large_hpowersgd_topk_one_bucket(rank):
     """hPowerSGD keeps a dense per-matrix error cut down to the int(0.5 * 0.4 * numel) largest
-    magnitudes (hPowerSGD_hook.py:90-97,553-554): count and threshold property on a full bucket."""
+    magnitudes (hPowerSGD_hook.py:90-97,553-554): count and threshold property on a full bucket,
+    and the products against float64 on the device (Q = X^T P, M^ = P (P^T X), P orthonormal),
+    at the configuration's rank 8 and at its rank-32 variant."""
     from conef_amd.hPowerSGD_hook import _should_compress, hPowerSGDState, hpowerSGD_hook
     shapes = buckets_of(bert_large_shapes())[3]
-    state = hPowerSGDState(None, matrix_approximation_rank=8, start_powerSGD_iter=2, use_error_compression=True,
+    state = hPowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, use_error_compression=True,
                            topk_ratio=0.4)
     state.iter = 2
     total = sum(numel(s) for s in shapes)
@@ -228,21 +231,37 @@ def test_bert_large_hpowersgd_topk_one_bucket():
     for step in range(2):
         g = torch.randn(total, generator=gen, device="cuda") * 5e-4
         before = g.clone()
+        state.settle()
         old = {k: e.clone() for k, e in state.error_dict.get(0, {}).items()}
         hpowerSGD_hook(state, FakeGradBucket(g, shapes)).wait()
+        state.settle()                      # the top-k of this step's errors may run on a side stream
         cnt = 0
+        p_off = q_off = 0
+        p_mem, q_mem = state.p_memory_dict[0], state.q_memory_dict[0]
         for b, a, s in zip(views(before, shapes), views(g, shapes), shapes):
             n, m = s[0], numel(s) // s[0]
-            if not _should_compress(n, m, min(n, m, 8), 2)[0]:
+            r = min(n, m, rank)
+            if not _should_compress(n, m, r, 2)[0]:
+                assert torch.equal(a, b)
                 continue
             err = state.error_dict[0][cnt]
             k = max(1, int(0.5 * 0.4 * numel(s)))
             assert int((err != 0).sum()) == k
-            full = (b + old[cnt] if cnt in old else b) - a          # the residual before sparsification
+            x = (b + old[cnt] if cnt in old else b).reshape(n, m)    # gradient + remembered error
+            full = x - a.reshape(n, m)                               # the residual before sparsification
             kept = err != 0
-            assert torch.equal(err[kept], full.view_as(err)[kept])
-            assert float(full.view_as(err)[~kept].abs().max()) <= float(err[kept].abs().min())
+            assert torch.equal(err[kept], full[kept])
+            assert float(full[~kept].abs().max()) <= float(err[kept].abs().min())
+            p = p_mem[p_off:p_off + n * r].view(n, r)
+            q = q_mem[q_off:q_off + m * r].view(m, r)
+            p_off += n * r
+            q_off += m * r
+            x64, p64 = x.double(), p.double()
+            np.testing.assert_allclose((p64.t() @ p64).cpu().numpy(), np.eye(r), atol=5e-5, err_msg="P^T P of %s" % (s,))
+            assert_close(q, (x64.t() @ p64).float(), what="Q = X^T P of %s" % (s,))
+            assert_close(a.reshape(n, m), (p64 @ (p64.t() @ x64)).float(), what="projection identity of %s" % (s,))
             cnt += 1
+        assert p_off == p_mem.numel() and q_off == q_mem.numel()
 
 
 def lstm_gradient(shapes, step):

@@ -322,6 +322,26 @@ def test_randomblock_partition_invariants(oracle, conef):
                 # disjoint partition: output + residual == g + e bit for bit
                 np.testing.assert_array_equal(out + err, x)
                 assert (err[mask] == 0).all()
+            else:
+                # the composition of the sketched branch (RandomBlock_hook.py:190,231-243), through the
+                # sketch class alone: the block holds g + (1 - beta) * unsketch(old sketch), and the new
+                # sketch is ONE update, with beta, of that sum with the block zeroed
+                n, m = ins[ti].shape[0], ins[ti].size // ins[ti].shape[0]
+                twin = oracle.DenseCS(n, m, 0.5)
+                if old_err:
+                    twin.cs[...] = old_err[k]
+                x = ins[ti].reshape(n, m).copy()
+                twin.query(x, 1 - st.beta)
+                np.testing.assert_array_equal(out[mask], x.reshape(-1)[mask])
+                rest_of_x = np.where(mask, np.float32(0), x.reshape(-1)).reshape(n, m)
+                twin.update(rest_of_x, st.beta)
+                np.testing.assert_array_equal(st.error_dict[0][k].cs, twin.cs)
+                # and the update really took the zeroed copy: with the block left in, the sketch differs
+                other = oracle.DenseCS(n, m, 0.5)
+                if old_err:
+                    other.cs[...] = old_err[k]
+                other.update(x, st.beta)
+                assert not np.array_equal(other.cs, twin.cs)
             np.testing.assert_array_equal(np.concatenate([out[st.last_starts[k]:end], out[:rest]]),
                                           payload[off:off + block])
             off += block
