@@ -2,8 +2,9 @@
 
 The plan (built once per sketch by ``conef_plan_build_host``) lists where every column goes, so
 that the count-sketch update runs without atomics and adds each bucket's terms in ascending
-column order: per-bucket column lists when a row fits LDS (``kind`` 1), two binned streaming
-passes through a staging buffer for a few long rows (``kind`` 0).
+column order: per-bucket column lists when a row fits LDS (``kind`` 1), the same lists cut into
+column panels for longer rows of a tall matrix (``kind`` 2), two binned streaming passes through a
+staging buffer for long rows of a matrix with few of them (``kind`` 0).
 """
 import numpy as np
 import torch
@@ -57,11 +58,18 @@ class SketchPlan:
     def host_ptr(self):
         return self.host.ctypes.data
 
-    BINNED, ROWLIST = 0, 1
+    BINNED, ROWLIST, PANELS = 0, 1, 2
 
     @property
     def in_place(self):
-        """Whether the fused steps may write the sketch they read (row lists) or need a second buffer."""
+        """Whether the fused steps may write the sketch they read (row lists, whole or in panels) or
+        need a second buffer and a staging buffer (binned)."""
+        return self.kind in (self.ROWLIST, self.PANELS)
+
+    @property
+    def batchable(self):
+        """Whether the PowerSGD batch entry points (all sketches of a bucket in one launch, the
+        residual fused) take this plan: whole row lists only."""
         return self.kind == self.ROWLIST
 
     @staticmethod

@@ -342,7 +342,7 @@ def _run_round(state, bucket, error_mode):
                 it.w = cs.range
                 it.plan_host, it.plan_dev = (sk_plan.host_ptr, sk_plan.device.data_ptr()) if sk_plan is not None else (None, None)
                 plan.sketches.append((cs, sk_plan))
-            plan.batched_update = all(p is not None and p.in_place for _, p in plan.sketches)
+            plan.batched_update = all(p is not None and p.batchable for _, p in plan.sketches)
             plan.fused_sketch = state.matrix_approximation_rank <= 8 and plan.batched_update
         for cnt, (cs, _) in enumerate(plan.sketches):
             items[cnt].cs = cs.cs.data_ptr()

@@ -5,12 +5,14 @@ Differences a maintainer should know about:
   * the kernels are precompiled gfx950 code reached through libconef_hip.so, not CuPy/NVRTC;
   * alpha, beta, a, b travel by value, so ``a``/``b`` are Python ints, not 1-element device tensors;
   * updates run on a plan built once per sketch (no atomics, deterministic, the accumulation order
-    of the reference's serial definition): per-bucket column lists when a row fits LDS, two binned
-    streaming passes for a flat bucket viewed as at most 8 long rows.  The binned fused step writes
-    into a second buffer and ``self.cs`` is rebound to it; shapes neither kind covers (long rows
-    and more than 8 of them) fall back to float atomics;
+    of the reference's serial definition): per-bucket column lists when a row fits LDS, the same
+    lists in column panels for longer rows of a tall matrix, two binned streaming passes (over
+    groups of 8 rows) for long rows of a matrix with few of them.  The binned fused step writes
+    into a second buffer and ``self.cs`` is rebound to it.  A shape no plan covers falls back to
+    float atomics and says so in the log, once;
   * ``state_dict``/``load_state_dict`` round-trip (the reference's __setstate__ loses a, b).
 """
+import logging
 import os
 
 import torch
@@ -20,6 +22,17 @@ from .._plan import SketchPlan
 
 HASH_A = 994443   # CountSketch.py:112
 HASH_B = 609478   # CountSketch.py:113
+
+_WARNED = set()   # shapes that have been told about their fallback
+
+
+def _warn_no_plan(n, d, w):
+    """Once per shape: its updates run on float atomics (slower, and the order in which a cell
+    receives its terms is no longer fixed)."""
+    if (n, d, w) not in _WARNED:
+        _WARNED.add((n, d, w))
+        logging.warning("count sketch of a [%d, %d] tensor at width %d: no accumulation plan covers this shape, "
+                        "its updates fall back to float atomics (slower; accumulation order not fixed)" % (n, d, w))
 
 
 class DenseCS:
@@ -94,6 +107,10 @@ class DenseCS:
                     self._plan = SketchPlan.shared(self.N, self.D, self.range, self.a, self.b, self.cs.device, chunk, tbin)
                 except ValueError:       # e.g. one bucket collects more columns than a bin image can hold
                     self._plan = False
+            else:
+                self._plan = False
+            if self._plan is False:
+                _warn_no_plan(self.N, self.D, self.range)
         if self._plan is False:
             return None
         if self._plan is not None and self._plan.key != (self.N, self.D, self.range, self.a, self.b):

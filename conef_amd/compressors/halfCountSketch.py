@@ -30,11 +30,11 @@ class DenseCS:
         self._plan = None
 
     def plan(self):
-        """Row-list plan (built on first use) or None; CONEF_PLAN=0 disables it."""
+        """Row-list plan, whole or in column panels (built on first use), or None; CONEF_PLAN=0 disables it."""
         if self._plan is None and os.environ.get("CONEF_PLAN", "1") != "0":
             if SketchPlan.applicable(self.N, self.D, self.range):
                 plan = SketchPlan.shared(self.N, self.D, self.range, self.a, self.b, self.cs.device)
-                self._plan = plan if plan.kind == SketchPlan.ROWLIST else False
+                self._plan = plan if plan.kind in (SketchPlan.ROWLIST, SketchPlan.PANELS) else False
         return self._plan or None
 
     def state_dict(self):

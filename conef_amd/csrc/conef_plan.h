@@ -28,14 +28,20 @@
 #include "conef_device.h"
 #include "conef_sketch_core.h"
 #include "conef_rowlist.h"
+#include "conef_panels.h"
 
 constexpr uint32_t kConefPlanMagic = 0x50464E43u;   // "CNFP"
 constexpr int kConefPlanMaxRows = 8;
-// Two kinds of plan share the header.  Row lists (conef_rowlist.h): a row fits LDS, any number of
-// rows, tables csr / ent (column | sign << 15) / pk only, no staging buffer.  Binned (this file):
-// long rows, at most 8 of them.
+// Three kinds of plan share the header.  Row lists (conef_rowlist.h): a row fits LDS, any number of
+// rows, tables csr / ent (column | sign << 15) / pk only, no staging buffer.  Row lists in column
+// panels (conef_panels.h): rows too long for that on a matrix with rows enough to fill the machine,
+// tables ent / entb / pk, no staging buffer.  Binned (this file): a few long rows, in groups of up to 8.
 constexpr int64_t kConefPlanBinned = 0;
 constexpr int64_t kConefPlanRowlist = 1;
+constexpr int64_t kConefPlanPanels = 2;
+// Tall matrices go to the panels (one pass over the tensor); with fewer row tiles than this the
+// binned passes, which split the columns over the machine, are the better fit.
+constexpr int64_t kConefPanelMinTiles = 256;
 
 struct ConefPlanHeader {
     uint32_t magic;
@@ -48,6 +54,7 @@ struct ConefPlanHeader {
     int32_t nbins;
     int32_t max_bin_records;   // largest number of columns that map into one bin
     int64_t off_pos;           // uint16[d]: record position of column i inside its chunk image
+                               // (panels: the bucket of every list entry, `entb`)
     int64_t off_seg;           // uint32[nbins][nchunks+1]: (start inside chunk image) | (offset inside bin image << 16);
                                // entry [nchunks] holds the bin's record count in the high half
     int64_t off_csr;           // uint32[w+1]: first entry of bucket j
@@ -55,7 +62,7 @@ struct ConefPlanHeader {
     int64_t off_pk;            // uint32[d]: bucket | (sign bit << 31) of every column, for the column-order work
     int64_t total_bytes;
     int64_t workspace_bytes;   // staging buffer: n * d floats, rounded up (binned plans only)
-    int64_t kind;              // kConefPlanBinned or kConefPlanRowlist
+    int64_t kind;              // kConefPlanBinned, kConefPlanRowlist or kConefPlanPanels
     int64_t seeds;             // sign-hash seeds the tables were built with, sa << 32 | sb
     int64_t off_order;         // row lists: uint16[w], the buckets by falling list length (ties: by index)
 };
@@ -89,9 +96,34 @@ inline bool conef_plan_shape(int64_t n, int64_t d, int32_t w, int32_t hint_chunk
         h->workspace_bytes = 0;
         return true;
     }
-    if (n > kConefPlanMaxRows) return false;
+    ConefPanelShape pl;
+    const bool panels_fit = hint_chunk <= 0 && hint_bin <= 0 && conef_panel_shape(n, d, w, &pl);
+    if (panels_fit && pl.tiles >= kConefPanelMinTiles) {
+        memset(h, 0, sizeof(*h));
+        h->magic = kConefPlanMagic;
+        h->version = 1;
+        h->kind = kConefPlanPanels;
+        h->n = n;
+        h->d = d;
+        h->w = w;
+        h->chunk_cols = pl.pc;
+        h->nchunks = (int32_t)((d + pl.pc - 1) / pl.pc);
+        int64_t off = conef_align256(sizeof(ConefPlanHeader));
+        h->off_ent = off;
+        off += conef_align256(2 * d + 16);
+        h->off_pos = off;
+        off += conef_align256(2 * d + 16);
+        h->off_pk = off;
+        off += conef_align256(4 * d + 16);
+        h->total_bytes = off;
+        h->workspace_bytes = 0;
+        return true;
+    }
+    if (n / kConefPlanMaxRows > 65535) return false;     // the row groups are a grid dimension
     memset(h, 0, sizeof(*h));
-    int64_t c = hint_chunk > 0 ? hint_chunk : (100 * 1024) / (4 * n);   // a 100 KB chunk image: one workgroup per CU
+    // long rows in groups of up to 8: the tiles are those of a full group
+    const int64_t ng = n < kConefPlanMaxRows ? n : kConefPlanMaxRows;
+    int64_t c = hint_chunk > 0 ? hint_chunk : (100 * 1024) / (4 * ng);   // a 100 KB chunk image: one workgroup per CU
     if (c > 16384) c = 16384;
     c = c / 1024 * 1024;
     if (c < 1024) c = 1024;
@@ -101,7 +133,7 @@ inline bool conef_plan_shape(int64_t n, int64_t d, int32_t w, int32_t hint_chunk
     } else {
         // aim at a bin image of about 52 KB (two workgroups per CU): records = 52K / (4n),
         // buckets = records * w / d
-        double records = 52.0 * 1024 / (4.0 * n);
+        double records = 52.0 * 1024 / (4.0 * ng);
         t = (int64_t)(records * (double)w / (double)d);
         if (t >= 64) t = t / 64 * 64;      // narrow sketches: fewer buckets than lanes per bin rather than an image that overflows LDS
     }
@@ -168,6 +200,31 @@ inline bool conef_plan_fill(void* buf, const ConefPlanHeader& shape, int32_t a, 
         });
         for (int32_t j = 0; j < h.w; ++j) rord[j] = (uint16_t)by_len[(size_t)j];
         memcpy(rbase, &h, sizeof(h));
+        return true;
+    }
+    if (h.kind == kConefPlanPanels) {
+        char* pbase = (char*)buf;
+        memset(pbase, 0, (size_t)h.total_bytes);
+        uint16_t* pent = (uint16_t*)(pbase + h.off_ent);
+        uint16_t* pentb = (uint16_t*)(pbase + h.off_pos);
+        uint32_t* ppk = (uint32_t*)(pbase + h.off_pk);
+        ConefMod pmod = conef_make_mod(h.w);
+        for (int64_t i = 0; i < d; ++i) ppk[i] = conef_bucket_sign((int32_t)i, pmod, a, b, sa, sb);
+        const int64_t pc = h.chunk_cols;
+        std::vector<uint32_t> first((size_t)h.w + 1);
+        for (int64_t c0 = 0; c0 < d; c0 += pc) {
+            const int64_t c1 = c0 + pc < d ? c0 + pc : d;
+            std::fill(first.begin(), first.end(), 0u);
+            for (int64_t i = c0; i < c1; ++i) first[(ppk[i] & 0x7fffffffu) + 1]++;
+            for (int32_t j = 0; j < h.w; ++j) first[(size_t)j + 1] += first[(size_t)j];
+            for (int64_t i = c0; i < c1; ++i) {        // ascending columns inside every bucket
+                const uint32_t j = ppk[i] & 0x7fffffffu;
+                const uint32_t k = first[j]++;
+                pent[c0 + k] = (uint16_t)((uint32_t)(i - c0) | ((ppk[i] >> 31) << 15));
+                pentb[c0 + k] = (uint16_t)j;
+            }
+        }
+        memcpy(pbase, &h, sizeof(h));
         return true;
     }
     const int32_t w = h.w, C = h.chunk_cols, T = h.bin_buckets, nbins = h.nbins, nchunks = h.nchunks;
@@ -247,6 +304,14 @@ inline ConefRowlistView conef_rowlist_view(const ConefPlanHeader* host, const vo
     const char* b = (const char*)dev;
     ConefRowlistView v = {(const uint32_t*)(b + host->off_csr), (const uint16_t*)(b + host->off_ent),
                           (const uint32_t*)(b + host->off_pk), (const uint16_t*)(b + host->off_order)};
+    return v;
+}
+
+inline ConefPanelView conef_panel_view(const ConefPlanHeader* host, const void* dev)
+{
+    const char* b = (const char*)dev;
+    ConefPanelView v = {(const uint16_t*)(b + host->off_ent), (const uint16_t*)(b + host->off_pos),
+                        (const uint32_t*)(b + host->off_pk), host->chunk_cols};
     return v;
 }
 
@@ -354,9 +419,13 @@ static __device__ unsigned long long conef_trace_buf[2][1024][8];
 // the image leaves LDS with linear 16-byte stores.
 template <int NROWS, typename Stage, bool VEC>
 __global__ void __launch_bounds__(1024)
-conef_binned_stage_kernel(Stage stage, ConefPlanView plan, float* __restrict__ staging, int64_t d, int nblocks_padded)
+conef_binned_stage_kernel(Stage stage, ConefPlanView plan, float* __restrict__ staging, int64_t d, int nblocks_padded,
+                          int row_first)
 {
     extern __shared__ float conef_img[];   // [chunk_cols][NROWS]
+    // blockIdx.y: the group of NROWS rows, each with its own region of the staging buffer
+    const int rg = row_first + (int)blockIdx.y * NROWS;
+    staging += (int64_t)rg * d;
     const int chunk = conef_xcd_major(blockIdx.x, nblocks_padded, plan.flags);
     CONEF_STAMP(0, 0, 0);
     if (chunk >= plan.nchunks) return;
@@ -369,7 +438,7 @@ conef_binned_stage_kernel(Stage stage, ConefPlanView plan, float* __restrict__ s
         if (VEC && valid == 4) {
             float g[NROWS][4];
 #pragma unroll
-            for (int r = 0; r < NROWS; ++r) stage.load4(r, c0, g[r]);
+            for (int r = 0; r < NROWS; ++r) stage.load4(rg + r, c0, g[r]);
             const uint2 pp = *reinterpret_cast<const uint2*>(plan.pos + c0);   // chunk starts are multiples of 4
             const uint32_t p0 = (pp.x & 0xffffu) * NROWS, p1 = (pp.x >> 16) * NROWS;
             const uint32_t p2 = (pp.y & 0xffffu) * NROWS, p3 = (pp.y >> 16) * NROWS;
@@ -383,7 +452,7 @@ conef_binned_stage_kernel(Stage stage, ConefPlanView plan, float* __restrict__ s
         } else {
             for (int k = 0; k < valid; ++k) {
                 uint32_t pk = plan.pos[c0 + k] * NROWS;
-                for (int r = 0; r < NROWS; ++r) conef_img[pk + r] = stage.element(r, c0 + k);
+                for (int r = 0; r < NROWS; ++r) conef_img[pk + r] = stage.element(rg + r, c0 + k);
             }
         }
     }
@@ -430,28 +499,32 @@ template <int NROWS, bool FUSED_QUERY>
 __attribute__((amdgpu_num_sgpr(72))) __global__ void __launch_bounds__(1024, 8)
 conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView plan, const float* cs_in, float* cs_out,
                                int32_t w, float alpha, double one_minus_beta, int nblocks_padded, int max_bin_records,
-                               int glog, int col_threads, ConefBlockWork bw)
+                               int glog, int col_threads, ConefBlockWork bw, int row_first, int64_t d)
 {
     extern __shared__ float conef_img[];
     const int gthreads = blockDim.x - col_threads;      // threads that work on the bin
+    const float* cs_all = cs_in;                        // the column-order work looks up cells of any row
+    {
+        // blockIdx.y: the group of NROWS rows this workgroup's bin work is for
+        const int64_t rg = row_first + (int64_t)blockIdx.y * NROWS;
+        staging += rg * d;
+        cs_in += rg * w;
+        cs_out += rg * w;
+    }
     if ((int)threadIdx.x >= gthreads) {
         // ---- column-order work of the fused step.  These waves owe the bin's threads nothing:
         // they pass the workgroup's one barrier first and then work on their own.
         __syncthreads();
         CONEF_STAMP(1, gthreads, 5);
-        const int64_t me = blockIdx.x * (int64_t)col_threads + (threadIdx.x - gthreads);
-        const int64_t nworkers = (int64_t)gridDim.x * col_threads;
+        const int64_t me = ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * col_threads + (threadIdx.x - gthreads);
+        const int64_t nworkers = (int64_t)gridDim.x * gridDim.y * col_threads;
         const int64_t bquads = (bw.block + 3) >> 2;
         for (int64_t q = me; q < bquads; q += nworkers) {
             int64_t p0 = q << 2;
             int n = bw.block - p0 < 4 ? (int)(bw.block - p0) : 4;
             int64_t f = bw.blk.start + p0;
             if (f >= bw.numel) f -= bw.numel;
-            int64_t r = 0, col = f;                 // at most 8 rows: no 64-bit division needed
-            while (col >= bw.m) {
-                col -= bw.m;
-                ++r;
-            }
+            int64_t r = f / bw.m, col = f - r * bw.m;
             float* px[4];
             float g[4], cell[4];
             uint32_t pk[4];
@@ -471,7 +544,7 @@ conef_binned_accumulate_kernel(const float* __restrict__ staging, ConefPlanView 
                 }
             }
 #pragma unroll
-            for (int k = 0; k < 4; ++k) cell[k] = cs_in[rr[k] * (int64_t)w + (pk[k] & 0x7fffffffu)];
+            for (int k = 0; k < 4; ++k) cell[k] = cs_all[rr[k] * (int64_t)w + (pk[k] & 0x7fffffffu)];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 if (k < n) {
@@ -630,24 +703,17 @@ inline size_t conef_binned_lds_b(const ConefPlanHeader* hp, int nrows)
 }
 
 
+// Pass A over `groups` groups of NROWS rows, the first of them starting at row `row_first`.
 template <int NROWS, typename Stage>
-int conef_launch_binned_rows(Stage stage, const ConefPlanHeader* hp, const void* plan_dev, float* staging,
-                             const float* cs_in, float* cs_out, float alpha, float beta, bool vec_ok,
-                             ConefBlockWork bw, hipStream_t s)
+int conef_launch_stage_rows(Stage stage, const ConefPlanHeader* hp, const void* plan_dev, float* staging, bool vec_ok,
+                            int row_first, int groups, hipStream_t s)
 {
     ConefPlanView view = conef_plan_view(hp, plan_dev);
-    const double omb = 1. - (double)beta;
     size_t lds_a = (size_t)hp->chunk_cols * NROWS * 4;
-    size_t lds_b = conef_binned_lds_b(hp, NROWS);
-    if (lds_a > 160 * 1024 || lds_b > 160 * 1024) return CONEF_ERR_INVALID;
-    int ga = (hp->nchunks + 7) & ~7, gb = (hp->nbins + 7) & ~7;
+    if (lds_a > 160 * 1024) return CONEF_ERR_INVALID;
+    int ga = (hp->nchunks + 7) & ~7;
     int threads_a = (hp->chunk_cols / 4 + 63) & ~63;
     if (threads_a > 1024) threads_a = 1024;
-    int tpad = (hp->bin_buckets + 63) & ~63;
-    int col_threads = bw.x ? 256 : 0;                   // waves of pass B that do the fused step's column work
-    if (tpad + col_threads > 1024) col_threads = 1024 - tpad;
-    if (bw.x && col_threads < 64) return CONEF_ERR_INVALID;
-    int threads_b = (1024 - col_threads) / tpad * tpad + col_threads;
     hipError_t e;
     if (vec_ok && hp->d % 4 == 0) {
         auto ka = conef_binned_stage_kernel<NROWS, Stage, true>;
@@ -655,38 +721,66 @@ int conef_launch_binned_rows(Stage stage, const ConefPlanHeader* hp, const void*
             e = hipFuncSetAttribute((const void*)ka, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_a);
             if (e != hipSuccess) return (int)e;
         }
-        hipLaunchKernelGGL(ka, dim3(ga), dim3(threads_a), lds_a, s, stage, view, staging, hp->d, ga);
+        hipLaunchKernelGGL(ka, dim3(ga, groups), dim3(threads_a), lds_a, s, stage, view, staging, hp->d, ga, row_first);
     } else {
         auto ka = conef_binned_stage_kernel<NROWS, Stage, false>;
         if (lds_a > 48 * 1024) {
             e = hipFuncSetAttribute((const void*)ka, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_a);
             if (e != hipSuccess) return (int)e;
         }
-        hipLaunchKernelGGL(ka, dim3(ga), dim3(threads_a), lds_a, s, stage, view, staging, hp->d, ga);
+        hipLaunchKernelGGL(ka, dim3(ga, groups), dim3(threads_a), lds_a, s, stage, view, staging, hp->d, ga, row_first);
     }
-    auto kb = conef_binned_accumulate_kernel<NROWS, Stage::kFusedQuery>;
+    return (int)hipGetLastError();
+}
+
+// Pass B over the same groups; `bw` (the fused step's column-order work over the whole tensor) rides in it.
+template <int NROWS, bool FUSED_QUERY>
+int conef_launch_accumulate_rows(const ConefPlanHeader* hp, const void* plan_dev, const float* staging, const float* cs_in,
+                                 float* cs_out, float alpha, float beta, ConefBlockWork bw, int row_first, int groups,
+                                 hipStream_t s)
+{
+    ConefPlanView view = conef_plan_view(hp, plan_dev);
+    const double omb = 1. - (double)beta;
+    size_t lds_b = conef_binned_lds_b(hp, NROWS);
+    if (lds_b > 160 * 1024) return CONEF_ERR_INVALID;
+    int gb = (hp->nbins + 7) & ~7;
+    int tpad = (hp->bin_buckets + 63) & ~63;
+    int col_threads = bw.x ? 256 : 0;                   // waves of pass B that do the fused step's column work
+    if (tpad + col_threads > 1024) col_threads = 1024 - tpad;
+    if (bw.x && col_threads < 64) return CONEF_ERR_INVALID;
+    int threads_b = (1024 - col_threads) / tpad * tpad + col_threads;
+    auto kb = conef_binned_accumulate_kernel<NROWS, FUSED_QUERY>;
     if (lds_b > 48 * 1024) {
-        e = hipFuncSetAttribute((const void*)kb, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_b);
+        hipError_t e = hipFuncSetAttribute((const void*)kb, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_b);
         if (e != hipSuccess) return (int)e;
     }
     // lanes per segment: the power of two above 1.3 x the mean segment length, 8..64
     double mean_seg = (double)hp->chunk_cols * hp->bin_buckets / (double)hp->w * 1.3;
     int glog = 3;
     while (glog < 6 && (1 << glog) < mean_seg) ++glog;
-    hipLaunchKernelGGL(kb, dim3(gb), dim3(threads_b), lds_b, s, staging, view, cs_in, cs_out, hp->w, alpha, omb, gb,
-                       hp->max_bin_records, glog, col_threads, bw);
+    hipLaunchKernelGGL(kb, dim3(gb, groups), dim3(threads_b), lds_b, s, staging, view, cs_in, cs_out, hp->w, alpha, omb, gb,
+                       hp->max_bin_records, glog, col_threads, bw, row_first, hp->d);
     return (int)hipGetLastError();
 }
 
+// The two passes over all rows of the plan's tensor: whole groups of 8 rows in one launch of each
+// pass (the group is the second grid dimension), the remaining 1 to 7 rows in a launch of their
+// own.  Every pass A runs before the first pass B, because the column-order work that rides in
+// pass B rewrites the tensor pass A reads.
 template <typename Stage>
 int conef_launch_binned(Stage stage, const ConefPlanHeader* hp, const void* plan_dev, float* staging,
                         const float* cs_in, float* cs_out, float alpha, float beta, bool vec_ok, ConefBlockWork bw,
                         hipStream_t s)
 {
-    switch ((int)hp->n) {
-#define CONEF_CASE(NR)                                                                                            \
-    case NR:                                                                                                      \
-        return conef_launch_binned_rows<NR, Stage>(stage, hp, plan_dev, staging, cs_in, cs_out, alpha, beta, vec_ok, bw, s)
+    const int full = (int)(hp->n / kConefPlanMaxRows), rem = (int)(hp->n % kConefPlanMaxRows);
+    if (full > 65535) return CONEF_ERR_INVALID;
+    int rc = CONEF_OK;
+    if (full > 0) rc = conef_launch_stage_rows<kConefPlanMaxRows, Stage>(stage, hp, plan_dev, staging, vec_ok, 0, full, s);
+    if (rc != CONEF_OK) return rc;
+    const int rf = full * kConefPlanMaxRows;
+    switch (rem) {
+#define CONEF_CASE(NR) \
+    case NR: rc = conef_launch_stage_rows<NR, Stage>(stage, hp, plan_dev, staging, vec_ok, rf, 1, s); break
         CONEF_CASE(1);
         CONEF_CASE(2);
         CONEF_CASE(3);
@@ -694,16 +788,37 @@ int conef_launch_binned(Stage stage, const ConefPlanHeader* hp, const void* plan
         CONEF_CASE(5);
         CONEF_CASE(6);
         CONEF_CASE(7);
-        CONEF_CASE(8);
 #undef CONEF_CASE
     }
-    return CONEF_ERR_INVALID;
+    if (rc != CONEF_OK) return rc;
+    ConefBlockWork none = {};
+    if (full > 0)
+        rc = conef_launch_accumulate_rows<kConefPlanMaxRows, Stage::kFusedQuery>(hp, plan_dev, staging, cs_in, cs_out, alpha,
+                                                                                 beta, bw, 0, full, s);
+    if (rc != CONEF_OK) return rc;
+    const ConefBlockWork& rest = full > 0 ? none : bw;
+    switch (rem) {
+#define CONEF_CASE(NR)                                                                                              \
+    case NR:                                                                                                        \
+        rc = conef_launch_accumulate_rows<NR, Stage::kFusedQuery>(hp, plan_dev, staging, cs_in, cs_out, alpha, beta, rest, \
+                                                                  rf, 1, s);                                        \
+        break
+        CONEF_CASE(1);
+        CONEF_CASE(2);
+        CONEF_CASE(3);
+        CONEF_CASE(4);
+        CONEF_CASE(5);
+        CONEF_CASE(6);
+        CONEF_CASE(7);
+#undef CONEF_CASE
+    }
+    return rc;
 }
 
 // validates a host-side plan header against the call's shape
 inline bool conef_plan_matches(const ConefPlanHeader* hp, int64_t n, int64_t d, int32_t w, int32_t a, int32_t b)
 {
     return hp && hp->magic == kConefPlanMagic && hp->version == 1 &&
-           (hp->kind == kConefPlanBinned || hp->kind == kConefPlanRowlist) && hp->n == n && hp->d == d && hp->w == w &&
+           (hp->kind == kConefPlanBinned || hp->kind == kConefPlanRowlist || hp->kind == kConefPlanPanels) && hp->n == n && hp->d == d && hp->w == w &&
            hp->a == a && hp->b == b;
 }

@@ -22,14 +22,14 @@ int conef_launch_query_table_f16(float* x, const void* cs_half, int64_t n, int64
 
 extern "C" {
 
-// Bytes of a plan for an [n,d] tensor sketched at width w; 0 when no planned path applies (rows
-// too long for LDS and more than 8 of them), -1 on invalid arguments.  chunk_cols / bin_buckets:
-// 0 picks the kind and its defaults, a positive value asks for a binned plan with that tiling.
+// Bytes of a plan for an [n,d] tensor sketched at width w; 0 when no planned path applies (more
+// than half a million long rows), -1 on invalid arguments.  chunk_cols / bin_buckets: 0 picks the
+// kind and its defaults, a positive value asks for a binned plan with that tiling.
 int64_t conef_plan_bytes(int64_t n, int64_t d, int32_t w, int32_t chunk_cols, int32_t bin_buckets)
 {
     if (n < 1 || d < 1 || w < 1 || w > (1 << 30) || d > 0x7fffffffLL) return -1;
     ConefPlanHeader h;
-    if (!conef_plan_shape(n, d, w, chunk_cols, bin_buckets, &h)) return n > kConefPlanMaxRows ? 0 : -1;
+    if (!conef_plan_shape(n, d, w, chunk_cols, bin_buckets, &h)) return 0;
     return h.total_bytes;
 }
 
@@ -45,7 +45,9 @@ int conef_plan_build_host_seeded(void* plan_host, int64_t plan_bytes, int64_t n,
     if (plan_bytes < h.total_bytes) return CONEF_ERR_INVALID;
     if (!conef_plan_fill(plan_host, h, a, b, sa, sb)) return CONEF_ERR_INVALID;
     const ConefPlanHeader* built = (const ConefPlanHeader*)plan_host;
-    if (built->kind == kConefPlanBinned && conef_binned_lds_b(built, (int)n) > 160 * 1024) return CONEF_ERR_INVALID;
+    if (built->kind == kConefPlanBinned &&
+        conef_binned_lds_b(built, (int)(n < kConefPlanMaxRows ? n : kConefPlanMaxRows)) > 160 * 1024)
+        return CONEF_ERR_INVALID;
     return CONEF_OK;
 }
 
@@ -73,6 +75,10 @@ int conef_cs_update_planned_f32(const float* vec, const float* cs_in, float* cs_
         return conef_launch_rowlist(front, conef_rowlist_view(hp, plan_dev), cs_in, cs_out, n, d, w, beta,
                                     (hipStream_t)stream);
     }
+    if (hp->kind == kConefPlanPanels) {
+        ConefPanelVec front = {vec, aligned16(vec) && d % 4 == 0};
+        return conef_launch_panels(front, conef_panel_view(hp, plan_dev), cs_in, cs_out, n, d, w, beta, (hipStream_t)stream);
+    }
     if (!workspace) return CONEF_ERR_INVALID;
     ConefStageVec stage = {vec, d};
     ConefBlockWork none = {};
@@ -89,6 +95,11 @@ int conef_cs_update_planned_f16(const float* vec, const void* cs_in_half, void* 
     const ConefPlanHeader* hp = (const ConefPlanHeader*)plan_host;
     if (!conef_plan_matches(hp, n, d, w, a, b) || !plan_dev || !vec || !cs_in_half || !cs_out_half)
         return CONEF_ERR_INVALID;
+    if (hp->kind == kConefPlanPanels) {
+        ConefPanelVec front = {vec, aligned16(vec) && d % 4 == 0};
+        return conef_launch_panels(front, conef_panel_view(hp, plan_dev), (const __half*)cs_in_half, (__half*)cs_out_half, n,
+                                   d, w, beta, (hipStream_t)stream);
+    }
     if (hp->kind != kConefPlanRowlist) return CONEF_ERR_INVALID;
     ConefListVec front = {vec, aligned16(vec) && d % 4 == 0};
     return conef_launch_rowlist(front, conef_rowlist_view(hp, plan_dev), (const __half*)cs_in_half,
@@ -121,8 +132,8 @@ int conef_cs_query_planned_f16(float* x, const void* cs_half, const void* plan_h
     return conef_launch_query_table_f16(x, cs_half, n, d, w, alpha, a, b, pk, (hipStream_t)stream);
 }
 
-// 0 = binned (needs the workspace, fused step needs cs_out != cs_in), 1 = row lists (no
-// workspace, in place allowed), -1 = not a plan.
+// 0 = binned (needs the workspace, fused step needs cs_out != cs_in), 1 = row lists, 2 = row lists in
+// column panels (both: no workspace, in place allowed), -1 = not a plan.
 int conef_plan_kind(const void* plan_host)
 {
     const ConefPlanHeader* h = (const ConefPlanHeader*)plan_host;
@@ -145,6 +156,10 @@ int conef_randblock_conef_step_planned_f32(float* x, const float* cs_in, float* 
         ConefListRandBlock front = {x, payload, blk, alpha};
         return conef_launch_rowlist(front, conef_rowlist_view(hp, plan_dev), cs_in, cs_out, n, m, w, beta,
                                     (hipStream_t)stream);
+    }
+    if (hp->kind == kConefPlanPanels) {
+        ConefPanelRandBlock front = {x, payload, blk, alpha, aligned16(x) && m % 4 == 0};
+        return conef_launch_panels(front, conef_panel_view(hp, plan_dev), cs_in, cs_out, n, m, w, beta, (hipStream_t)stream);
     }
     if (!workspace) return CONEF_ERR_INVALID;
     if (cs_in == cs_out) return CONEF_ERR_INVALID;   // the block is finished while buckets are being rewritten

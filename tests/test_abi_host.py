@@ -199,10 +199,10 @@ def test_plans_are_shared_and_released():
     assert p4.kind == SketchPlan.BINNED and p4.workspace_bytes >= 4 * 5 * 130_000
     held = _pools.held_bytes()
     assert held["plans"] == p1.device.numel() + p3.device.numel() + p4.device.numel() and held["staging"] == 0
-    with pytest.raises(ValueError):
-        SketchPlan.shared(9, 1_300_000, 130_000, 994443, 609478, cpu)      # long rows and more than 8 of them
+    with pytest.raises(ValueError):       # long rows in more groups of 8 than a grid dimension holds: no plan
+        SketchPlan.shared(8 * 65536, 100_000, 100_000, 994443, 609478, cpu)
     with pytest.raises(ValueError):                                       # ... remembered, not rebuilt
-        SketchPlan.shared(9, 1_300_000, 130_000, 994443, 609478, cpu)
+        SketchPlan.shared(8 * 65536, 100_000, 100_000, 994443, 609478, cpu)
     conef_amd.release()
     assert _pools.held_bytes()["plans"] == 0
     assert p1.header()["w"] == 65                                        # still valid for its holder

@@ -251,10 +251,14 @@ def test_rejects_host_tensors():
 
 # ---- long rows: the planned (atomic-free) path is deterministic and follows the oracle's order ----
 
-PLANNED_SHAPES = [  # (n, d, sketch_size, kind): 0 = binned long rows, 1 = row lists
+PLANNED_SHAPES = [  # (n, d, sketch_size, kind): 0 = binned long rows, 1 = row lists, 2 = row lists in column panels
     (5, 40_003, 0.1, 0), (5, 100_000, 0.1, 0), (2, 65_537, 0.5, 0), (1, 300_001, 0.05, 0), (8, 30_000, 0.9, 0), (5, 24_577, 0.004, 0),
     (8, 20_000, 0.9, 0), (3, 8191, 1.0, 1), (8, 20_000, 0.05, 1), (1, 1, 0.5, 1), (3, 17, 0.3, 1), (64, 576, 0.2, 1), (40, 5760, 0.2, 1),
-    (2100, 650, 0.1, 1), (4099, 1024, 0.1, 1), (7, 24_576, 0.05, 1), (33, 1023, 2.0, 1), (20_000, 66, 0.1, 1)]
+    (2100, 650, 0.1, 1), (4099, 1024, 0.1, 1), (7, 24_576, 0.05, 1), (33, 1023, 2.0, 1), (20_000, 66, 0.1, 1),
+    # long rows and more than 8 of them (the reference kernel takes any N and D, CountSketch.py:27-67,143-158):
+    # the binned passes over groups of 8 rows (a last group of 1..7), and the panels for tall matrices
+    (16, 50_000, 0.1, 0), (9, 100_000, 0.1, 0), (11, 40_003, 0.1, 0), (64, 200_000, 0.1, 0), (23, 30_002, 0.9, 0),
+    (600, 25_088, 0.1, 2), (257, 30_001, 0.4, 2), (1030, 40_000, 0.01, 2), (513, 24_578, 0.5, 2)]
 
 
 @pytest.mark.parametrize("n,d,ss,kind", PLANNED_SHAPES)
@@ -348,11 +352,66 @@ def test_atomic_fallback_still_matches(oracle, monkeypatch):
     cs.update(dev(v), 0.9)
     o.update(v, 0.9)
     assert_close(cs.cs, o.cs, what="atomic path")
-    big = DenseCS(12, 100_000, 0.1)          # more than 8 rows: no plan, atomics
-    monkeypatch.delenv("CONEF_PLAN")
+    big = DenseCS(12, 100_000, 0.1)          # the same kernel at 12 rows, where a plan would have been found
     assert big.plan() is None
     ob = oracle.DenseCS(12, 100_000, 0.1)
     v = (np.random.RandomState(3).randn(12, 100_000) * 1e-3).astype(np.float32)
     big.update(dev(v), 0.9)
     ob.update(v, 0.9)
     assert_close(big.cs, ob.cs, what="atomic path, 12 rows")
+
+
+def test_a_shape_without_a_plan_says_so_once(monkeypatch, caplog):
+    """No shape falls back to float atomics silently: a sketch that finds no plan logs a warning,
+    once per shape."""
+    import logging
+    from conef_amd.compressors import CountSketch
+    monkeypatch.setattr(CountSketch.SketchPlan, "applicable", staticmethod(lambda *a, **k: False))
+    CountSketch._WARNED.discard((6, 3000, 600))
+    with caplog.at_level(logging.WARNING):
+        for _ in range(3):
+            cs = CountSketch.DenseCS(6, 3000, 0.2)
+            assert cs.plan() is None
+    hits = [r for r in caplog.records if "float atomics" in r.getMessage()]
+    assert len(hits) == 1 and "[6, 3000]" in hits[0].getMessage()
+
+
+def test_full_vgg_fc_layer_on_panels_bit_exact(oracle):
+    """[4096, 25088] (the first fully connected layer of VGG-16): a row is too long for whole row
+    lists, the matrix tall enough for the panels."""
+    from conef_amd.compressors.CountSketch import DenseCS
+    n, d, ss = 4096, 25_088, 0.1
+    cs = DenseCS(n, d, ss)
+    assert cs.plan() is not None and cs.plan().kind == 2
+    o = oracle.DenseCS(n, d, ss)
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    for step in range(2):
+        v = torch.randn(n, d, generator=gen, device="cuda") * 1e-3
+        cs.update(v, 0.9)
+        o.update(to_np(v), 0.9)
+        np.testing.assert_array_equal(to_np(cs.cs), o.cs)
+
+
+@pytest.mark.parametrize("n,d,ss,kind", [(600, 25_088, 0.1, 2), (257, 30_001, 0.4, 2), (16, 50_000, 0.1, 0),
+                                         (9, 100_000, 0.1, 0), (19, 40_003, 0.3, 0)])
+def test_randblock_step_on_panels_and_row_groups_bit_exact(oracle, n, d, ss, kind):
+    """The fused RandomBlock + sketch step (RandomBlock_hook.py:190,216-243,272-280) on the plans for
+    long rows of a matrix with more than 8 of them: block, zeros, payload and the new sketch against
+    the oracle's fused step, bit for bit, with a block that wraps around the end and one that does not."""
+    from conef_amd.compressors.CountSketch import DenseCS
+    rng = np.random.RandomState(n + d)
+    cs = DenseCS(n, d, ss)
+    assert cs.plan() is not None and cs.plan().kind == kind
+    ocs = np.zeros((n, cs.range), np.float32)
+    numel = n * d
+    block = max(1, int(0.1 * numel))
+    for step, start in enumerate([numel - block // 3, 12_345, 7 * d + 3]):
+        x = (rng.randn(n, d) * 1e-3).astype(np.float32)
+        xd = dev(x)
+        payload = torch.empty(block, device="cuda")
+        cs.randblock_step(xd, payload, start, block, 1 - 0.9, 0.9)
+        opay = np.empty(block, np.float32)
+        oracle.randblock_conef_step(x, ocs, opay, start, block, 1 - 0.9, 0.9)
+        np.testing.assert_array_equal(to_np(xd), x, err_msg="decompressed gradient, step %d" % step)
+        np.testing.assert_array_equal(to_np(payload), opay, err_msg="payload, step %d" % step)
+        np.testing.assert_array_equal(to_np(cs.cs), ocs, err_msg="sketch, step %d" % step)

@@ -68,7 +68,8 @@ def replay(h, vec, cs, beta, oracle):
 
 
 @pytest.mark.parametrize("n,d,w,chunk,tbin", [(5, 9000, 900, 1024, 64), (1, 5000, 5000, 2048, 128),
-                                              (8, 3001, 77, 1024, 64), (3, 30011, 4000, 0, 0)])
+                                              (8, 3001, 77, 1024, 64), (3, 30011, 4000, 0, 0),
+                                              (11, 9000, 900, 1024, 64), (9, 30011, 4000, 0, 0)])
 def test_plan_replay_matches_oracle_bit_for_bit(oracle, n, d, w, chunk, tbin):
     rng = np.random.RandomState(d)
     h = build_plan(n, d, w, chunk, tbin)
@@ -141,10 +142,70 @@ def test_rowlist_plan_replay_matches_oracle_bit_for_bit(oracle, n, d, w):
     np.testing.assert_array_equal(got, want)
 
 
+def build_panels(n, d, w):
+    from conef_amd import _lib
+    lib = _lib.load()
+    nb = lib.conef_plan_bytes(n, d, w, 0, 0)
+    assert nb > 0
+    buf = np.zeros(nb, np.uint8)
+    assert lib.conef_plan_build_host(buf.ctypes.data, nb, n, d, w, A, B, 0, 0) == 0
+    assert lib.conef_plan_kind(buf.ctypes.data) == 2
+    assert lib.conef_plan_workspace_bytes(buf.ctypes.data) == 0
+    i32, i64 = buf[:128].view(np.int32), buf[:136].view(np.int64)
+    pc = int(i32[9])
+    assert pc % 8 == 0 and int(i32[10]) == (d + pc - 1) // pc
+    ent = buf[int(i64[10]):int(i64[10]) + 2 * d].view(np.uint16)
+    entb = buf[int(i64[7]):int(i64[7]) + 2 * d].view(np.uint16)
+    pk = buf[int(i64[11]):int(i64[11]) + 4 * d].view(np.uint32)
+    return pc, ent, entb, pk
+
+
+@pytest.mark.parametrize("n,d,w", [(600, 25_088, 2508), (257, 30_001, 12_000), (1030, 40_000, 400)])
+def test_panel_plan_replay_matches_oracle_bit_for_bit(oracle, n, d, w):
+    """The kernel's walk, panel after panel, from the plan's tables alone: the thread that meets the
+    first entry of a bucket's group adds the group's terms in the listed order."""
+    pc, ent, entb, pk = build_panels(n, d, w)
+    bucket, sign = oracle.hash_table(d, w)
+    np.testing.assert_array_equal(pk & 0x7fffffff, bucket.astype(np.uint32))
+    np.testing.assert_array_equal(pk >> 31, (sign > 0).astype(np.uint32))
+    rows = 3                                                    # the tables are the same for every row
+    rng = np.random.RandomState(d)
+    vec = rng.randn(rows, d).astype(np.float32)
+    cs0 = rng.randn(rows, w).astype(np.float32)
+    omb = 1.0 - float(np.float32(0.9))
+    got = cs0.copy()
+    seen = np.zeros(d, bool)
+    for c0 in range(0, d, pc):
+        cols = min(pc, d - c0)
+        e_ent, e_b = ent[c0:c0 + cols].astype(np.int64), entb[c0:c0 + cols].astype(np.int64)
+        col = c0 + (e_ent & 0x7fff)
+        assert (col < c0 + cols).all() and not seen[col].any()
+        seen[col] = True
+        np.testing.assert_array_equal(e_b, bucket[col])                       # every entry names its column's bucket
+        np.testing.assert_array_equal(e_ent >> 15, (sign[col] > 0).astype(np.int64))
+        assert (np.diff(e_b) >= 0).all()                                      # grouped by bucket ...
+        same = np.diff(e_b) == 0
+        assert (np.diff(col)[same] > 0).all()                                 # ... ascending columns inside a group
+        for e in range(cols):
+            s = 1.0 if e_ent[e] >> 15 else -1.0
+            j = e_b[e]
+            term = (s * vec[:, col[e]].astype(np.float64) - omb * cs0[:, j].astype(np.float64)).astype(np.float32)
+            got[:, j] = got[:, j] + term
+    assert seen.all()
+    want = cs0.copy()
+    oracle.cs_update(vec, want, 0.9)
+    np.testing.assert_array_equal(got, want)
+
+
 @pytest.mark.parametrize("n,d,w,kind", [(5, 1_300_000, 130_000, 0), (640, 5760, 1152, 1), (33278, 650, 65, 1),
                                         (7, 24_576, 1228, 1), (8, 20_000, 1000, 1), (8, 20_000, 18_000, 0),
                                         (8, 30_000, 27_000, 0), (1, 1, 1, 1), (3, 8191, 8191, 1), (20_000, 66, 6, 1),
-                                        (5, 24_577, 100, 0), (33, 1023, 2046, 1)])
+                                        (5, 24_577, 100, 0), (33, 1023, 2046, 1),
+                                        # rows too long for whole row lists: tall matrices take the panels, matrices
+                                        # with few rows (or a sketch too wide for LDS) the binned passes in row groups
+                                        (4096, 25_088, 2508, 2), (4096, 25_088, 12_544, 2), (16, 50_000, 5000, 0),
+                                        (9, 100_000, 10_000, 0), (64, 200_000, 20_000, 0), (9, 1_300_000, 130_000, 0),
+                                        (2000, 30_000, 30_000, 0), (1024, 24_577, 2457, 2)])
 def test_which_kind_of_plan_a_shape_gets(n, d, w, kind):
     from conef_amd import _lib
     lib = _lib.load()
@@ -158,9 +219,10 @@ def test_which_kind_of_plan_a_shape_gets(n, d, w, kind):
 def test_plan_argument_checks():
     from conef_amd import _lib
     lib = _lib.load()
-    assert lib.conef_plan_bytes(9, 100_000, 100, 0, 0) == 0       # long rows and more than 8 of them: no plan
+    assert lib.conef_plan_bytes(9, 100_000, 100, 0, 0) > 0        # long rows and more than 8 of them: binned, in row groups
     assert lib.conef_plan_bytes(9, 1000, 100, 0, 0) > 0           # short rows: row lists, any number of rows
-    assert lib.conef_plan_bytes(9, 1000, 100, 1024, 64) == 0      # a binned plan was asked for
+    assert lib.conef_plan_bytes(9, 1000, 100, 1024, 64) > 0       # a binned plan was asked for
+    assert lib.conef_plan_bytes(8 * 65536, 100_000, 100, 1024, 64) == 0   # more row groups than a grid dimension holds
     assert lib.conef_plan_bytes(0, 1000, 100, 0, 0) == -1
     buf = np.zeros(64, np.uint8)
     assert lib.conef_plan_build_host(buf.ctypes.data, 64, 5, 1000, 100, A, B, 0, 0) == -1   # buffer too small
