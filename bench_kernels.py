@@ -90,7 +90,9 @@ def main():
 
     sketch_shapes = [("cfg2 flat bucket", 5, 1_300_000, 0.1), ("cfg3 WRN conv", 640, 5760, 0.2),
                      ("cfg5 BERT ffn", 1024, 4096, 0.1), ("cfg5 BERT attn", 1024, 1024, 0.1),
-                     ("cfg4 LSTM embedding", 33278, 650, 0.1), ("cfg1 ResNet-20 conv", 64, 576, 0.5)]
+                     ("cfg4 LSTM embedding", 33278, 650, 0.1), ("cfg1 ResNet-20 conv", 64, 576, 0.5),
+                     # rows too long for whole row lists and more than 8 of them: panels / binned row groups
+                     ("VGG-16 fc6", 4096, 25088, 0.1), ("64 long rows", 64, 200_000, 0.1)]
 
     # ------------------------------------------------------------------ count sketch
     for tag, n, d, ss in sketch_shapes:
@@ -112,7 +114,7 @@ def main():
                    lambda s, n=n, d=d, w=w, plan=plan, staging=staging: ck(lib.conef_cs_query_planned_f32(
                        s[0].data_ptr(), s[1].data_ptr(), plan.host_ptr, plan.device.data_ptr(), staging, n, d, w, 0.1, A, B,
                        stream), "query planned"))
-            timeit("cs_update_planned_f32 (%s) %s [%d,%d] W=%d" % ("row lists" if plan.in_place else "binned", tag, n, d, w),
+            timeit("cs_update_planned_f32 (%s) %s [%d,%d] W=%d" % (("binned", "row lists", "row lists in panels")[plan.kind], tag, n, d, w),
                    4 * n * d + 8 * n * w, make,
                    lambda s, n=n, d=d, w=w, plan=plan: ck(lib.conef_cs_update_planned_f32(
                        s[0].data_ptr(), s[1].data_ptr(), s[1].data_ptr(), plan.host_ptr, plan.device.data_ptr(),

@@ -35,7 +35,7 @@ constexpr int kConefPlanMaxRows = 8;
 // Three kinds of plan share the header.  Row lists (conef_rowlist.h): a row fits LDS, any number of
 // rows, tables csr / ent (column | sign << 15) / pk only, no staging buffer.  Row lists in column
 // panels (conef_panels.h): rows too long for that on a matrix with rows enough to fill the machine,
-// tables ent / entb / pk, no staging buffer.  Binned (this file): a few long rows, in groups of up to 8.
+// tables epos / entg / colb / pk, no staging buffer.  Binned (this file): a few long rows, in groups of up to 8.
 constexpr int64_t kConefPlanBinned = 0;
 constexpr int64_t kConefPlanRowlist = 1;
 constexpr int64_t kConefPlanPanels = 2;
@@ -54,7 +54,7 @@ struct ConefPlanHeader {
     int32_t nbins;
     int32_t max_bin_records;   // largest number of columns that map into one bin
     int64_t off_pos;           // uint16[d]: record position of column i inside its chunk image
-                               // (panels: the bucket of every list entry, `entb`)
+                               // (panels: `entg`; their `epos` sits at off_ent, their `colb` at off_csr)
     int64_t off_seg;           // uint32[nbins][nchunks+1]: (start inside chunk image) | (offset inside bin image << 16);
                                // entry [nchunks] holds the bin's record count in the high half
     int64_t off_csr;           // uint32[w+1]: first entry of bucket j
@@ -109,9 +109,11 @@ inline bool conef_plan_shape(int64_t n, int64_t d, int32_t w, int32_t hint_chunk
         h->chunk_cols = pl.pc;
         h->nchunks = (int32_t)((d + pl.pc - 1) / pl.pc);
         int64_t off = conef_align256(sizeof(ConefPlanHeader));
-        h->off_ent = off;
+        h->off_ent = off;                       // epos: uint16[d] by column, entry of its panel | sign << 15
         off += conef_align256(2 * d + 16);
-        h->off_pos = off;
+        h->off_pos = off;                       // entg: uint32[d] by panel and entry, bucket | group length << 16
+        off += conef_align256(4 * d + 16);
+        h->off_csr = off;                       // colb: uint16[d] by column, the column's bucket
         off += conef_align256(2 * d + 16);
         h->off_pk = off;
         off += conef_align256(4 * d + 16);
@@ -205,8 +207,9 @@ inline bool conef_plan_fill(void* buf, const ConefPlanHeader& shape, int32_t a, 
     if (h.kind == kConefPlanPanels) {
         char* pbase = (char*)buf;
         memset(pbase, 0, (size_t)h.total_bytes);
-        uint16_t* pent = (uint16_t*)(pbase + h.off_ent);
-        uint16_t* pentb = (uint16_t*)(pbase + h.off_pos);
+        uint16_t* pepos = (uint16_t*)(pbase + h.off_ent);
+        uint32_t* pentg = (uint32_t*)(pbase + h.off_pos);
+        uint16_t* pcolb = (uint16_t*)(pbase + h.off_csr);
         uint32_t* ppk = (uint32_t*)(pbase + h.off_pk);
         ConefMod pmod = conef_make_mod(h.w);
         for (int64_t i = 0; i < d; ++i) ppk[i] = conef_bucket_sign((int32_t)i, pmod, a, b, sa, sb);
@@ -220,8 +223,16 @@ inline bool conef_plan_fill(void* buf, const ConefPlanHeader& shape, int32_t a, 
             for (int64_t i = c0; i < c1; ++i) {        // ascending columns inside every bucket
                 const uint32_t j = ppk[i] & 0x7fffffffu;
                 const uint32_t k = first[j]++;
-                pent[c0 + k] = (uint16_t)((uint32_t)(i - c0) | ((ppk[i] >> 31) << 15));
-                pentb[c0 + k] = (uint16_t)j;
+                pepos[i] = (uint16_t)(k | ((ppk[i] >> 31) << 15));
+                pcolb[i] = (uint16_t)j;
+                pentg[c0 + k] = j;
+            }
+            for (int64_t k = c1 - c0 - 1, run = 0; k >= 0; --k) {        // the first entry of a group carries its length
+                ++run;
+                if (k == 0 || pentg[c0 + k - 1] != pentg[c0 + k]) {
+                    pentg[c0 + k] |= (uint32_t)run << 16;
+                    run = 0;
+                }
             }
         }
         memcpy(pbase, &h, sizeof(h));
@@ -310,8 +321,8 @@ inline ConefRowlistView conef_rowlist_view(const ConefPlanHeader* host, const vo
 inline ConefPanelView conef_panel_view(const ConefPlanHeader* host, const void* dev)
 {
     const char* b = (const char*)dev;
-    ConefPanelView v = {(const uint16_t*)(b + host->off_ent), (const uint16_t*)(b + host->off_pos),
-                        (const uint32_t*)(b + host->off_pk), host->chunk_cols};
+    ConefPanelView v = {(const uint32_t*)(b + host->off_pos), (const uint16_t*)(b + host->off_ent),
+                        (const uint16_t*)(b + host->off_csr), host->chunk_cols};
     return v;
 }
 

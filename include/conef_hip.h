@@ -109,14 +109,18 @@ int conef_cs3_value_f32(const float* vec, const float* in0, const float* in1, co
 /* The hash is a fixed function of (column, w, a, b), so where every column of an [n,d] tensor
  * goes is known before the first step.  A plan built once per sketch turns the update into
  * streaming passes without atomics that add every bucket's terms in ascending column order -
- * deterministic, and bit for bit the order of the reference's serial definition.  Two kinds:
+ * deterministic, and bit for bit the order of the reference's serial definition.  Three kinds
+ * cover every shape the reference's kernel takes (any N, D: CountSketch.py:27-67,143-158):
  *   row lists  a row fits LDS (d <= 24576), any number of rows: one pass, per-bucket column
  *              lists, no workspace, cs_out may be cs_in;
- *   binned     rows too long for LDS, n <= 8 (a flat bucket viewed as a few long rows): two
- *              passes through a staging workspace of n*d floats.
+ *   panels     longer rows of a matrix tall enough to fill the machine with row tiles (and
+ *              w <= 65535): the same lists cut into column panels, the tile's cells resident in
+ *              LDS while the panels go by; one pass, no workspace, cs_out may be cs_in;
+ *   binned     long rows otherwise (a flat bucket viewed as a few long rows): two passes through
+ *              a staging workspace of n*d floats, over groups of 8 rows.
  * No counterpart in the reference (its update is one atomicAdd per element, CountSketch.py:63). */
 
-/* Bytes of a plan; 0 when neither kind applies (long rows and n > 8), -1 on invalid arguments.
+/* Bytes of a plan; 0 when no kind applies (more than 8 * 65535 long rows), -1 on invalid arguments.
  * chunk_cols / bin_buckets: 0 picks kind and tiling, a positive value asks for a binned plan with
  * that tiling (columns per staging workgroup, buckets per accumulating workgroup). */
 int64_t conef_plan_bytes(int64_t n, int64_t d, int32_t w, int32_t chunk_cols, int32_t bin_buckets);
@@ -130,14 +134,14 @@ int conef_plan_build_host(void* plan_host, int64_t plan_bytes, int64_t n, int64_
 int conef_plan_build_host_seeded(void* plan_host, int64_t plan_bytes, int64_t n, int64_t d, int32_t w, int32_t a,
                                  int32_t b, int32_t sa, int32_t sb, int32_t chunk_cols, int32_t bin_buckets);
 /* Bytes of device staging memory the planned entry points need (binned: n*d floats, rounded up;
- * row lists: 0, the workspace argument may then be null). */
+ * row lists and panels: 0, the workspace argument may then be null). */
 int64_t conef_plan_workspace_bytes(const void* plan_host);
-/* 0 = binned, 1 = row lists, -1 = not a plan. */
+/* 0 = binned, 1 = row lists, 2 = row lists in column panels, -1 = not a plan. */
 int conef_plan_kind(const void* plan_host);
 
 /* conef_cs_update_f32 on a plan.  cs_out may be the same buffer as cs_in.  Calls that share a
  * workspace must be ordered on one stream.  The f16 form (fp16-storage sketch, replaces
- * halfCountSketch.py:151-172) takes row-list plans only. */
+ * halfCountSketch.py:151-172) takes row-list plans, whole or in panels. */
 int conef_cs_update_planned_f16(const float* vec, const void* cs_in_half, void* cs_out_half, const void* plan_host,
                                 const void* plan_dev, int64_t n, int64_t d, int32_t w, float beta, int32_t a,
                                 int32_t b, void* stream);

@@ -154,44 +154,55 @@ def build_panels(n, d, w):
     i32, i64 = buf[:128].view(np.int32), buf[:136].view(np.int64)
     pc = int(i32[9])
     assert pc % 8 == 0 and int(i32[10]) == (d + pc - 1) // pc
-    ent = buf[int(i64[10]):int(i64[10]) + 2 * d].view(np.uint16)
-    entb = buf[int(i64[7]):int(i64[7]) + 2 * d].view(np.uint16)
+    epos = buf[int(i64[10]):int(i64[10]) + 2 * d].view(np.uint16)
+    entg = buf[int(i64[7]):int(i64[7]) + 4 * d].view(np.uint32)
+    colb = buf[int(i64[9]):int(i64[9]) + 2 * d].view(np.uint16)
     pk = buf[int(i64[11]):int(i64[11]) + 4 * d].view(np.uint32)
-    return pc, ent, entb, pk
+    return pc, epos, entg, colb, pk
 
 
 @pytest.mark.parametrize("n,d,w", [(600, 25_088, 2508), (257, 30_001, 12_000), (1030, 40_000, 400)])
 def test_panel_plan_replay_matches_oracle_bit_for_bit(oracle, n, d, w):
-    """The kernel's walk, panel after panel, from the plan's tables alone: the thread that meets the
-    first entry of a bucket's group adds the group's terms in the listed order."""
-    pc, ent, entb, pk = build_panels(n, d, w)
+    """The kernel's two steps, panel after panel, from the plan's tables alone: every column's term
+    is parked at the entry the plan names for it, then the first entry of a bucket's group adds the
+    group's terms in the order they sit in."""
+    pc, epos, entg, colb, pk = build_panels(n, d, w)
+    assert pc <= 4096
     bucket, sign = oracle.hash_table(d, w)
     np.testing.assert_array_equal(pk & 0x7fffffff, bucket.astype(np.uint32))
     np.testing.assert_array_equal(pk >> 31, (sign > 0).astype(np.uint32))
+    np.testing.assert_array_equal(colb, bucket.astype(np.uint16))
+    np.testing.assert_array_equal(epos >> 15, (sign > 0).astype(np.uint16))
     rows = 3                                                    # the tables are the same for every row
     rng = np.random.RandomState(d)
     vec = rng.randn(rows, d).astype(np.float32)
     cs0 = rng.randn(rows, w).astype(np.float32)
     omb = 1.0 - float(np.float32(0.9))
     got = cs0.copy()
-    seen = np.zeros(d, bool)
     for c0 in range(0, d, pc):
         cols = min(pc, d - c0)
-        e_ent, e_b = ent[c0:c0 + cols].astype(np.int64), entb[c0:c0 + cols].astype(np.int64)
-        col = c0 + (e_ent & 0x7fff)
-        assert (col < c0 + cols).all() and not seen[col].any()
-        seen[col] = True
-        np.testing.assert_array_equal(e_b, bucket[col])                       # every entry names its column's bucket
-        np.testing.assert_array_equal(e_ent >> 15, (sign[col] > 0).astype(np.int64))
+        e = (epos[c0:c0 + cols] & 0x7fff).astype(np.int64)
+        assert sorted(e.tolist()) == list(range(cols))                         # a permutation of the panel
+        e_b = (entg[c0:c0 + cols] & 0xffff).astype(np.int64)
+        np.testing.assert_array_equal(e_b[e], colb[c0:c0 + cols])              # every entry names its column's bucket
         assert (np.diff(e_b) >= 0).all()                                      # grouped by bucket ...
-        same = np.diff(e_b) == 0
-        assert (np.diff(col)[same] > 0).all()                                 # ... ascending columns inside a group
-        for e in range(cols):
-            s = 1.0 if e_ent[e] >> 15 else -1.0
-            j = e_b[e]
-            term = (s * vec[:, col[e]].astype(np.float64) - omb * cs0[:, j].astype(np.float64)).astype(np.float32)
-            got[:, j] = got[:, j] + term
-    assert seen.all()
+        lens = (entg[c0:c0 + cols] >> 16).astype(np.int64)                    # ... the first of a group carries its length
+        first = np.concatenate([[True], np.diff(e_b) != 0])
+        assert (lens[~first] == 0).all()
+        np.testing.assert_array_equal(lens[first], np.diff(np.concatenate([np.flatnonzero(first), [cols]])))
+        col_of = np.empty(cols, np.int64)
+        col_of[e] = np.arange(cols)
+        assert (np.diff(col_of)[np.diff(e_b) == 0] > 0).all()                 # ... ascending columns inside a group
+        # park
+        s = np.where(epos[c0:c0 + cols] >> 15, 1.0, -1.0)
+        terms = np.empty((cols, rows), np.float32)
+        v = vec[:, c0:c0 + cols].astype(np.float64)
+        decay = omb * cs0[:, colb[c0:c0 + cols].astype(np.int64)].astype(np.float64)
+        terms[e, :] = (s[None, :] * v - decay).astype(np.float32).T
+        # walk
+        for k in np.flatnonzero(lens):
+            for kk in range(k, k + lens[k]):
+                got[:, e_b[k]] = got[:, e_b[k]] + terms[kk, :]
     want = cs0.copy()
     oracle.cs_update(vec, want, 0.9)
     np.testing.assert_array_equal(got, want)
