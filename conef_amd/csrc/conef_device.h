@@ -4,8 +4,33 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 #define CONEF_OK 0
 #define CONEF_ERR_INVALID (-1)
+
+// ------------------------------------------------------------- launch helper ----
+// A kernel that wants more than 48 KB of dynamic LDS has to be allowed to, per device.  The runtime
+// call costs the host a few microseconds, a hook issues a handful of such launches per bucket: the
+// largest size granted per (kernel, device) is remembered and the runtime is only asked again for
+// a larger one.  (The one piece of bookkeeping the library keeps between calls; guarded by a mutex.)
+inline hipError_t conef_allow_lds(const void* kernel, size_t bytes)
+{
+    if (bytes <= 48 * 1024) return hipSuccess;
+    static std::mutex lock;
+    static std::map<std::pair<const void*, int>, size_t> granted;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> hold(lock);
+    size_t& have = granted[std::make_pair(kernel, dev)];
+    if (have >= bytes) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess) have = bytes;
+    return e;
+}
 
 // ------------------------------------------------------------------ hash ----
 // Integer mixer of the count sketch (reference: communication/compressors/CountSketch.py:7-18).

@@ -728,17 +728,13 @@ int conef_launch_stage_rows(Stage stage, const ConefPlanHeader* hp, const void* 
     hipError_t e;
     if (vec_ok && hp->d % 4 == 0) {
         auto ka = conef_binned_stage_kernel<NROWS, Stage, true>;
-        if (lds_a > 48 * 1024) {
-            e = hipFuncSetAttribute((const void*)ka, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_a);
-            if (e != hipSuccess) return (int)e;
-        }
+        e = conef_allow_lds((const void*)ka, lds_a);
+        if (e != hipSuccess) return (int)e;
         hipLaunchKernelGGL(ka, dim3(ga, groups), dim3(threads_a), lds_a, s, stage, view, staging, hp->d, ga, row_first);
     } else {
         auto ka = conef_binned_stage_kernel<NROWS, Stage, false>;
-        if (lds_a > 48 * 1024) {
-            e = hipFuncSetAttribute((const void*)ka, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_a);
-            if (e != hipSuccess) return (int)e;
-        }
+        e = conef_allow_lds((const void*)ka, lds_a);
+        if (e != hipSuccess) return (int)e;
         hipLaunchKernelGGL(ka, dim3(ga, groups), dim3(threads_a), lds_a, s, stage, view, staging, hp->d, ga, row_first);
     }
     return (int)hipGetLastError();
@@ -761,8 +757,8 @@ int conef_launch_accumulate_rows(const ConefPlanHeader* hp, const void* plan_dev
     if (bw.x && col_threads < 64) return CONEF_ERR_INVALID;
     int threads_b = (1024 - col_threads) / tpad * tpad + col_threads;
     auto kb = conef_binned_accumulate_kernel<NROWS, FUSED_QUERY>;
-    if (lds_b > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)kb, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_b);
+    {
+        hipError_t e = conef_allow_lds((const void*)kb, lds_b);
         if (e != hipSuccess) return (int)e;
     }
     // lanes per segment: the power of two above 1.3 x the mean segment length, 8..64

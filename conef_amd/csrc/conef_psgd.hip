@@ -1804,10 +1804,7 @@ int launch_mq(float* x, const float* err, const float* cs, const uint32_t* pktab
             }
             float* out = g.splits > 1 ? (float*)workspace : p;
             auto k = psgd_mfma_mq_kernel<MODE>;
-            if (lds > 48 * 1024) {
-                hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-                if (e != hipSuccess) return (int)e;
-            }
+            if (hipError_t e = conef_allow_lds((const void*)k, lds); e != hipSuccess) return (int)e;
             hipLaunchKernelGGL(k, dim3((unsigned)g.row_tiles, (unsigned)g.splits), dim3(kMfmaThreads), lds, s, x, err, cs,
                                pktab, q, out, n, (int)m, r, g.cols_per_split, mod, alpha, hs);
             if (g.splits > 1) {
@@ -2367,10 +2364,7 @@ int conef_gram_schmidt_f32(float* a, int64_t rows, int32_t r, float eps, void* w
 #define CONEF_GS(RP)                                                                                              \
     do {                                                                                                          \
         auto k = gram_schmidt_lds_kernel<RP>;                                                                     \
-        if (lds > 48 * 1024) {                                                                                    \
-            hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
-            if (e != hipSuccess) return (int)e;                                                                   \
-        }                                                                                                         \
+        if (hipError_t e = conef_allow_lds((const void*)k, lds); e != hipSuccess) return (int)e; \
         hipLaunchKernelGGL(k, dim3(1), dim3(threads), lds, s, a, (int)rows, r, eps);                              \
     } while (0)
         CONEF_RANK_SWITCH(r, CONEF_GS)
@@ -3258,17 +3252,11 @@ int pqt_sketch_group(const ConefPsgdItem* items, const std::vector<int>& members
         if (shape.lds > lds) lds = shape.lds;
     }
     auto kern = psgd_residual_rowlist_batch_kernel<RP, FAST>;
-    if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-    }
+    if (hipError_t e = conef_allow_lds((const void*)kern, lds); e != hipSuccess) return (int)e;
     const double omb = 1. - (double)beta;
     if (ahead && ahead->count > 0 && table.size() <= (size_t)kPsgdBatchMax) {
         auto fused = psgd_residual_rowlist_gs_batch_kernel<RP, FAST>;
-        if (lds > 48 * 1024) {
-            hipError_t e = hipFuncSetAttribute((const void*)fused, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return (int)e;
-        }
+        if (hipError_t e = conef_allow_lds((const void*)fused, lds); e != hipSuccess) return (int)e;
         const GsAhead g = *ahead;
         return run_batches(table, blocks, [&](const PsgdBatch<RowlistResidualItem<RP, FAST>>& bt, int grid) {
             hipLaunchKernelGGL(fused, dim3((unsigned)(grid + g.count)), dim3(kConefRowlistThreads), lds, s, bt, omb, g);
@@ -3498,11 +3486,7 @@ int conef_psgd_sketch_update_batch_f32(const ConefPsgdItem* items, int32_t count
         blocks.push_back((int)shape.tiles);
         if (shape.lds > lds) lds = shape.lds;
     }
-    if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)psgd_rowlist_vec_batch_kernel,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-    }
+    if (hipError_t e = conef_allow_lds((const void*)psgd_rowlist_vec_batch_kernel, lds); e != hipSuccess) return (int)e;
     const double omb = 1. - (double)beta;
     hipStream_t s = (hipStream_t)stream;
     return run_batches(table, blocks, [&](const PsgdBatch<RowlistVecItem>& bt, int grid) {

@@ -172,11 +172,8 @@ int conef_randblock_step_batch_f32(const ConefRandBlockItem* items, int32_t coun
         if (shape.lds > lds) lds = shape.lds;
     }
     if (!table.empty()) {
-        if (lds > 48 * 1024) {
-            hipError_t e = hipFuncSetAttribute((const void*)randblock_rowlist_batch_kernel,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return (int)e;
-        }
+        hipError_t e = conef_allow_lds((const void*)randblock_rowlist_batch_kernel, lds);
+        if (e != hipSuccess) return (int)e;
         const double omb = 1. - (double)beta;
         int rc = rb_run(table, blocks, [&](const RbBatch<ListItem>& bt, int grid) {
             hipLaunchKernelGGL(randblock_rowlist_batch_kernel, dim3((unsigned)grid), dim3(kConefRowlistThreads), lds, s,

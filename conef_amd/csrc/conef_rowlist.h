@@ -490,10 +490,8 @@ int conef_launch_rowlist(Front front, ConefRowlistView plan, const CsT* cs_in, C
     ConefRowlistShape shape;
     if (!conef_rowlist_shape(n, d, w, Front::kNeedsCells, &shape)) return CONEF_ERR_INVALID;
     auto k = conef_rowlist_kernel<CsT, Front>;
-    if (shape.lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)shape.lds);
-        if (e != hipSuccess) return (int)e;
-    }
+    hipError_t e = conef_allow_lds((const void*)k, shape.lds);
+    if (e != hipSuccess) return (int)e;
     const double omb = 1. - (double)beta;   // (1. - beta) with beta an fp32 value, CountSketch.py:38,63
     hipLaunchKernelGGL(k, dim3((unsigned)shape.tiles), dim3(kConefRowlistThreads), shape.lds, s, front, plan, cs_in,
                        cs_out, n, (int)d, (int)w, shape.rb, omb, shape.pk_lds);
