@@ -127,15 +127,28 @@ class _RoundPlan:
     compressed, the table of matrices the batch entry points read, the views into the P / Q
     arenas.  Built on the first step of a bucket and reused while the bucket keeps its buffer
     and layout, so that a step costs a handful of foreign calls however many tensors it has."""
-    __slots__ = ("key", "shapes", "work", "passthrough", "before", "after", "total_ps", "total_qs", "arena_key", "ps",
+    __slots__ = ("small", "sig", "errs_sig", "cs_static", "env_ahead", "env_topk_side", "env_small", "key", "shapes", "work", "passthrough", "before", "after", "total_ps", "total_qs", "arena_key", "ps",
                  "qs", "items", "count", "sketches", "fused_sketch", "batched_update", "residual_offsets",
                  "topk_table", "q_next", "q_next_ptrs", "q_next_ready", "made", "q_next_views", "items_next", "q_next_event",
                  "topk_event", "ws_need", "handoff_event", "gs_table", "topk_number", "q_next_number")
 
 
+def _layout_signature(grads):
+    """What a step compares instead of every tensor's shape: a bucket keeps its buffer, its length
+    (both part of the plan's key) and its parameters for as long as DDP keeps the bucket."""
+    return (len(grads), grads[0].shape, grads[-1].shape) if grads else (0, None, None)
+
+
 def _build_round(state, grads, shapes, key, error_mode):
     plan = _RoundPlan()
     plan.key, plan.shapes = key, shapes
+    plan.sig = _layout_signature(grads)
+    plan.errs_sig = None
+    plan.cs_static = False
+    # switches read when the plan is built (a bucket's plan lives as long as its buffer does)
+    plan.env_ahead = os.environ.get("CONEF_ROUND_AHEAD", "1") != "0"
+    plan.env_topk_side = os.environ.get("CONEF_TOPK_SIDE", "1") != "0"
+    plan.env_small = os.environ.get("CONEF_ROUND_SMALL", "1") != "0"
     plan.work, plan.passthrough = [], []
     plan.before = plan.after = plan.total_ps = plan.total_qs = 0
     for tensor in grads:                                            # Step I (:394-418)
@@ -158,6 +171,7 @@ def _build_round(state, grads, shapes, key, error_mode):
         it = plan.items[cnt]
         it.x, it.n, it.m, it.r, it.w = matrix.data_ptr(), n, m, rank, 1
     plan.arena_key = None
+    plan.small = None               # (mode1, mode3) -> whether the bucket's round runs as one launch (a bucket of small matrices)
     plan.sketches = []
     plan.fused_sketch = False
     plan.batched_update = False
@@ -191,7 +205,7 @@ def topk_table_is_stale(table, tensors, topk_ratio):
     return table is None or table[0] != tuple(t.data_ptr() for t in tensors) or table[5] != topk_ratio
 
 
-def plan_for(state, bucket_index, grads, shapes, key, error_mode, device, stream_now):
+def plan_for(state, bucket_index, grads, key, error_mode, device, stream_now):
     """The bucket's cached round plan, rebuilt when its buffer or layout changed.  What the
     replaced plan's last round left running on the side stream works on tensors that outlive the
     plan (the error tensors in ``state.error_dict``, the Q arena): the pending top-k is handed on
@@ -199,9 +213,9 @@ def plan_for(state, bucket_index, grads, shapes, key, error_mode, device, stream
     round is about to run on (``stream_now()``) is ordered after a pending copy of the Q arena
     here, since the new plan no longer knows of it."""
     plan = state.round_cache.get(bucket_index)
-    if plan is None or plan.key != key or plan.shapes != shapes:
+    if plan is None or plan.key != key or plan.sig != _layout_signature(grads):
         old = plan
-        plan = _build_round(state, grads, shapes, key, error_mode)
+        plan = _build_round(state, grads, [t.shape for t in grads], key, error_mode)
         if old is not None:
             plan.topk_number, plan.topk_event = old.topk_number, old.topk_event
             if old.q_next_number is not None:
@@ -286,10 +300,9 @@ def _run_round(state, bucket, error_mode):
     errs = state.error_dict.get(bucket_index)
 
     grads = _bucket.gradients(bucket)
-    shapes = [t.shape for t in grads]
     key = (base_ptr, total_length, error_mode, state.matrix_approximation_rank, state.min_compression_rate,
            getattr(state, "sketch_size", None), dense_err.data_ptr() if dense_err is not None else 0)
-    plan = plan_for(state, bucket_index, grads, shapes, key, error_mode, device, lambda: _lib.current_stream(device))
+    plan = plan_for(state, bucket_index, grads, key, error_mode, device, lambda: _lib.current_stream(device))
     work, items, count = plan.work, plan.items, plan.count
     state.total_numel_before_compression += plan.before
     state.total_numel_after_compression += plan.after
@@ -331,7 +344,9 @@ def _run_round(state, bucket, error_mode):
                 errs[cnt] = torch.zeros_like(matrix)
             items[cnt].err = errs[cnt].data_ptr()
     elif error_mode == "conef":
-        if len(plan.sketches) != count or any(errs.get(cnt) is not cs for cnt, (cs, _) in enumerate(plan.sketches)):
+        # (the dict of a bucket's sketches is only ever replaced as a whole, with the round cache cleared:
+        # load_state_dict; its identity and size stand for its entries)
+        if plan.errs_sig != (id(errs), len(errs)) or len(plan.sketches) != count:
             plan.sketches = []
             for cnt, (matrix, n, m, rank) in enumerate(work):
                 if cnt not in errs:
@@ -344,8 +359,16 @@ def _run_round(state, bucket, error_mode):
                 plan.sketches.append((cs, sk_plan))
             plan.batched_update = all(p is not None and p.batchable for _, p in plan.sketches)
             plan.fused_sketch = state.matrix_approximation_rank <= 8 and plan.batched_update
-        for cnt, (cs, _) in enumerate(plan.sketches):
-            items[cnt].cs = cs.cs.data_ptr()
+            plan.small = None
+            plan.errs_sig = (id(errs), len(errs))
+            # sketches on row lists are updated in place: their cells never move.  The others swap
+            # two buffers, so their pointers are refreshed every step.
+            plan.cs_static = all(p is not None and p.in_place for _, p in plan.sketches)
+            for cnt, (cs, _) in enumerate(plan.sketches):
+                items[cnt].cs = cs.cs.data_ptr()
+        if not plan.cs_static:
+            for cnt, (cs, _) in enumerate(plan.sketches):
+                items[cnt].cs = cs.cs.data_ptr()
     elif error_mode == "conef_v2":
         for cnt, (matrix, n, m, rank) in enumerate(work):
             if cnt not in errs:
@@ -398,8 +421,18 @@ def _run_round(state, bucket, error_mode):
         mode3 = 3 if error_mode == "conef" and plan.batched_update else 1
     else:
         mode3 = 0
-    if (state.matrix_approximation_rank > 8 and state.warm_start and count
-            and int(getattr(state, "hook_streams", 1) or 1) <= 1 and os.environ.get("CONEF_ROUND_AHEAD", "1") != "0"):
+    if plan.small is None or plan.small[0] != (mode1, mode3):
+        # a bucket of small matrices (every one fits a workgroup's LDS with its factors): the whole round in one launch
+        fits = bool(count and mode3 in (0, 1, 2) and plan.env_small
+                    and lib.conef_psgd_round_small_fits(items, count, mode1, mode3, HASH_A, HASH_B))
+        plan.small = ((mode1, mode3), fits)
+    if plan.small[1]:
+        plan.q_next_ready = False
+        rc = lib.conef_psgd_round_small_f32(items, count, mode1, mode3, float(alpha), float(state.beta) if mode3 == 2 else 0.0,
+                                            eps, HASH_A, HASH_B, stream)
+        _lib.check(rc, "conef_psgd_round_small_f32")
+    elif (state.matrix_approximation_rank > 8 and state.warm_start and count
+            and int(getattr(state, "hook_streams", 1) or 1) <= 1 and plan.env_ahead):
         # Ranks on the matrix cores: the round as its separate launches, with the Gram-Schmidt of the new
         # Q factors (which the reference runs at the start of the bucket's next round,
         # powerSGD_hook.py:496-497: 27-35 us of dependent steps on a few workgroups) on a side stream,
@@ -409,7 +442,7 @@ def _run_round(state, bucket, error_mode):
         _round_with_q_on_the_side(state, plan, lib, items, count, mode1, mode3, alpha, eps, ws_ptr, ws_len, stream,
                                   device, q_mem, qs)
     elif (mode3 in (0, 1, 2) and state.matrix_approximation_rank <= 8 and state.warm_start and count and count <= 24
-            and os.environ.get("CONEF_ROUND_AHEAD", "1") != "0"):
+            and plan.env_ahead):
         # The bucket's next round starts by orthogonalising the Q factors this round leaves
         # (powerSGD_hook.py:496-497): a few workgroups and an idle machine.  Workgroups of this
         # round's last launch do it instead, into a second buffer, where the kernel allows
@@ -436,8 +469,7 @@ def _run_round(state, bucket, error_mode):
                                       eps, HASH_A, HASH_B, ws_ptr, ws_len, stream)
         _lib.check(rc, "conef_psgd_round_f32")
     if error_mode == "topk":
-        if (count and int(getattr(state, "hook_streams", 1) or 1) <= 1
-                and os.environ.get("CONEF_ROUND_AHEAD", "1") != "0" and os.environ.get("CONEF_TOPK_SIDE", "1") != "0"):
+        if count and int(getattr(state, "hook_streams", 1) or 1) <= 1 and plan.env_ahead and plan.env_topk_side:
             # The sparsification only touches the error tensors, which nobody reads before this bucket's
             # next round: it runs on a side stream while this stream goes on with the next bucket (five
             # streaming passes next to launches that are mostly latency).  Same kernels, same values.

@@ -23,6 +23,7 @@
 #include "conef_gs_lanes.h"
 #include "conef_gs_gram.h"
 #include "conef_psgd_stream.h"
+#include "conef_psgd_small.h"
 #include "conef_hip.h"      // ConefPsgdItem, and a check of this file's definitions against the public header
 
 extern "C" int conef_cs_query_f32(float* x, const float* cs, int64_t n, int64_t d, int32_t w, float alpha, int32_t a,
@@ -3607,6 +3608,92 @@ int conef_psgd_round_ahead_f32(const ConefPsgdItem* items, int32_t count, int32_
     if (made) *made = used ? 1 : 0;
     if (pqt_mode == 3) rc = conef_psgd_sketch_update_batch_f32(items, count, beta, a, b, stream);
     return rc;
+}
+
+// Whether conef_psgd_round_small_f32 takes this bucket: every matrix has at most 16384 elements (and
+// fits one workgroup's LDS with its factors and its sketch's bucket lists), ranks up to 8, and
+// (modes 2) a row-list plan per sketch.
+int conef_psgd_round_small_fits(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, int32_t a,
+                                int32_t b)
+{
+    if (count < 1 || !items || mq_mode < 0 || mq_mode > 2 || pqt_mode < 0 || pqt_mode > 2) return 0;
+    if ((mq_mode == 2) != (pqt_mode == 2)) return 0;
+    for (int k = 0; k < count; ++k) {
+        const ConefPsgdItem& it = items[k];
+        if (!item_ok(it) || it.r > 8 || it.n * it.m > kSmallMaxElements) return 0;
+        if ((mq_mode == 1 || pqt_mode == 1) && !it.err) return 0;
+        int w = 0;
+        if (mq_mode == 2) {
+            const ConefPlanHeader* hp = (const ConefPlanHeader*)it.plan_host;
+            if (!it.cs || !it.plan_dev || !conef_plan_matches(hp, it.n, it.m, it.w, a, b) || hp->kind != kConefPlanRowlist)
+                return 0;
+            w = it.w;
+        }
+        if (small_lds_bytes((int)it.n, (int)it.m, rank_bound(it.r), w) > kSmallLdsLimit) return 0;
+    }
+    return 1;
+}
+
+// The round of conef_psgd_round_f32 for a bucket of small matrices, in ONE launch: a workgroup per
+// matrix, the matrix in LDS, workgroup barriers between the stages (conef_psgd_small.h).
+int conef_psgd_round_small_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, float alpha,
+                               float beta, float eps, int32_t a, int32_t b, void* stream)
+{
+    if (!conef_psgd_round_small_fits(items, count, mq_mode, pqt_mode, a, b)) return CONEF_ERR_INVALID;
+    hipStream_t s = (hipStream_t)stream;
+    const double omb = 1. - (double)beta;
+    for (int k0 = 0; k0 < count; k0 += kSmallMaxItems) {
+        const int nb = count - k0 < kSmallMaxItems ? count - k0 : kSmallMaxItems;
+        SmallBatch batch;
+        int rp = 1;
+        size_t lds = 0;
+        for (int k = 0; k < nb; ++k) {
+            const ConefPsgdItem& it = items[k0 + k];
+            SmallItem& t = batch.item[k];
+            t.x = it.x;
+            t.err = it.err;
+            t.cs = it.cs;
+            t.csr = nullptr;
+            t.ent = nullptr;
+            t.pk = nullptr;
+            t.w = 0;
+            if (mq_mode == 2) {
+                const ConefRowlistView v = conef_rowlist_view((const ConefPlanHeader*)it.plan_host, it.plan_dev);
+                t.csr = v.csr;
+                t.ent = v.ent;
+                t.pk = v.pk;
+                t.w = it.w;
+            }
+            t.p = it.p;
+            t.q = it.q;
+            t.n = (int)it.n;
+            t.m = (int)it.m;
+            t.r = it.r;
+            t.fast = it.m % 4 == 0 && aligned16(it.x) && ((mq_mode != 1 && pqt_mode != 1) || aligned16(it.err));
+            if (rank_bound(it.r) > rp) rp = rank_bound(it.r);
+        }
+        for (int k = 0; k < nb; ++k) {
+            const size_t need = small_lds_bytes(batch.item[k].n, batch.item[k].m, rp, batch.item[k].w);
+            if (need > lds) lds = need;
+        }
+        if (lds > kSmallLdsLimit) return CONEF_ERR_INVALID;      // a low-rank item next to a rank-8 one: sized for the launch's rank
+#define CONEF_SMALL(RP)                                                                                         \
+    do {                                                                                                        \
+        auto kern = psgd_small_round_kernel<RP>;                                                                \
+        if (hipError_t e = conef_allow_lds((const void*)kern, lds); e != hipSuccess) return (int)e;             \
+        hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3(kSmallThreads), lds, s, batch, mq_mode, pqt_mode, alpha, omb, eps); \
+    } while (0)
+        switch (rp) {
+            case 1: CONEF_SMALL(1); break;
+            case 2: CONEF_SMALL(2); break;
+            case 4: CONEF_SMALL(4); break;
+            default: CONEF_SMALL(8); break;
+        }
+#undef CONEF_SMALL
+        const int rc = (int)hipGetLastError();
+        if (rc != CONEF_OK) return rc;
+    }
+    return CONEF_OK;
 }
 
 int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, float alpha,

@@ -346,6 +346,22 @@ int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_m
                          float beta, float eps, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
                          void* stream);
 
+/* The same round in ONE launch for a bucket of small matrices (a few thousand elements each, where a
+ * round of separate launches is nothing but launch latency): a workgroup
+ * per matrix keeps the matrix, both factors and the sketch's bucket lists in LDS and takes it through
+ * the reference's steps in the reference's order - orthogonalise Q, X = M + error, P = X Q,
+ * orthogonalise P, Q = X^T P, M = P Q^T, residual to the dense error or into the sketch (a bucket's
+ * terms in ascending column order).  Replaces powerSGD_hook.py:473-564 at world size 1.
+ * mq_mode / pqt_mode as above (0, 1, or both 2); no workspace.  conef_psgd_round_small_fits says
+ * (1 / 0) whether a bucket qualifies: every matrix has at most 16384 elements (one workgroup does
+ * all of a matrix's work: beyond that the separate launches, which spread a matrix over many
+ * workgroups, are faster), ranks up to 8, a row-list plan per sketch in mode 2; the round returns
+ * CONEF_ERR_INVALID for a bucket that does not. */
+int conef_psgd_round_small_fits(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, int32_t a,
+                                int32_t b);
+int conef_psgd_round_small_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, float alpha,
+                               float beta, float eps, int32_t a, int32_t b, void* stream);
+
 /* The middle of that round as a call of its own, for a caller that splits the round (the hooks above
  * rank 8 do, to orthogonalise the new Q on a side stream meanwhile): P = X Q with the Q factors of
  * `first` (a copy of `items` whose q may point elsewhere; null: items' own), P orthogonalised

@@ -530,6 +530,10 @@ def psgd_resync_factory(st, ost, mode, free_steps=4):
         elif mode in ("conef", "conef_v2"):
             for k in ost.error_dict[0]:
                 ost.error_dict[0][k].cs[...] = to_np(st.error_dict[0][k].cs)
+        elif mode == "topk":
+            st.settle()
+            for k in ost.error_dict[0]:
+                ost.error_dict[0][k][...] = to_np(st.error_dict[0][k])
     return resync
 
 
@@ -586,6 +590,80 @@ def test_powersgd_hook_parity(oracle, shapes, rank, ss, mode):
         # values are 10x below these bounds; a regression that doubled the drift of a step or two would not be
         assert drift[3] <= 1e-5
         assert drift[-1] <= FREE_RUNNING_DRIFT_AT_STEP_10[mode], drift
+
+
+SMALL_BUCKETS = [
+    [(16, 27), (16,), (28, 576), (10, 64), (10,), (33, 40), (3, 5), (1, 9), (7, 1023)],
+    [(24, 64, 3, 3), (64,), (50, 300), (120, 130)],
+]
+
+
+@pytest.mark.parametrize("eps", [0.0, 1e-8])
+@pytest.mark.parametrize("rank", [1, 2, 4, 8])
+@pytest.mark.parametrize("mode", [None, "ef", "conef", "topk"])
+def test_small_bucket_round_in_one_launch(monkeypatch, oracle, mode, rank, eps):
+    """A bucket of small matrices (at most 16384 elements each) runs its round as one launch, a workgroup
+    per matrix (powerSGD_hook.py:473-564 in the reference's order of steps): against the oracle
+    with the state carried over four steps, odd shapes and shapes narrower than the rank included,
+    and against the same state run through the separate launches."""
+    from conef_amd import _lib
+    lib = _lib.load()
+    for shapes in SMALL_BUCKETS:
+        st, hook = _state_for(mode, rank, 0.3, orthogonalization_epsilon=eps)
+        ost = oracle.PowerSGDOracle(matrix_approximation_rank=rank, error_mode=mode, sketch_size=0.3, beta=0.9,
+                                    topk_ratio=0.4, orthogonalization_epsilon=eps)
+        # (matrices of a few rows make ill-conditioned factors: from the second step on the oracle
+        # restarts from the device's state, as in test_powersgd_hook_parity)
+        run_steps(hook, st, ost, shapes, 4, check=psgd_check_factory(st, ost, mode),
+                  resync=psgd_resync_factory(st, ost, mode, free_steps=2))
+        assert st.round_cache[0].small[1], "the bucket was expected to take the one-launch round"
+        # the same steps through the separate launches: the same results to rounding
+        monkeypatch.setenv("CONEF_ROUND_SMALL", "0")
+        other, _ = _state_for(mode, rank, 0.3, orthogonalization_epsilon=eps)
+        run_steps(hook, other, oracle.PowerSGDOracle(matrix_approximation_rank=rank, error_mode=mode, sketch_size=0.3,
+                                                     beta=0.9, topk_ratio=0.4, orthogonalization_epsilon=eps),
+                  shapes, 4, check=lambda step, gd, og: None)
+        monkeypatch.delenv("CONEF_ROUND_SMALL")
+        assert not other.round_cache[0].small[1]
+        assert_close(st.p_memory_dict[0], other.p_memory_dict[0], rel=1e-4, what="P, one launch against separate launches")
+        assert_close(st.q_memory_dict[0], other.q_memory_dict[0], rel=1e-4, what="Q, one launch against separate launches")
+    # a bucket with one matrix of more than 16384 elements does not qualify
+    st, hook = _state_for(mode, rank, 0.3)
+    st.iter = 2
+    big = [(16, 144), (64, 576)]
+    hook(st, FakeGradBucket(grads(numel_of(big), 5).cuda(), big)).wait()
+    assert not st.round_cache[0].small[1]
+    assert lib.conef_psgd_round_small_fits(None, 0, 0, 0, 1, 1) == 0
+
+
+@pytest.mark.parametrize("eps", [0.0, 1e-8])
+@pytest.mark.parametrize("mode", ["ef", "conef"])
+def test_small_bucket_with_an_all_zero_gradient_matrix(oracle, mode, eps):
+    """The one-launch round on a frozen parameter's all-zero gradient: NaN where the reference's
+    0 / 0 gives NaN (epsilon 0), zeros at epsilon != 0, the bucket's other matrices untouched."""
+    shapes = [(28, 576), (64,), (32, 288), (10, 64)]
+    zero_at = 2
+    st, hook = _state_for(mode, 2, 0.5, orthogonalization_epsilon=eps)
+    ost = oracle.PowerSGDOracle(matrix_approximation_rank=2, error_mode=mode, sketch_size=0.5, beta=0.9,
+                                orthogonalization_epsilon=eps)
+    st.iter = 2
+    offs = np.cumsum([0] + [int(np.prod(s)) for s in shapes])
+    for step in range(3):
+        g = grads(numel_of(shapes), 900 + step)
+        g[offs[zero_at]:offs[zero_at + 1]] = 0
+        gd = g.cuda()
+        hook(st, FakeGradBucket(gd, shapes)).wait()
+        assert st.round_cache[0].small[1]
+        og = g.numpy().copy()
+        ost.step(0, og, shapes)
+        got = to_np(gd)
+        for k in range(len(shapes)):
+            _nan_aware_close(got[offs[k]:offs[k + 1]], og[offs[k]:offs[k + 1]], "eps %g step %d tensor %d" % (eps, step, k))
+        if mode == "conef":
+            for k in ost.error_dict[0]:
+                _nan_aware_close(st.error_dict[0][k].cs, ost.error_dict[0][k].cs, "sketch %d step %d" % (k, step))
+        else:
+            _nan_aware_close(st.error_dict[0], ost.error_dict[0], "dense error step %d" % step)
 
 
 @pytest.mark.parametrize("shapes,rank,ss", PSGD_CASES[:3])

@@ -71,17 +71,19 @@ def test_a_rebuilt_round_plan_still_waits_for_the_side_stream():
     try:
         state = SimpleNamespace(round_cache={}, matrix_approximation_rank=2, min_compression_rate=2)
         grads = [torch.zeros(16, 32), torch.zeros(7)]
-        shapes = [g.shape for g in grads]
         main = FakeStream(21)
-        first = engine.plan_for(state, 0, grads, shapes, ("buffer-a",), "topk", device, lambda: main)
+        first = engine.plan_for(state, 0, grads, ("buffer-a",), "topk", device, lambda: main)
         assert state.round_cache[0] is first and first.count == 1 and main.waited_for == []
         # the same key: the same plan, nothing to order
-        assert engine.plan_for(state, 0, grads, shapes, ("buffer-a",), "topk", device, lambda: main) is first
+        assert engine.plan_for(state, 0, grads, ("buffer-a",), "topk", device, lambda: main) is first
+        # the same buffer with another layout: a new plan
+        assert engine.plan_for(state, 0, grads[:1], ("buffer-a",), "topk", device, lambda: main) is not first
+        first = engine.plan_for(state, 0, grads, ("buffer-a",), "topk", device, lambda: main)
         # its round left a top-k and a Gram-Schmidt of the next Q factors on the side stream
         first.topk_event = "topk-done"
         first.topk_number = _pools.side_recorded(device, "topk-done")
         # the bucket's buffer moves: a new plan, which inherits the pending top-k ...
-        second = engine.plan_for(state, 0, grads, shapes, ("buffer-b",), "topk", device, lambda: main)
+        second = engine.plan_for(state, 0, grads, ("buffer-b",), "topk", device, lambda: main)
         assert second is not first and state.round_cache[0] is second
         assert (second.topk_number, second.topk_event) == (first.topk_number, "topk-done")
         assert main.waited_for == []
@@ -94,7 +96,7 @@ def test_a_rebuilt_round_plan_still_waits_for_the_side_stream():
         assert [p.topk_event for p in state.round_cache.values()] == ["topk-done"]
         # a pending copy of the Q arena is waited for when the plan that knew of it goes
         second.q_next_number = _pools.side_recorded(device, "q-copied")
-        third = engine.plan_for(state, 0, grads, shapes, ("buffer-c",), "topk", device, lambda: main)
+        third = engine.plan_for(state, 0, grads, ("buffer-c",), "topk", device, lambda: main)
         assert third.q_next_number is None and main.waited_for == ["topk-done", "q-copied"]
     finally:
         _pools._SIDE_ORDER.pop(device, None)
