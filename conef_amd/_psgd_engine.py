@@ -247,28 +247,48 @@ def run_round(state, bucket, error_mode):
     matrix) | 'conef_v2' (count sketch over the [m,n] re-view of each matrix's memory,
     powerSGD_hook.py:918-920,1074-1076) | 'topk' (dense per matrix, magnitude-sparsified).
 
-    With ``state.hook_streams`` > 1 the round is enqueued on one of that many side streams: the
-    side stream first waits for the stream the hook was called on (the gradients are ready there),
-    and the returned Future carries the side stream's completion event, which is what DDP (or any
-    caller of ``wait()``) orders its own stream after."""
-    streams = int(getattr(state, "hook_streams", 1) or 1)
+    With ``state.hook_streams`` = N > 1 the buckets of a step are dealt out over N streams: bucket
+    i with i % N == 0 stays on the stream the hook was called on, the others go to one of N - 1 side
+    streams.  A side stream first waits for the hook's stream (the gradients are ready there), and
+    the returned Future carries the side stream's completion event, which is what DDP (or any caller
+    of ``wait()``) orders its own stream after.  (Handing a bucket to another stream costs the host
+    about 30 us, more than issuing its four launches: every N-th bucket is spared that.)"""
     input_tensor = _bucket.buffer(bucket)
+    streams = streams_for(state, input_tensor)
     if streams <= 1 or not input_tensor.is_cuda or state.iter < state.start_powerSGD_iter:
-        return _run_round(state, bucket, error_mode)
+        return _run_round(state, bucket, error_mode, 1)
     device = input_tensor.device
     index = _bucket.index(bucket)
-    side = _side_stream(device, index, streams)
+    lane = index % streams
+    if lane == 0:
+        return _run_round(state, bucket, error_mode, streams)
+    side = _side_stream(device, lane - 1, streams - 1)
     # the side stream starts where the hook's stream is now (one event per side stream, recorded again
     # for every bucket: a wait takes the event as it is when the wait is enqueued)
-    event = _pools.side_event(device, index, streams)
+    event = _pools.side_event(device, lane - 1, streams - 1)
     event.record(_lib.current_stream(device))
     side.wait_event(event)
     input_tensor.record_stream(side)
     with _lib.on_stream(side):
-        return _run_round(state, bucket, error_mode)
+        return _run_round(state, bucket, error_mode, streams)
 
 
-def _run_round(state, bucket, error_mode):
+AUTO_STREAMS_MIN_NUMEL = 1 << 20
+
+
+def streams_for(state, input_tensor):
+    """Streams the rounds of this state's buckets are dealt out over (the hook's own included).
+    ``state.hook_streams`` 0 leaves it to the bucket's size: buckets of a million elements or more
+    alternate between the hook's stream and a side stream (a bucket's launches that are mostly
+    latency then overlap the neighbouring bucket's streaming passes), a smaller one stays on the
+    hook's stream, where handing it over would cost more than it brings."""
+    streams = int(getattr(state, "hook_streams", 1) or 0)
+    if streams == 0:
+        streams = 2 if input_tensor.numel() >= AUTO_STREAMS_MIN_NUMEL else 1
+    return streams
+
+
+def _run_round(state, bucket, error_mode, streams=1):
     group, world_size = _bucket.group_and_size(state.process_group)
     input_tensor = _bucket.buffer(bucket)
 
@@ -432,7 +452,7 @@ def _run_round(state, bucket, error_mode):
                                             eps, HASH_A, HASH_B, stream)
         _lib.check(rc, "conef_psgd_round_small_f32")
     elif (state.matrix_approximation_rank > 8 and state.warm_start and count
-            and int(getattr(state, "hook_streams", 1) or 1) <= 1 and plan.env_ahead):
+            and streams <= 1 and plan.env_ahead):
         # Ranks on the matrix cores: the round as its separate launches, with the Gram-Schmidt of the new
         # Q factors (which the reference runs at the start of the bucket's next round,
         # powerSGD_hook.py:496-497: 27-35 us of dependent steps on a few workgroups) on a side stream,
@@ -469,7 +489,7 @@ def _run_round(state, bucket, error_mode):
                                       eps, HASH_A, HASH_B, ws_ptr, ws_len, stream)
         _lib.check(rc, "conef_psgd_round_f32")
     if error_mode == "topk":
-        if count and int(getattr(state, "hook_streams", 1) or 1) <= 1 and plan.env_ahead and plan.env_topk_side:
+        if count and streams <= 1 and plan.env_ahead and plan.env_topk_side:
             # The sparsification only touches the error tensors, which nobody reads before this bucket's
             # next round: it runs on a side stream while this stream goes on with the next bucket (five
             # streaming passes next to launches that are mostly latency).  Same kernels, same values.

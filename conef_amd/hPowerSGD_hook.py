@@ -89,10 +89,13 @@ class hPowerSGDState(Checkpointable):
         # Not in the reference: with hook_streams > 1 bucket i runs on side stream i % hook_streams
         # of its device (the Future orders the consumer after it, as the reference's Futures order it
         # after the work of the communication stream), so the latency-bound launches of one bucket
-        # overlap the streaming passes of the next.  None: two streams above rank 8, where a
-        # bucket's round is ten launches (BERT-large rank 32: 4.4 ms a step against 6.0), else one.
+        # overlap the streaming passes of the next; bucket i with i % hook_streams == 0 stays on
+        # the hook's own stream.  None: three streams above rank 8, where a bucket's round is ten
+        # launches; up to rank 8 each bucket's size decides (0: two streams for buckets of a million
+        # elements or more - BERT-large rank 8 with a top-k error: 4.0 ms a step against 4.7 - one
+        # for smaller ones).  The top-k of the errors runs on a side stream of its own either way.
         if hook_streams is None:
-            hook_streams = 2 if matrix_approximation_rank > 8 else 1
+            hook_streams = 3 if matrix_approximation_rank > 8 else 0
         self.hook_streams = hook_streams
         self.use_error_compression = use_error_compression
         self.topk_ratio = topk_ratio

@@ -98,10 +98,15 @@ def test_hooks_register_directly():
 
 
 def test_hook_streams_is_taken_from_the_namespace_when_present():
-    """Not a flag of the reference's drivers: one stream up to rank 8 and two above unless the
-    namespace says otherwise."""
+    """Not a flag of the reference's drivers.  Unless the namespace says otherwise: three streams above
+    rank 8; up to rank 8 each bucket's size decides (0)."""
+    import torch
+    from conef_amd import _psgd_engine
     for name in ("ef_powersgd", "conef_powersgd", "hefsgd_powersgd"):
-        assert make(name)[0].hook_streams == 1
+        assert make(name)[0].hook_streams == 0
+        state = make(name)[0]
+        assert _psgd_engine.streams_for(state, torch.empty(1 << 20)) == 2
+        assert _psgd_engine.streams_for(state, torch.empty(1000)) == 1
         assert make(name, hook_streams=2)[0].hook_streams == 2
-        assert make(name, matrix_approximation_rank=32)[0].hook_streams == 2
+        assert make(name, matrix_approximation_rank=32)[0].hook_streams == 3
         assert make(name, matrix_approximation_rank=32, hook_streams=1)[0].hook_streams == 1

@@ -553,8 +553,11 @@ PSGD_CASES = [
 ]
 
 
-# placeholders until measured on the device
-FREE_RUNNING_DRIFT_AT_STEP_10 = {None: 1.0, "ef": 1.0, "conef": 1.0}
+# ResNet-20 at rank 2, the hook and the oracle each running on their own state for ten steps with no
+# resynchronisation: relative L2 distance of the decompressed buckets at the tenth step.  Measured on an
+# MI355X: 5.3e-7 without error feedback, 5.7e-6 with the dense error, 7.4e-7 with the sketched one; the
+# bounds leave a factor of about four.
+FREE_RUNNING_DRIFT_AT_STEP_10 = {None: 2e-6, "ef": 2e-5, "conef": 3e-6}
 
 
 @pytest.mark.parametrize("shapes,rank,ss", PSGD_CASES)
@@ -586,8 +589,8 @@ def test_powersgd_hook_parity(oracle, shapes, rank, ss, mode):
     assert before == steps * numel_of(shapes) and 0 < after < before and rate > 1
     if drift:
         print("free-running drift per step (%s): %s" % (mode, " ".join("%.2e" % d for d in drift)))
-        # relative L2 distance of the decompressed bucket at the configuration's last step: the measured
-        # values are 10x below these bounds; a regression that doubled the drift of a step or two would not be
+        # relative L2 distance of the decompressed bucket: the fp32 tolerance still holds four steps in,
+        # and the tenth step stays within a small factor of what was measured
         assert drift[3] <= 1e-5
         assert drift[-1] <= FREE_RUNNING_DRIFT_AT_STEP_10[mode], drift
 
@@ -820,12 +823,12 @@ def test_powersgd_rounds_on_side_streams(mode):
                                 use_error_compression=True, topk_ratio=0.4, hook_streams=streams)
             hook = hpowerSGD_hook
         else:
-            # rank 32 takes two streams when the state is not told otherwise (None)
+            # rank 32 takes three streams when the state is not told otherwise (None)
             st = PowerSGDState(None, matrix_approximation_rank=32 if mode == "conef32" else 8, start_powerSGD_iter=2,
                                use_error_feedback=True, use_error_compression=mode.startswith("conef"), sketch_size=0.1,
                                beta=0.9, hook_streams=None if mode == "conef32" and streams == 3 else streams)
             hook = powerSGD_hook
-            assert st.hook_streams == (2 if mode == "conef32" and streams == 3 else streams)
+            assert st.hook_streams == streams
         st.iter = 2
         outs = []
         for step in range(4):
