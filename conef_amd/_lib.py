@@ -57,7 +57,8 @@ SIGNATURES = {
     "conef_psgd_sketch_update_batch_f32": [_P, _I32, _F32, _I32, _I32, _P],
     "conef_psgd_round_f32": [_P, _I32, _I32, _I32, _F32, _F32, _F32, _I32, _I32, _P, _I64, _P],
     "conef_psgd_round_small_fits": [_P, _I32, _I32, _I32, _I32, _I32],
-    "conef_psgd_round_small_f32": [_P, _I32, _I32, _I32, _F32, _F32, _F32, _I32, _I32, _P],
+    "conef_psgd_round_small_workspace_bytes": [_P, _I32],
+    "conef_psgd_round_small_f32": [_P, _I32, _I32, _I32, _F32, _F32, _F32, _I32, _I32, _P, _I64, _P],
     "conef_psgd_round_ahead_f32": [_P, _I32, _I32, _I32, _F32, _F32, _F32, _I32, _I32, _P, _I32, _P, _P, _I64, _P],
     "conef_psgd_mtp_f32": [_P, _P, _P, _I64, _I64, _I32, _P, _I64, _P],
     "conef_psgd_pqt_f32": [_P, _P, _P, _I64, _I64, _I32, _P],
@@ -101,7 +102,8 @@ class RandBlockItem(ctypes.Structure):
 
 
 _RETURNS_I64 = ("conef_topk_workspace_bytes", "conef_topk_batch_workspace_bytes", "conef_plan_bytes",
-                "conef_plan_workspace_bytes", "conef_psgd_workspace_bytes", "conef_psgd_batch_workspace_bytes")
+                "conef_plan_workspace_bytes", "conef_psgd_workspace_bytes", "conef_psgd_batch_workspace_bytes",
+                "conef_psgd_round_small_workspace_bytes")
 
 _handle = None
 

@@ -449,7 +449,7 @@ def _run_round(state, bucket, error_mode, streams=1):
     if plan.small[1]:
         plan.q_next_ready = False
         rc = lib.conef_psgd_round_small_f32(items, count, mode1, mode3, float(alpha), float(state.beta) if mode3 == 2 else 0.0,
-                                            eps, HASH_A, HASH_B, stream)
+                                            eps, HASH_A, HASH_B, ws_ptr, ws_len, stream)
         _lib.check(rc, "conef_psgd_round_small_f32")
     elif (state.matrix_approximation_rank > 8 and state.warm_start and count
             and streams <= 1 and plan.env_ahead):

@@ -2070,6 +2070,7 @@ inline bool gsg_wants(const float* a, int64_t rows, int r)
 }
 
 std::atomic<unsigned> g_gsg_launches{0};
+std::atomic<unsigned> g_small_launches{0};
 
 // One launch over `count` matrices of rank r (workgroup ranges in batch.first).  A normal launch:
 // at most 128 workgroups of 256 threads, which a GPU that is running anything else still holds
@@ -3417,8 +3418,10 @@ int64_t conef_psgd_batch_workspace_bytes(const ConefPsgdItem* items, int32_t cou
         int64_t b = conef_psgd_workspace_bytes(items[k].n, items[k].m, items[k].r);
         if (b > single) single = b;
     }
-    return conef_align256(single) + conef_align256(4 * mtp_batch_layout(items, count, nullptr)) +
-           conef_align256(4 * mfma_batch_layout(items, count, nullptr)) + defer_region_bytes(items, count);
+    const int64_t launches = conef_align256(single) + conef_align256(4 * mtp_batch_layout(items, count, nullptr)) +
+                             conef_align256(4 * mfma_batch_layout(items, count, nullptr)) + defer_region_bytes(items, count);
+    const int64_t small = conef_psgd_round_small_workspace_bytes(items, count);      // the one-launch round's records
+    return small > launches ? small : launches;
 }
 
 int conef_psgd_mq_batch_f32(const ConefPsgdItem* items, int32_t count, int32_t mode, float alpha, int32_t a, int32_t b,
@@ -3610,17 +3613,21 @@ int conef_psgd_round_ahead_f32(const ConefPsgdItem* items, int32_t count, int32_
     return rc;
 }
 
-// Whether conef_psgd_round_small_f32 takes this bucket: every matrix has at most 16384 elements (and
-// fits one workgroup's LDS with its factors and its sketch's bucket lists), ranks up to 8, and
-// (modes 2) a row-list plan per sketch.
+// Whether conef_psgd_round_small_f32 takes this bucket: at most 24 matrices of at most 73728 elements
+// each (a matrix goes whole to one workgroup up to 10240 elements, over up to 16 otherwise), 128
+// workgroups in all, every workgroup's rows fit its LDS with the factors and the sketch's bucket
+// lists, ranks up to 8, and (modes 2) a row-list plan per sketch.
 int conef_psgd_round_small_fits(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, int32_t a,
                                 int32_t b)
 {
-    if (count < 1 || !items || mq_mode < 0 || mq_mode > 2 || pqt_mode < 0 || pqt_mode > 2) return 0;
+    if (count < 1 || count > kSmallMaxItems || !items || mq_mode < 0 || mq_mode > 2 || pqt_mode < 0 || pqt_mode > 2) return 0;
     if ((mq_mode == 2) != (pqt_mode == 2)) return 0;
+    int rp = 1, wgs = 0;
+    for (int k = 0; k < count; ++k)
+        if (item_ok(items[k]) && rank_bound(items[k].r) > rp) rp = rank_bound(items[k].r);      // a launch is sized for its largest rank
     for (int k = 0; k < count; ++k) {
         const ConefPsgdItem& it = items[k];
-        if (!item_ok(it) || it.r > 8 || it.n * it.m > kSmallMaxElements) return 0;
+        if (!item_ok(it) || it.r > 8 || it.n * it.m > kSmallMaxSlices * kSmallSliceElements) return 0;
         if ((mq_mode == 1 || pqt_mode == 1) && !it.err) return 0;
         int w = 0;
         if (mq_mode == 2) {
@@ -3629,24 +3636,48 @@ int conef_psgd_round_small_fits(const ConefPsgdItem* items, int32_t count, int32
                 return 0;
             w = it.w;
         }
-        if (small_lds_bytes((int)it.n, (int)it.m, rank_bound(it.r), w) > kSmallLdsLimit) return 0;
+        int rows_per;
+        wgs += small_slices(it.n, it.m, &rows_per);
+        if (small_lds_bytes(rows_per, (int)it.n, (int)it.m, rp, w) > kSmallLdsLimit) return 0;
     }
-    return 1;
+    return wgs <= kSmallMaxWgs ? 1 : 0;
+}
+
+// Bytes of workspace conef_psgd_round_small_f32 needs for this bucket (the records its sliced
+// matrices exchange; 0 when every matrix goes to one workgroup).
+int64_t conef_psgd_round_small_workspace_bytes(const ConefPsgdItem* items, int32_t count)
+{
+    if (count < 0 || (count > 0 && !items)) return -1;
+    int64_t recs = 0;
+    for (int k = 0; k < count; ++k) {
+        if (!item_ok(items[k])) return -1;
+        int rows_per;
+        const int sl = small_slices(items[k].n, items[k].m, &rows_per);
+        recs += (small_record_count(items[k].n, items[k].m, items[k].r, sl) + 31) / 32 * 32;
+    }
+    return recs * 8;
 }
 
 // The round of conef_psgd_round_f32 for a bucket of small matrices, in ONE launch: a workgroup per
 // matrix, the matrix in LDS, workgroup barriers between the stages (conef_psgd_small.h).
 int conef_psgd_round_small_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, float alpha,
-                               float beta, float eps, int32_t a, int32_t b, void* stream)
+                               float beta, float eps, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
+                               void* stream)
 {
     if (!conef_psgd_round_small_fits(items, count, mq_mode, pqt_mode, a, b)) return CONEF_ERR_INVALID;
+    const int64_t ws_need = conef_psgd_round_small_workspace_bytes(items, count);
+    if (ws_need > 0 && (!workspace || workspace_bytes < ws_need || ((uintptr_t)workspace & 7))) return CONEF_ERR_INVALID;
     hipStream_t s = (hipStream_t)stream;
     const double omb = 1. - (double)beta;
-    for (int k0 = 0; k0 < count; k0 += kSmallMaxItems) {
-        const int nb = count - k0 < kSmallMaxItems ? count - k0 : kSmallMaxItems;
+    unsigned tag = (g_small_launches.fetch_add(1u) + 1u) * 0x9E3779B9u;      // never the tag of the records' last use
+    if (tag == 0u) tag = 1u;
+    {
+        const int k0 = 0, nb = count;
         SmallBatch batch;
-        int rp = 1;
+        batch.count = nb;
+        int rp = 1, wgs = 0;
         size_t lds = 0;
+        unsigned long long* recs = (unsigned long long*)workspace;
         for (int k = 0; k < nb; ++k) {
             const ConefPsgdItem& it = items[k0 + k];
             SmallItem& t = batch.item[k];
@@ -3670,18 +3701,23 @@ int conef_psgd_round_small_f32(const ConefPsgdItem* items, int32_t count, int32_
             t.m = (int)it.m;
             t.r = it.r;
             t.fast = it.m % 4 == 0 && aligned16(it.x) && ((mq_mode != 1 && pqt_mode != 1) || aligned16(it.err));
+            t.slices = small_slices(it.n, it.m, &t.rows_per);
+            t.first = wgs;
+            wgs += t.slices;
+            t.recs = t.slices > 1 ? recs : nullptr;
+            recs += (small_record_count(it.n, it.m, it.r, t.slices) + 31) / 32 * 32;
             if (rank_bound(it.r) > rp) rp = rank_bound(it.r);
         }
         for (int k = 0; k < nb; ++k) {
-            const size_t need = small_lds_bytes(batch.item[k].n, batch.item[k].m, rp, batch.item[k].w);
+            const size_t need = small_lds_bytes(batch.item[k].rows_per, batch.item[k].n, batch.item[k].m, rp, batch.item[k].w);
             if (need > lds) lds = need;
         }
-        if (lds > kSmallLdsLimit) return CONEF_ERR_INVALID;      // a low-rank item next to a rank-8 one: sized for the launch's rank
+        if (lds > kSmallLdsLimit || wgs > kSmallMaxWgs) return CONEF_ERR_INVALID;
 #define CONEF_SMALL(RP)                                                                                         \
     do {                                                                                                        \
         auto kern = psgd_small_round_kernel<RP>;                                                                \
         if (hipError_t e = conef_allow_lds((const void*)kern, lds); e != hipSuccess) return (int)e;             \
-        hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3(kSmallThreads), lds, s, batch, mq_mode, pqt_mode, alpha, omb, eps); \
+        hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(kSmallThreads), lds, s, batch, tag, mq_mode, pqt_mode, alpha, omb, eps); \
     } while (0)
         switch (rp) {
             case 1: CONEF_SMALL(1); break;

@@ -18,19 +18,38 @@
 //
 // Global memory is touched once per operand: the gradient is read and the low-rank product written,
 // the sketch cells are gathered and rewritten, P and Q are read and written.
+//
+// A matrix of more than kSmallWholeElements elements is dealt out by rows over several workgroups
+// (`slices`), because everything a workgroup does for its rows - loading them, the products, the
+// gathers of sketch cells, the list walks - runs on one CU.  Rows are independent in steps 2, 3 and 6;
+// the slices meet twice: after step 3 every slice publishes its rows of the raw P and collects the
+// others' (step 4 then runs on the whole P in every slice, the same arithmetic on the same values),
+// and in step 5 every slice publishes its rows' share of X^T P and all add the shares up in slice
+// order.  Published values are 8-byte records {launch tag, float}: one relaxed agent-scope load
+// tells a reader whether the record is this launch's, so nothing is cleared between launches and no
+// fence is needed.  The waits are bounded: a slice whose peers never show up (they were never
+// resident) counts a give-up, leaves NaN in its rows of the result and ends.
 #pragma once
 #include "conef_device.h"
+#include "conef_gs_lanes.h"      // gs_count_give_up
 #include "conef_sketch_core.h"
 
 constexpr int kSmallThreads = 1024;
 constexpr int kSmallWaves = kSmallThreads / 64;
 constexpr int kSmallMaxItems = 24;
 constexpr size_t kSmallLdsLimit = 160 * 1024;     // all of a CU's LDS: one workgroup a CU
-// One workgroup does all of a matrix's work on one CU - its gathers of sketch cells, its list walks -
-// where the separate launches spread a matrix over many.  Up to about this many elements the
-// launches saved outweigh that ([32,288]: 16 us for the round against 24 us of four launches;
-// [64,576], 36864 elements: 32 us); a bucket with a larger matrix takes the separate launches.
-constexpr int64_t kSmallMaxElements = 16384;
+// One workgroup does all the work for its rows on one CU - their gathers of sketch cells, their list
+// walks - where the separate launches spread a matrix over many: [32,288] takes 14 us in the kernel
+// and [64,576] on one workgroup 33 us, against 24-30 us for a round of four launches.
+// Matrices above kSmallWholeElements go over slices of about kSmallSliceElements ([64,576] over
+// eight workgroups: 15 us against 33 us on one), at most kSmallMaxSlices of them; a launch holds at
+// most kSmallMaxWgs workgroups, far fewer than the machine has CUs, so the slices of a matrix (which
+// are neighbours in the grid) are resident together.
+constexpr int64_t kSmallWholeElements = 10240;
+constexpr int64_t kSmallSliceElements = 4608;
+constexpr int kSmallMaxSlices = 16;
+constexpr int kSmallMaxWgs = 128;
+constexpr unsigned kSmallSpinLimit = 1u << 20;
 
 struct SmallItem {
     float* x;               // [n,m] gradient in, P Q^T out
@@ -43,11 +62,51 @@ struct SmallItem {
     float* q;               // [m,r]
     int n, m, r, w;
     int fast;               // m % 4 == 0 and x (and err, where used) 16-byte aligned: the element-wise phases go by column quads
+    int slices;             // workgroups the rows are dealt over
+    int rows_per;           // rows a slice (the last one may hold fewer)
+    int first;              // the matrix's first workgroup in the launch
+    unsigned long long* recs;   // slices > 1: n*r records of the raw P, then slices * r*m records of the shares of X^T P
 };
 
 struct SmallBatch {
     SmallItem item[kSmallMaxItems];
+    int count;
 };
+
+// Slices a matrix goes over, and rows a slice.
+inline int small_slices(int64_t n, int64_t m, int* rows_per)
+{
+    int64_t s = n * m <= kSmallWholeElements ? 1 : (n * m + kSmallSliceElements - 1) / kSmallSliceElements;
+    if (s > kSmallMaxSlices) s = kSmallMaxSlices;
+    if (s > n) s = n;
+    const int64_t rp = (n + s - 1) / s;
+    *rows_per = (int)rp;
+    return (int)((n + rp - 1) / rp);
+}
+
+inline int64_t small_record_count(int64_t n, int64_t m, int r, int slices) { return slices > 1 ? n * r + (int64_t)slices * r * m : 0; }
+
+// A published float of this launch: waits (bounded) until the record carries the tag.
+__device__ __forceinline__ float small_await(const unsigned long long* rec, unsigned long long first, unsigned tag, int* failed)
+{
+    unsigned long long v = first;
+    unsigned spins = 0;
+    while ((unsigned)(v >> 32) != tag) {
+        ++spins;
+        if (spins > kSmallSpinLimit || ((spins & 255u) == 0 && *(volatile int*)failed)) {
+            *(volatile int*)failed = 1;
+            return 0.f;
+        }
+        __builtin_amdgcn_s_sleep(1);
+        v = __hip_atomic_load(rec, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return __uint_as_float((unsigned)v);
+}
+
+__device__ __forceinline__ void small_publish(unsigned long long* rec, float v, unsigned tag)
+{
+    __hip_atomic_store(rec, ((unsigned long long)tag << 32) | __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 __device__ __forceinline__ void ld4s(const float* p, float* v)
 {
@@ -63,14 +122,18 @@ __host__ __device__ inline int small_row_stride(int rp) { return rp > 1 ? rp + 1
 
 // floats of LDS before the (16-bit) bucket lists: matrix, Q, P, two sets of per-wave partial sums, and
 // with a sketch (w > 0) its list offsets and column table
-__host__ __device__ inline size_t small_lds_floats(int n, int m, int rp, int w)
+// (nl: the rows a workgroup holds, n: the rows of the matrix, whose whole P every slice keeps)
+__host__ __device__ inline size_t small_lds_floats(int nl, int n, int m, int rp, int w)
 {
     const size_t rs = (size_t)small_row_stride(rp);
-    return (((size_t)n * m + 3) & ~(size_t)3) + (size_t)m * rs + (size_t)n * rs + 2 * (size_t)kSmallWaves * rp + (size_t)w + 1 + 3 +
+    return (((size_t)nl * m + 3) & ~(size_t)3) + (size_t)m * rs + (size_t)n * rs + 2 * (size_t)kSmallWaves * rp + 3 + 4 + (size_t)w + 1 + 3 +
            (w > 0 ? (((size_t)m + 3) & ~(size_t)3) : 0);
 }
 
-inline size_t small_lds_bytes(int n, int m, int rp, int w) { return small_lds_floats(n, m, rp, w) * 4 + (((size_t)m + 7) & ~(size_t)7) * 2; }
+inline size_t small_lds_bytes(int nl, int n, int m, int rp, int w)
+{
+    return small_lds_floats(nl, n, m, rp, w) * 4 + (((size_t)m + 7) & ~(size_t)7) * 2;
+}
 
 // In-place Gram-Schmidt (powerSGD_hook.py:21-43) of a [rows, r] matrix in LDS (row stride RS), all
 // threads of the workgroup.  A thread keeps to its own rows, so a column step is one reduction of
@@ -148,21 +211,31 @@ struct SmallWalk {
 // `err`, 2 residual into the sketch.  FAST: the item's `fast`.
 template <int RP, bool FAST>
 __device__ __forceinline__ void
-psgd_small_round_body(const SmallItem& it, int mq_mode, int pqt_mode, float alpha, double one_minus_beta, float eps)
+psgd_small_round_body(const SmallItem& it, int slice, unsigned tag, int mq_mode, int pqt_mode, float alpha,
+                      double one_minus_beta, float eps)
 {
     constexpr int RS = RP > 1 ? RP + 1 : 1;
     constexpr int W = FAST ? 4 : 1;                        // elements a thread takes at a time
     extern __shared__ float small_lds[];
-    const int n = it.n, m = it.m, r = it.r, w = it.w;
+    const int rows = it.n, m = it.m, r = it.r, w = it.w;   // rows: of the whole matrix
+    const int slices = it.slices;
+    const int row0 = slice * it.rows_per;
+    const int n = rows - row0 < it.rows_per ? rows - row0 : it.rows_per;       // this workgroup's rows
     const int total = n * m;
+    float* const gx = it.x + (size_t)row0 * m;
+    float* const gerr = it.err ? it.err + (size_t)row0 * m : nullptr;
+    float* const gcs = it.cs ? it.cs + (size_t)row0 * w : nullptr;
     float* X = small_lds;
     float* Qs = X + ((total + 3) & ~3);
-    float* Ps = Qs + m * RS;
-    float* red = Ps + n * RS;
-    uint32_t* csr_l = reinterpret_cast<uint32_t*>(red + 2 * kSmallWaves * RP);
+    float* Pall = Qs + m * RS;                             // the whole P
+    float* Ps = Pall + row0 * RS;                          // this workgroup's rows of it
+    float* red = Pall + rows * RS;
+    int* failed = reinterpret_cast<int*>(small_lds + (((int)(red + 2 * kSmallWaves * RP - small_lds) + 3) & ~3));
+    uint32_t* csr_l = reinterpret_cast<uint32_t*>(failed + 4);
     uint32_t* pk_l = csr_l + ((w + 1 + 3) & ~3);
     uint16_t* ent_l = reinterpret_cast<uint16_t*>(pk_l + (mq_mode == 2 ? ((m + 3) & ~3) : 0));
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    if (tid == 0) *failed = 0;
 
     // ---- 1. Q into LDS (padding columns zero); the sketch's tables ride along
     {
@@ -213,11 +286,11 @@ psgd_small_round_body(const SmallItem& it, int mq_mode, int pqt_mode, float alph
                 const bool in = tid + (half * QH + u) * kSmallThreads < groups;
                 const int row = in ? issue.row : 0, col = in ? issue.col : 0;
                 const int e = (row * width + col) * 4;
-                gq[u] = *reinterpret_cast<const float4*>(it.x + e);
-                if (mq_mode == 1) ld4s(it.err + e, ev[u]);
+                gq[u] = *reinterpret_cast<const float4*>(gx + e);
+                if (mq_mode == 1) ld4s(gerr + e, ev[u]);
                 if (mq_mode == 2) {
                     const uint4 pw = *reinterpret_cast<const uint4*>(pk_l + col * 4);
-                    const float* cells = it.cs + row * w;
+                    const float* cells = gcs + row * w;
                     ev[u][0] = cells[pw.x & 0x7fffffffu];
                     ev[u][1] = cells[pw.y & 0x7fffffffu];
                     ev[u][2] = cells[pw.z & 0x7fffffffu];
@@ -261,11 +334,11 @@ psgd_small_round_body(const SmallItem& it, int mq_mode, int pqt_mode, float alph
                 const int row = in ? at.row : 0, col = in ? at.col : 0;
                 where[u] = in ? row * m + col : -1;
                 const int e = in ? where[u] : 0;
-                gv[u] = it.x[e];
-                if (mq_mode == 1) ev[u] = it.err[e];
+                gv[u] = gx[e];
+                if (mq_mode == 1) ev[u] = gerr[e];
                 if (mq_mode == 2) {
                     pw[u] = pk_l[col];
-                    ev[u] = it.cs[row * w + (int)(pw[u] & 0x7fffffffu)];
+                    ev[u] = gcs[row * w + (int)(pw[u] & 0x7fffffffu)];
                 }
                 at.next(m);
             }
@@ -296,12 +369,29 @@ psgd_small_round_body(const SmallItem& it, int mq_mode, int pqt_mode, float alph
 #pragma unroll
         for (int c = 0; c < RP; ++c) {
             const float s = conef_wave_sum(acc[c]);
-            if (lane == 0) Ps[row * RS + c] = s;
+            if (lane == 0) {
+                Ps[row * RS + c] = s;
+                if (slices > 1 && c < r) small_publish(it.recs + (size_t)(row0 + row) * r + c, s, tag);
+            }
         }
     }
+    if (slices > 1) {
+        // the other slices' rows of the raw P
+        for (int e = tid; e < rows * r; e += kSmallThreads) {
+            const int row = e / r, c = e - row * r;
+            if (row >= row0 && row < row0 + n) continue;
+            const unsigned long long* rec = it.recs + e;
+            Pall[row * RS + c] = small_await(rec, __hip_atomic_load(rec, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), tag, failed);
+        }
+        if (r < RP)
+            for (int e = tid; e < rows * (RP - r); e += kSmallThreads) {
+                const int row = e / (RP - r);
+                if (row < row0 || row >= row0 + n) Pall[row * RS + r + (e - row * (RP - r))] = 0.f;
+            }
+    }
     __syncthreads();
-    // ---- 4.
-    small_gram_schmidt<RP>(Ps, n, r, eps, red);
+    // ---- 4. (on the whole P, in every slice alike)
+    small_gram_schmidt<RP>(Pall, rows, r, eps, red);
 
     // ---- 5. Q = X^T P, left in LDS column by column (QT[c][col]: the last step reads quads of it) in
     // the place of the old Q, which nobody needs any more.  The columns go over the lanes; a matrix
@@ -344,14 +434,45 @@ psgd_small_round_body(const SmallItem& it, int mq_mode, int pqt_mode, float alph
             }
             __syncthreads();
         }
-        for (int e = tid; e < m * r; e += kSmallThreads) {
-            const int col = e / r, c = e - col * r;
-            it.q[e] = QT[c * m + col];
+        if (slices > 1) {
+            // this slice's share of X^T P out, then all shares added up in slice order: the same sum in
+            // every slice.  A thread publishes and collects the same entries, so no barrier in between.
+            unsigned long long* shares = it.recs + (size_t)rows * r;
+            const int count = r * m;
+            for (int e = tid; e < count; e += kSmallThreads) small_publish(shares + (size_t)slice * count + e, QT[e], tag);
+            for (int e = tid; e < count; e += kSmallThreads) {
+                float sum = 0.f;
+                for (int g0 = 0; g0 < slices; g0 += 4) {           // four shares requested at a time
+                    unsigned long long first[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int g = g0 + u;
+                        first[u] = g < slices && g != slice
+                                       ? __hip_atomic_load(shares + (size_t)g * count + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                       : 0ull;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int g = g0 + u;
+                        if (g < slices) {
+                            const float v = g == slice ? QT[e] : small_await(shares + (size_t)g * count + e, first[u], tag, failed);
+                            sum = g == 0 ? v : __fadd_rn(sum, v);
+                        }
+                    }
+                }
+                QT[e] = sum;
+            }
+            __syncthreads();
         }
+        if (slice == 0)
+            for (int e = tid; e < m * r; e += kSmallThreads) {
+                const int col = e / r, c = e - col * r;
+                it.q[e] = QT[c * m + col];
+            }
     }
     for (int e = tid; e < n * r; e += kSmallThreads) {
         const int row = e / r;
-        it.p[e] = Ps[row * RS + (e - row * r)];
+        it.p[(size_t)row0 * r + e] = Ps[row * RS + (e - row * r)];
     }
 
     // the old cells the residual will be added onto are requested now and travel during step 6
@@ -360,7 +481,7 @@ psgd_small_round_body(const SmallItem& it, int mq_mode, int pqt_mode, float alph
     float aux[kCells];
 #pragma unroll
     for (int u = 0; u < kCells; ++u)
-        aux[u] = pairs > 0 ? it.cs[tid + u * kSmallThreads < pairs ? tid + u * kSmallThreads : pairs - 1] : 0.f;
+        aux[u] = pairs > 0 ? gcs[tid + u * kSmallThreads < pairs ? tid + u * kSmallThreads : pairs - 1] : 0.f;
 
     // ---- 6. M = P Q^T, residual kept in LDS (and, dense error feedback, written out)
     {
@@ -389,19 +510,25 @@ psgd_small_round_body(const SmallItem& it, int mq_mode, int pqt_mode, float alph
 #pragma unroll
             for (int k = 0; k < W; ++k) res[k] = __fsub_rn(xv[k], mh[k]);
             if (FAST) {
-                st4s(it.x + e, mh);
+                st4s(gx + e, mh);
                 st4s(X + e, res);
-                if (pqt_mode == 1) st4s(it.err + e, res);
+                if (pqt_mode == 1) st4s(gerr + e, res);
             } else {
-                it.x[e] = mh[0];
+                gx[e] = mh[0];
                 X[e] = res[0];
-                if (pqt_mode == 1) it.err[e] = res[0];
+                if (pqt_mode == 1) gerr[e] = res[0];
             }
             at.next(width);
         }
     }
-    if (pqt_mode != 2) return;
     __syncthreads();
+    if (*failed) {
+        // a peer never published: what this slice computed is not the round's result, and must not pass for it
+        if (tid == 0) gs_count_give_up();
+        for (int e = tid; e < total; e += kSmallThreads) gx[e] = __builtin_nanf("");
+        return;
+    }
+    if (pqt_mode != 2) return;
     // the residual into the sketch: one thread per (row, bucket), the bucket's columns ascending
     // (DenseCS.update, CountSketch.py:27-67: every term's decay reads the cell as it was before)
     {
@@ -417,7 +544,7 @@ psgd_small_round_body(const SmallItem& it, int mq_mode, int pqt_mode, float alph
                 const double sv = (double)__uint_as_float(__float_as_uint(xr[en & 0x7fffu]) ^ flip);
                 acc = __fadd_rn(acc, (float)__dsub_rn(sv, decay));
             }
-            it.cs[idx] = acc;
+            gcs[idx] = acc;
             at.next(w);
         };
 #pragma unroll
@@ -425,15 +552,18 @@ psgd_small_round_body(const SmallItem& it, int mq_mode, int pqt_mode, float alph
             const int idx = tid + u * kSmallThreads;
             if (idx < pairs) one(idx, aux[u]);
         }
-        for (int idx = tid + kCells * kSmallThreads; idx < pairs; idx += kSmallThreads) one(idx, it.cs[idx]);
+        for (int idx = tid + kCells * kSmallThreads; idx < pairs; idx += kSmallThreads) one(idx, gcs[idx]);
     }
 }
 
 template <int RP>
 __global__ void __launch_bounds__(kSmallThreads)
-psgd_small_round_kernel(SmallBatch batch, int mq_mode, int pqt_mode, float alpha, double one_minus_beta, float eps)
+psgd_small_round_kernel(SmallBatch batch, unsigned tag, int mq_mode, int pqt_mode, float alpha, double one_minus_beta, float eps)
 {
-    const SmallItem& it = batch.item[blockIdx.x];
-    if (it.fast) psgd_small_round_body<RP, true>(it, mq_mode, pqt_mode, alpha, one_minus_beta, eps);
-    else psgd_small_round_body<RP, false>(it, mq_mode, pqt_mode, alpha, one_minus_beta, eps);
+    int k = 0;
+    while (k + 1 < batch.count && (int)blockIdx.x >= batch.item[k + 1].first) ++k;
+    const SmallItem& it = batch.item[k];
+    const int slice = (int)blockIdx.x - it.first;
+    if (it.fast) psgd_small_round_body<RP, true>(it, slice, tag, mq_mode, pqt_mode, alpha, one_minus_beta, eps);
+    else psgd_small_round_body<RP, false>(it, slice, tag, mq_mode, pqt_mode, alpha, one_minus_beta, eps);
 }

@@ -352,15 +352,23 @@ int conef_psgd_round_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_m
  * the reference's steps in the reference's order - orthogonalise Q, X = M + error, P = X Q,
  * orthogonalise P, Q = X^T P, M = P Q^T, residual to the dense error or into the sketch (a bucket's
  * terms in ascending column order).  Replaces powerSGD_hook.py:473-564 at world size 1.
- * mq_mode / pqt_mode as above (0, 1, or both 2); no workspace.  conef_psgd_round_small_fits says
- * (1 / 0) whether a bucket qualifies: every matrix has at most 16384 elements (one workgroup does
- * all of a matrix's work: beyond that the separate launches, which spread a matrix over many
- * workgroups, are faster), ranks up to 8, a row-list plan per sketch in mode 2; the round returns
- * CONEF_ERR_INVALID for a bucket that does not. */
+ * A matrix of more than 10240 elements is dealt out by rows over up to 16 workgroups, which meet
+ * twice (the rows of the raw P, the shares of X^T P added in a fixed order) through 8-byte records
+ * {launch tag, value} in `workspace` (conef_psgd_round_small_workspace_bytes of it, 8-byte aligned;
+ * nothing to clear, contents are scratch): one workgroup does all the work for its rows on one CU,
+ * and beyond that size more CUs are worth two exchanges.  The waits are bounded; a workgroup whose
+ * peers never publish leaves NaN in its rows of M and counts in conef_gram_schmidt_give_ups.
+ * mq_mode / pqt_mode as above (0, 1, or both 2).  conef_psgd_round_small_fits says (1 / 0) whether
+ * a bucket qualifies: at most 24 matrices of at most 73728 elements each, 128 workgroups in all,
+ * every workgroup's rows fit LDS with the factors and the sketch's bucket lists, ranks up to 8, a
+ * row-list plan per sketch in mode 2; the round returns CONEF_ERR_INVALID for a bucket that does
+ * not.  conef_psgd_batch_workspace_bytes covers what this round needs. */
 int conef_psgd_round_small_fits(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, int32_t a,
                                 int32_t b);
+int64_t conef_psgd_round_small_workspace_bytes(const ConefPsgdItem* items, int32_t count);
 int conef_psgd_round_small_f32(const ConefPsgdItem* items, int32_t count, int32_t mq_mode, int32_t pqt_mode, float alpha,
-                               float beta, float eps, int32_t a, int32_t b, void* stream);
+                               float beta, float eps, int32_t a, int32_t b, void* workspace, int64_t workspace_bytes,
+                               void* stream);
 
 /* The middle of that round as a call of its own, for a caller that splits the round (the hooks above
  * rank 8 do, to orthogonalise the new Q on a side stream meanwhile): P = X Q with the Q factors of

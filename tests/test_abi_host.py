@@ -224,3 +224,51 @@ def test_threaded_oracle_step_is_the_single_threaded_one(oracle):
         np.testing.assert_array_equal(xa, xb)
         np.testing.assert_array_equal(pa, pb)
         np.testing.assert_array_equal(cs_a, cs_b)
+
+
+def test_one_launch_round_qualification_and_workspace(lib):
+    """Which buckets the one-launch PowerSGD round takes, and the records it asks workspace for: host
+    logic, nothing is launched (the pointers are never followed without a plan to check)."""
+    import ctypes
+    from conef_amd._lib import PsgdItem
+
+    def items_for(shapes, rank):
+        arr = (PsgdItem * len(shapes))()
+        for k, (n, m) in enumerate(shapes):
+            arr[k].x = arr[k].err = arr[k].p = arr[k].q = 256 * (k + 1)     # non-null, 16-byte aligned, never followed
+            arr[k].n, arr[k].m, arr[k].r = n, m, min(rank, n, m)
+        return arr
+
+    def slices(n, m):
+        s = 1 if n * m <= 10240 else min(-(-n * m // 4608), 16, n)
+        rows_per = -(-n // s)
+        return -(-n // rows_per)
+
+    def records(n, m, r):
+        s = slices(n, m)
+        return 0 if s == 1 else -(-(n * r + s * r * m) // 32) * 32
+
+    small = [(16, 27), (32, 288), (10, 64)]
+    arr = items_for(small, 2)
+    assert lib.conef_psgd_round_small_fits(arr, len(small), 0, 0, 994443, 609478) == 1
+    assert lib.conef_psgd_round_small_fits(arr, len(small), 1, 1, 994443, 609478) == 1
+    assert lib.conef_psgd_round_small_fits(arr, len(small), 2, 2, 994443, 609478) == 0     # no sketch, no plan
+    assert lib.conef_psgd_round_small_fits(arr, len(small), 2, 1, 994443, 609478) == 0     # modes 2 come together
+    assert lib.conef_psgd_round_small_workspace_bytes(arr, len(small)) == 0
+    sliced = [(64, 576), (64, 288), (37, 301), (16, 2304), (20, 2000)]
+    arr = items_for(sliced, 2)
+    assert lib.conef_psgd_round_small_fits(arr, len(sliced), 1, 1, 994443, 609478) == 1
+    assert lib.conef_psgd_round_small_workspace_bytes(arr, len(sliced)) == 8 * sum(records(n, m, 2) for n, m in sliced)
+    assert lib.conef_psgd_batch_workspace_bytes(arr, len(sliced)) >= lib.conef_psgd_round_small_workspace_bytes(arr, len(sliced))
+    # beyond sixteen slices' worth of elements, above rank 8, more than 24 matrices, more than 128 workgroups
+    assert lib.conef_psgd_round_small_fits(items_for([(128, 577)], 2), 1, 0, 0, 994443, 609478) == 0
+    assert lib.conef_psgd_round_small_fits(items_for([(64, 64)], 16), 1, 0, 0, 994443, 609478) == 0
+    assert lib.conef_psgd_round_small_fits(items_for([(8, 8)] * 25, 2), 25, 0, 0, 994443, 609478) == 0
+    assert lib.conef_psgd_round_small_fits(items_for([(64, 1024)] * 10, 2), 10, 0, 0, 994443, 609478) == 0
+    assert lib.conef_psgd_round_small_fits(items_for([(64, 1024)] * 8, 2), 8, 0, 0, 994443, 609478) == 1
+    # a slice that does not fit LDS with its factors: one row of 30000 columns
+    assert lib.conef_psgd_round_small_fits(items_for([(2, 30000)], 2), 1, 0, 0, 994443, 609478) == 0
+    # the round itself refuses what does not qualify, and a workspace that is too small, before any launch
+    arr = items_for(sliced, 2)
+    assert lib.conef_psgd_round_small_f32(arr, len(sliced), 1, 1, 0.0, 0.0, 0.0, 994443, 609478, None, 0, None) != 0
+    assert lib.conef_psgd_round_small_f32(items_for([(128, 577)], 2), 1, 0, 0, 0.0, 0.0, 0.0, 994443, 609478, None, 0, None) != 0
