@@ -130,7 +130,7 @@ class _RoundPlan:
     __slots__ = ("small", "sig", "errs_sig", "cs_static", "env_ahead", "env_topk_side", "env_small", "key", "shapes", "work", "passthrough", "before", "after", "total_ps", "total_qs", "arena_key", "ps",
                  "qs", "items", "count", "sketches", "fused_sketch", "batched_update", "residual_offsets",
                  "topk_table", "q_next", "q_next_ptrs", "q_next_ready", "made", "q_next_views", "items_next", "q_next_event",
-                 "topk_event", "ws_need", "handoff_event", "gs_table", "topk_number", "q_next_number")
+                 "topk_event", "ws_need", "handoff_event", "gs_table", "topk_number", "q_next_number", "is_wide", "wide")
 
 
 def _layout_signature(grads):
@@ -171,6 +171,9 @@ def _build_round(state, grads, shapes, key, error_mode):
         it = plan.items[cnt]
         it.x, it.n, it.m, it.r, it.w = matrix.data_ptr(), n, m, rank, 1
     plan.arena_key = None
+    # a rank above 32 goes through column chunks of the factors (conef_amd/_psgd_wide.py)
+    plan.is_wide = any(rank > 32 for _, _, _, rank in plan.work)
+    plan.wide = None
     plan.small = None               # (mode1, mode3) -> whether the bucket's round runs as one launch (a bucket of small matrices)
     plan.sketches = []
     plan.fused_sketch = False
@@ -347,6 +350,9 @@ def _run_round(state, bucket, error_mode, streams=1):
         plan.arena_key = (p_mem.data_ptr(), q_mem.data_ptr())
         plan.q_next = None
         plan.q_next_ready = False
+        if plan.is_wide and plan.wide is None:
+            from ._psgd_wide import WideRound
+            plan.wide = WideRound(work, plan.ps, plan.qs, device)
     if need_randomize_qs:
         plan.q_next_ready = False
     qs = plan.qs
@@ -398,7 +404,7 @@ def _run_round(state, bucket, error_mode, streams=1):
     wait_for_side_topk(plan, device, lambda: _lib.current_stream(device))
     eps = float(state.orthogonalization_epsilon)
     if plan.ws_need is None:
-        plan.ws_need = max(lib.conef_psgd_batch_workspace_bytes(items, count), 256)
+        plan.ws_need = plan.wide.ws_need if plan.is_wide else max(lib.conef_psgd_batch_workspace_bytes(items, count), 256)
     ws = _workspace(device, stream, plan.ws_need)
     ws_ptr, ws_len = ws.data_ptr(), ws.numel()
     if need_randomize_qs:
@@ -441,12 +447,28 @@ def _run_round(state, bucket, error_mode, streams=1):
         mode3 = 3 if error_mode == "conef" and plan.batched_update else 1
     else:
         mode3 = 0
-    if plan.small is None or plan.small[0] != (mode1, mode3):
+    if plan.is_wide:
+        # A rank above 32: the error is added in passes of its own, the round runs on column chunks of
+        # the factors, and the residual leaves the round dense (a sketch is updated from it below).
+        plan.small = ((mode1, mode3), False)
+        plan.q_next_ready = False
+        if mode3 == 3:
+            mode3 = 1
+        for cnt, (matrix, n, m, rank) in enumerate(work):
+            if mode1 == 1:
+                _lib.check(lib.conef_ef_passthrough_f32(matrix.data_ptr(), items[cnt].err, n * m, stream), "conef_ef_passthrough_f32")
+            elif mode1 == 2:
+                errs[cnt].query(matrix, alpha)
+        dest = [items[cnt].err if mode3 == 1 else None for cnt in range(count)]
+        plan.wide.run(lib, plan.ps, plan.qs, dest, eps, ws_ptr, ws_len, stream)
+    elif plan.small is None or plan.small[0] != (mode1, mode3):
         # a bucket of small matrices (every one fits a workgroup's LDS with its factors): the whole round in one launch
         fits = bool(count and mode3 in (0, 1, 2) and plan.env_small
                     and lib.conef_psgd_round_small_fits(items, count, mode1, mode3, HASH_A, HASH_B))
         plan.small = ((mode1, mode3), fits)
-    if plan.small[1]:
+    if plan.is_wide:
+        pass
+    elif plan.small[1]:
         plan.q_next_ready = False
         rc = lib.conef_psgd_round_small_f32(items, count, mode1, mode3, float(alpha), float(state.beta) if mode3 == 2 else 0.0,
                                             eps, HASH_A, HASH_B, ws_ptr, ws_len, stream)
@@ -611,8 +633,8 @@ def run_batched_round(state, bucket):
     state.total_numel_before_compression += total_length
     state.total_numel_after_compression += side * rank * 2
     padded = side * side
-    if rank > side or rank > 32:
-        raise ValueError("matrix_approximation_rank %d does not fit a %d x %d matrix (at most 32)" % (rank, side, side))
+    if rank > side:
+        raise ValueError("matrix_approximation_rank %d does not fit a %d x %d matrix" % (rank, side, side))
 
     # the bucket buffer cannot grow in place, so a padded bucket is worked on in a square buffer
     if padded == total_length:
@@ -644,6 +666,24 @@ def run_batched_round(state, bucket):
     p, q = state.p_memory_dict[bucket_index], state.q_memory_dict[bucket_index]
 
     eps = float(state.orthogonalization_epsilon)
+    if rank > 32:
+        # column chunks of the factors (conef_amd/_psgd_wide.py), built once per bucket and square buffer
+        from ._psgd_wide import WideRound
+        wide = state.round_cache.get(bucket_index)
+        if wide is None or wide[0] != (square.data_ptr(), side, rank):
+            wide = ((square.data_ptr(), side, rank), WideRound([(square.view(side, side), side, side, rank)], [p], [q], device))
+            state.round_cache[bucket_index] = wide
+        ws = _workspace(device, stream, wide[1].ws_need)
+        if err is not None:
+            _lib.check(lib.conef_ef_passthrough_f32(square.data_ptr(), err.data_ptr(), padded, stream), "conef_ef_passthrough_f32")
+        wide[1].run(lib, [p], [q], [err.data_ptr() if err is not None else None], eps, ws.data_ptr(), ws.numel(), stream)
+        if square is not input_tensor:
+            input_tensor.copy_(square[:total_length])
+        if not state.warm_start:
+            state.p_memory_dict.clear()
+            state.q_memory_dict.clear()
+        state.maybe_increase_iter(bucket)
+        return _bucket.completed_future(input_tensor)
     ws = _workspace(device, stream, lib.conef_psgd_workspace_bytes(side, side, rank))
     ws_ptr, ws_len = ws.data_ptr(), ws.numel()
     _lib.check(lib.conef_gram_schmidt_f32(q.data_ptr(), side, rank, eps, ws_ptr, ws_len, stream),

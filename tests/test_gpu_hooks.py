@@ -685,6 +685,27 @@ def test_small_bucket_with_an_all_zero_gradient_matrix(oracle, mode, eps):
             _nan_aware_close(st.error_dict[0], ost.error_dict[0], "dense error step %d" % step)
 
 
+WIDE_SHAPES = [(700, 512), (512,), (260, 1200), (40, 90), (1024, 300), (129, 257)]
+
+
+@pytest.mark.parametrize("rank", [33, 48, 64, 100])
+@pytest.mark.parametrize("mode", [None, "ef", "conef", "topk"])
+def test_ranks_above_32(oracle, mode, rank):
+    """The reference takes any matrix_approximation_rank (powerSGD_hook.py:146-160).  Above 32 the
+    factors go through the kernels in column chunks (a remainder chunk first, then chunks of 32);
+    in the same bucket sit a matrix whose smaller side caps its rank at 40 (two chunks where its
+    neighbours have up to four) and odd shapes.  Against the oracle over four steps, state carried."""
+    st, hook = _state_for(mode, rank, 0.2)
+    ost = oracle.PowerSGDOracle(matrix_approximation_rank=rank, error_mode=mode, sketch_size=0.2, beta=0.9, topk_ratio=0.4)
+    # (from the second step on the oracle restarts from the device's state, as in test_powersgd_hook_parity: a
+    # matrix whose rank is its smaller side makes ill-conditioned factors, and a top-k set that flips feeds back)
+    run_steps(hook, st, ost, WIDE_SHAPES, 4, check=psgd_check_factory(st, ost, mode),
+              resync=psgd_resync_factory(st, ost, mode, free_steps=2))
+    assert st.round_cache[0].is_wide
+    rate, before, after = st.compression_stats()
+    assert 0 < after < before
+
+
 @pytest.mark.parametrize("shapes,rank,ss", PSGD_CASES[:3])
 def test_c2cs_hook_v2_parity(oracle, shapes, rank, ss):
     """The sketch lives on the [m,n] re-view of every compressed matrix's memory."""
@@ -698,7 +719,7 @@ def test_c2cs_hook_v2_parity(oracle, shapes, rank, ss):
 
 
 @pytest.mark.parametrize("total,rank,ef", [(64 * 64, 1, True), (5000, 2, True), (268_346, 1, True), (1000, 4, False),
-                                           (7, 1, True)])
+                                           (7, 1, True), (250_000, 40, True), (90_000, 64, False), (300 * 300 + 17, 70, True)])
 def test_batched_powersgd_hook_parity(oracle, total, rank, ef):
     from conef_amd.powerSGD_hook import PowerSGDState, batched_powerSGD_hook
     st = PowerSGDState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2, use_error_feedback=ef)
