@@ -114,7 +114,7 @@ def UnbiasedMtrx_hook(state: unbiasedMtrxState, bucket) -> torch.futures.Future[
         state.p_memory_dict[bucket_index] = torch.empty(total_ps, device=device, dtype=dtype)
         state.q_memory_dict[bucket_index] = torch.empty(total_qs, device=device, dtype=dtype)
     p_mem, q_mem = state.p_memory_dict[bucket_index], state.q_memory_dict[bucket_index]
-    ws = _workspace(device, stream, max([lib.conef_psgd_workspace_bytes(n, m, rank) for _, n, m, rank in work] or [256]))
+    ws = _workspace(device, stream, max([lib.conef_psgd_workspace_bytes(n, m, min(rank, 32)) for _, n, m, rank in work] or [256]))
     p_idx = q_idx = 0
     for matrix, n, m, rank in work:
         p = p_mem[p_idx: p_idx + n * rank].view(n, rank)
@@ -122,6 +122,28 @@ def UnbiasedMtrx_hook(state: unbiasedMtrxState, bucket) -> torch.futures.Future[
         p_idx += n * rank
         q_idx += m * rank
         set_random(q, state, device)                                                      # :231
+        if rank > 32:
+            # The kernels take ranks up to 32: a wider factor goes through them in column chunks,
+            # P_c = M Q_c for every chunk first (M is read, not written), then M = sum of P_c Q_c^T,
+            # the first chunk's product written into M and the others added to it in chunk order.
+            from ._psgd_wide import chunk_widths
+            chunks, o = [], 0
+            for wd in chunk_widths(rank):
+                pc, qc = torch.empty(n, wd, device=device, dtype=dtype), q[:, o:o + wd].contiguous()
+                _lib.check(lib.conef_psgd_mq_f32(matrix.data_ptr(), qc.data_ptr(), pc.data_ptr(), n, m, wd, ws.data_ptr(),
+                                                 ws.numel(), stream), "conef_psgd_mq_f32")
+                p[:, o:o + wd].copy_(pc)
+                chunks.append((pc, qc, wd))
+                o += wd
+            part = torch.empty(n, m, device=device, dtype=dtype)
+            for c, (pc, qc, wd) in enumerate(chunks):
+                out = matrix if c == 0 else part
+                _lib.check(lib.conef_psgd_pqt_f32(out.data_ptr(), pc.data_ptr(), qc.data_ptr(), n, m, wd, stream),
+                           "conef_psgd_pqt_f32")
+                if c > 0:
+                    _lib.check(lib.conef_ef_passthrough_f32(matrix.data_ptr(), part.data_ptr(), n * m, stream),
+                               "conef_ef_passthrough_f32")
+            continue
         _lib.check(lib.conef_psgd_mq_f32(matrix.data_ptr(), q.data_ptr(), p.data_ptr(), n, m, rank, ws.data_ptr(),
                                          ws.numel(), stream),
                    "conef_psgd_mq_f32")                                                   # :232

@@ -1315,11 +1315,13 @@ def test_hook_step_with_an_all_zero_gradient_matrix(monkeypatch, oracle, rank, m
 
 # ------------------------------------------------------- unbiased random matrix --
 
-def test_unbiased_mtrx_hook_parity(oracle):
+@pytest.mark.parametrize("shapes,rank", [([(64, 576), (64,), (300, 40), (2, 1024)], 4),
+                                         ([(700, 512), (512,), (260, 1200), (40, 90)], 70)])
+def test_unbiased_mtrx_hook_parity(oracle, shapes, rank):
     """M <- (M Q) Q^T with Q drawn from the device generator under the seeds of RandomState(421)
-    (unbiasedMtrx_hook.py:41-45,231-232,292): the same draws, then the oracle's products."""
+    (unbiasedMtrx_hook.py:41-45,231-232,292): the same draws, then the oracle's products.  (Rank 70:
+    the factors go through the kernels in column chunks.)"""
     from conef_amd.unbiasedMtrx_hook import UnbiasedMtrx_hook, unbiasedMtrxState
-    shapes, rank = [(64, 576), (64,), (300, 40), (2, 1024)], 4
     total = numel_of(shapes)
     st = unbiasedMtrxState(None, matrix_approximation_rank=rank, start_powerSGD_iter=2)
     st.iter = 2
