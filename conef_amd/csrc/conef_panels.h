@@ -137,6 +137,20 @@ struct ConefPanelRegs {      // by name: arrays here end up in scratch memory
     uint4 eg;
 };
 
+// quad i of a panel of q_row quads a row -> (row, quad of the row).  Panels are a power of two wide
+// except a matrix's last one, so the division is a shift nearly always.
+__device__ __forceinline__ void conef_panel_quad_at(int i, int q_row, int* row, int* q)
+{
+    if ((q_row & (q_row - 1)) == 0) {
+        const int sh = 31 - __clz(q_row);
+        *row = i >> sh;
+        *q = i & (q_row - 1);
+    } else {
+        *row = i / q_row;
+        *q = i - *row * q_row;
+    }
+}
+
 template <typename Front>
 __device__ __forceinline__ void
 conef_panel_request(const Front& front, const ConefPanelView& plan, ConefPanelRegs& r, int64_t row0, int rows, int c0, int d)
@@ -153,14 +167,16 @@ conef_panel_request(const Front& front, const ConefPanelView& plan, ConefPanelRe
     const float* raw = front.raw();
     {
         const int i = i0 < total ? i0 : total - 1;
-        const int row = i / q_row, q = i - row * q_row;
+        int row, q;
+        conef_panel_quad_at(i, q_row, &row, &q);
         r.g0 = *reinterpret_cast<const float4*>(raw + (row0 + row) * d + c0 + 4 * q);
         r.ep0 = *reinterpret_cast<const uint2*>(plan.epos + c0 + 4 * q);
         r.cb0 = *reinterpret_cast<const uint2*>(plan.colb + c0 + 4 * q);
     }
     {
         const int i = i1 < total ? i1 : total - 1;
-        const int row = i / q_row, q = i - row * q_row;
+        int row, q;
+        conef_panel_quad_at(i, q_row, &row, &q);
         r.g1 = *reinterpret_cast<const float4*>(raw + (row0 + row) * d + c0 + 4 * q);
         r.ep1 = *reinterpret_cast<const uint2*>(plan.epos + c0 + 4 * q);
         r.cb1 = *reinterpret_cast<const uint2*>(plan.colb + c0 + 4 * q);
@@ -174,7 +190,8 @@ __device__ __forceinline__ void
 conef_panel_park_quad(const Front& front, float4 g, uint2 ep, uint2 cb, int i, int q_row, int64_t row0, int rows, int c0,
                       int d, int w, float* terms, const float* aux, double one_minus_beta)
 {
-    const int row = i / q_row, q = i - row * q_row;
+    int row, q;
+    conef_panel_quad_at(i, q_row, &row, &q);
     const int64_t f = (row0 + row) * d + c0 + 4 * q;
     const uint32_t e[4] = {ep.x & 0xffffu, ep.x >> 16, ep.y & 0xffffu, ep.y >> 16};
     const uint32_t j[4] = {cb.x & 0xffffu, cb.x >> 16, cb.y & 0xffffu, cb.y >> 16};
