@@ -117,3 +117,54 @@ def test_hook_under_ddp(process_group, oracle, name, streams):
                              what="%s step %d bucket %d param %s" % (name, step, index, shp))
                 off += cnt
             assert off == want.size
+
+
+@pytest.mark.parametrize("name,rank", [("conef_powersgd", 4), ("hefsgd_powersgd", 4), ("conef_powersgd", 32)])
+def test_streams_chosen_by_bucket_size_under_ddp(process_group, name, rank):
+    """With ``hook_streams`` left alone, buckets of 2**20 elements or more alternate between the hook's
+    stream and a side stream (rank <= 8) or are dealt over three streams (above): under the real reducer
+    the parameters' gradients must come out bit for bit as with everything on one stream."""
+    from torch.nn.parallel import DistributedDataParallel as DDP
+
+    from conef_amd import _psgd_engine
+    from conef_amd.get_comm_hooks import make_state
+
+    def big_model():
+        torch.manual_seed(11)
+        return nn.Sequential(nn.Linear(1100, 1024), nn.ReLU(), nn.Linear(1024, 1200), nn.ReLU(), nn.Linear(1200, 1024),
+                             nn.ReLU(), nn.Linear(1024, 10))
+
+    results = []
+    for streams in (None, 1):
+        ddp = DDP(big_model().cuda(), device_ids=[0], bucket_cap_mb=4.5)
+        args = dict(ARGS, matrix_approximation_rank=rank)
+        state, hook = make_state(Namespace(grad_reducer=name, **args))
+        if streams is not None:
+            state.hook_streams = streams
+        else:
+            assert state.hook_streams == (3 if rank > 8 else 0)
+        seen = []
+
+        def watching(st, bucket, hook=hook, seen=seen):
+            seen.append(_psgd_engine.streams_for(st, bucket.buffer()))
+            return hook(st, bucket)
+
+        ddp.register_comm_hook(state, watching)
+        loss_fn = nn.CrossEntropyLoss()
+        grads_per_step = []
+        for step in range(7):
+            gen = torch.Generator().manual_seed(300 + step)
+            x = torch.randn(16, 1100, generator=gen).cuda()
+            y = torch.randint(0, 10, (16,), generator=gen).cuda()
+            ddp.zero_grad(set_to_none=True)
+            loss_fn(ddp(x), y).backward()
+            torch.cuda.synchronize()
+            grads_per_step.append([p.grad.detach().cpu().numpy().copy() for p in ddp.parameters()])
+        if streams is None:
+            assert max(seen) == (3 if rank > 8 else 2), "the large buckets were expected to be dealt over streams"
+        results.append(grads_per_step)
+        del ddp
+    for step, (a, b) in enumerate(zip(*results)):
+        for ga, gb in zip(a, b):
+            np.testing.assert_array_equal(ga, gb, err_msg="step %d" % step)
+    assert _psgd_engine.gram_schmidt_give_ups() == 0
