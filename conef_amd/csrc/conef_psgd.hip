@@ -3702,7 +3702,6 @@ int conef_psgd_round_small_f32(const ConefPsgdItem* items, int32_t count, int32_
             t.r = it.r;
             t.fast = it.m % 4 == 0 && aligned16(it.x) && ((mq_mode != 1 && pqt_mode != 1) || aligned16(it.err));
             t.slices = small_slices(it.n, it.m, &t.rows_per);
-            t.first = wgs;
             wgs += t.slices;
             t.recs = t.slices > 1 ? recs : nullptr;
             recs += (small_record_count(it.n, it.m, it.r, t.slices) + 31) / 32 * 32;
@@ -3713,11 +3712,42 @@ int conef_psgd_round_small_f32(const ConefPsgdItem* items, int32_t count, int32_
             if (need > lds) lds = need;
         }
         if (lds > kSmallLdsLimit || wgs > kSmallMaxWgs) return CONEF_ERR_INVALID;
+        // which workgroup does what: slices on the workgroups of XCDs 0..3 (b % 8 < 4), whole matrices on
+        // those of XCDs 4..7 first; with nothing sliced, in plain order
+        std::vector<unsigned short> sliced, whole;
+        for (int k = 0; k < nb; ++k) {
+            if (batch.item[k].slices > 1)
+                for (int sl = 0; sl < batch.item[k].slices; ++sl) sliced.push_back((unsigned short)(k | (sl << 8)));
+            else
+                whole.push_back((unsigned short)k);
+        }
+        for (int b2 = 0; b2 < kSmallMaxGrid; ++b2) batch.where[b2] = kSmallIdle;
+        int grid = wgs;
+        if (sliced.empty()) {
+            for (int b2 = 0; b2 < wgs; ++b2) batch.where[b2] = whole[(size_t)b2];
+        } else {
+            int groups = (wgs + 7) / 8;
+            if ((int)sliced.size() > 4 * groups) groups = ((int)sliced.size() + 3) / 4;
+            auto early = [](int e) { return (e / 4) * 8 + e % 4; };
+            auto late = [](int l) { return (l / 4) * 8 + 4 + l % 4; };
+            int e = 0, l = 0;
+            grid = 0;
+            for (unsigned short w2 : sliced) {
+                const int b2 = early(e++);
+                batch.where[b2] = w2;
+                if (b2 + 1 > grid) grid = b2 + 1;
+            }
+            for (unsigned short w2 : whole) {
+                const int b2 = l < 4 * groups ? late(l++) : early(e++);
+                batch.where[b2] = w2;
+                if (b2 + 1 > grid) grid = b2 + 1;
+            }
+        }
 #define CONEF_SMALL(RP)                                                                                         \
     do {                                                                                                        \
         auto kern = psgd_small_round_kernel<RP>;                                                                \
         if (hipError_t e = conef_allow_lds((const void*)kern, lds); e != hipSuccess) return (int)e;             \
-        hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(kSmallThreads), lds, s, batch, tag, mq_mode, pqt_mode, alpha, omb, eps); \
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kSmallThreads), lds, s, batch, tag, mq_mode, pqt_mode, alpha, omb, eps); \
     } while (0)
         switch (rp) {
             case 1: CONEF_SMALL(1); break;

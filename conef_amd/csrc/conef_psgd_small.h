@@ -64,12 +64,21 @@ struct SmallItem {
     int fast;               // m % 4 == 0 and x (and err, where used) 16-byte aligned: the element-wise phases go by column quads
     int slices;             // workgroups the rows are dealt over
     int rows_per;           // rows a slice (the last one may hold fewer)
-    int first;              // the matrix's first workgroup in the launch
     unsigned long long* recs;   // slices > 1: n*r records of the raw P, then slices * r*m records of the shares of X^T P
 };
 
+// Workgroup b of the grid runs on XCD b % 8 (the hardware deals workgroups out round robin), and
+// on this part the workgroups of XCDs 4..7 start about 2 us after those of XCDs 0..3 (measured
+// with timestamps: 0-3.2 us against 2.3-6.2 us for a grid of 58).  The slices of a matrix wait for
+// each other twice, so a late slice holds up its whole matrix: the launch's table puts the slices
+// on the early XCDs' workgroups and the matrices that go whole (and are done long before the
+// sliced ones) on the late ones; slots that are left over end at once.
+constexpr int kSmallMaxGrid = 2 * kSmallMaxWgs;
+constexpr unsigned short kSmallIdle = 0xffffu;
+
 struct SmallBatch {
     SmallItem item[kSmallMaxItems];
+    unsigned short where[kSmallMaxGrid];     // item | slice << 8 of every workgroup of the grid, or kSmallIdle
     int count;
 };
 
@@ -237,6 +246,26 @@ psgd_small_round_body(const SmallItem& it, int slice, unsigned tag, int mq_mode,
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     if (tid == 0) *failed = 0;
 
+    // The first quads of the matrix (and of the dense error) are asked for before anything else:
+    // they depend on nothing, and travel while Q and the tables arrive.
+    constexpr int QH = 5;
+    float4 gq_first[QH];
+    float ev_first[QH][4];
+    if (FAST) {
+        const int groups = total >> 2, width = m >> 2;
+        SmallWalk pre(tid, width);
+#pragma unroll
+        for (int u = 0; u < QH; ++u) {
+            // (a slot past the end asks for nothing: a request is a request, whatever its address)
+            if (tid + u * kSmallThreads < groups) {
+                const int e = (pre.row * width + pre.col) * 4;
+                gq_first[u] = *reinterpret_cast<const float4*>(gx + e);
+                if (mq_mode == 1) ld4s(gerr + e, ev_first[u]);
+            }
+            pre.next(width);
+        }
+    }
+
     // ---- 1. Q into LDS (padding columns zero); the sketch's tables ride along
     {
         constexpr int U = 4;
@@ -244,7 +273,10 @@ psgd_small_round_body(const SmallItem& it, int slice, unsigned tag, int mq_mode,
         for (int e0 = tid; e0 < count; e0 += U * kSmallThreads) {
             float t[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) t[u] = it.q[e0 + u * kSmallThreads < count ? e0 + u * kSmallThreads : count - 1];
+            for (int u = 0; u < U; ++u) {
+                t[u] = 0.f;
+                if (e0 + u * kSmallThreads < count) t[u] = it.q[e0 + u * kSmallThreads];
+            }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int e = e0 + u * kSmallThreads;
@@ -272,9 +304,9 @@ psgd_small_round_body(const SmallItem& it, int slice, unsigned tag, int mq_mode,
     // (and of the dense error, or every gather of a sketch cell) is requested before the first is
     // used, and Q is orthogonalised while they travel: the matrix is one trip to memory.
     if (FAST) {
-        // a matrix has at most 40960 elements, ten quads a thread: five are requested, Q is orthogonalised
+        // a matrix has at most 40960 elements, ten quads a thread: five are requested (the matrix's own
+        // values at the kernel's start, the sketch cells now that the table is there), Q is orthogonalised
         // while they travel, then the other five (all ten at once would not fit the registers)
-        constexpr int QH = 5;
         const int groups = total >> 2, width = m >> 2;
         SmallWalk issue(tid, width), finish(tid, width);
 #pragma unroll
@@ -284,11 +316,19 @@ psgd_small_round_body(const SmallItem& it, int slice, unsigned tag, int mq_mode,
 #pragma unroll
             for (int u = 0; u < QH; ++u) {
                 const bool in = tid + (half * QH + u) * kSmallThreads < groups;
-                const int row = in ? issue.row : 0, col = in ? issue.col : 0;
+                const int row = issue.row, col = issue.col;
                 const int e = (row * width + col) * 4;
-                gq[u] = *reinterpret_cast<const float4*>(gx + e);
-                if (mq_mode == 1) ld4s(gerr + e, ev[u]);
-                if (mq_mode == 2) {
+                if (half == 0) {
+                    gq[u] = gq_first[u];
+                    if (mq_mode == 1) {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) ev[u][k] = ev_first[u][k];
+                    }
+                } else if (in) {
+                    gq[u] = *reinterpret_cast<const float4*>(gx + e);
+                    if (mq_mode == 1) ld4s(gerr + e, ev[u]);
+                }
+                if (mq_mode == 2 && in) {
                     const uint4 pw = *reinterpret_cast<const uint4*>(pk_l + col * 4);
                     const float* cells = gcs + row * w;
                     ev[u][0] = cells[pw.x & 0x7fffffffu];
@@ -331,14 +371,15 @@ psgd_small_round_body(const SmallItem& it, int slice, unsigned tag, int mq_mode,
 #pragma unroll
             for (int u = 0; u < kAhead; ++u) {
                 const bool in = g0 + u * kSmallThreads < total;
-                const int row = in ? at.row : 0, col = in ? at.col : 0;
+                const int row = at.row, col = at.col;
                 where[u] = in ? row * m + col : -1;
-                const int e = in ? where[u] : 0;
-                gv[u] = gx[e];
-                if (mq_mode == 1) ev[u] = gerr[e];
-                if (mq_mode == 2) {
-                    pw[u] = pk_l[col];
-                    ev[u] = gcs[row * w + (int)(pw[u] & 0x7fffffffu)];
+                if (in) {
+                    gv[u] = gx[where[u]];
+                    if (mq_mode == 1) ev[u] = gerr[where[u]];
+                    if (mq_mode == 2) {
+                        pw[u] = pk_l[col];
+                        ev[u] = gcs[row * w + (int)(pw[u] & 0x7fffffffu)];
+                    }
                 }
                 at.next(m);
             }
@@ -440,27 +481,37 @@ psgd_small_round_body(const SmallItem& it, int slice, unsigned tag, int mq_mode,
             unsigned long long* shares = it.recs + (size_t)rows * r;
             const int count = r * m;
             for (int e = tid; e < count; e += kSmallThreads) small_publish(shares + (size_t)slice * count + e, QT[e], tag);
-            for (int e = tid; e < count; e += kSmallThreads) {
-                float sum = 0.f;
-                for (int g0 = 0; g0 < slices; g0 += 4) {           // four shares requested at a time
-                    unsigned long long first[4];
+            // (a thread takes two entries at a time and four slices' shares of each: eight requests in flight)
+            for (int e0 = tid; e0 < count; e0 += 2 * kSmallThreads) {
+                const int e1 = e0 + kSmallThreads;
+                const bool two = e1 < count;
+                float sum0 = 0.f, sum1 = 0.f;
+                for (int g0 = 0; g0 < slices; g0 += 4) {
+                    unsigned long long f0[4], f1[4];
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
                         const int g = g0 + u;
-                        first[u] = g < slices && g != slice
-                                       ? __hip_atomic_load(shares + (size_t)g * count + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                                       : 0ull;
+                        const bool ask = g < slices && g != slice;
+                        const unsigned long long* at = shares + (size_t)(ask ? g : slice) * count;
+                        f0[u] = ask ? __hip_atomic_load(at + e0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+                        f1[u] = ask && two ? __hip_atomic_load(at + e1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
                     }
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
                         const int g = g0 + u;
                         if (g < slices) {
-                            const float v = g == slice ? QT[e] : small_await(shares + (size_t)g * count + e, first[u], tag, failed);
-                            sum = g == 0 ? v : __fadd_rn(sum, v);
+                            const unsigned long long* at = shares + (size_t)g * count;
+                            const float v0 = g == slice ? QT[e0] : small_await(at + e0, f0[u], tag, failed);
+                            sum0 = g == 0 ? v0 : __fadd_rn(sum0, v0);
+                            if (two) {
+                                const float v1 = g == slice ? QT[e1] : small_await(at + e1, f1[u], tag, failed);
+                                sum1 = g == 0 ? v1 : __fadd_rn(sum1, v1);
+                            }
                         }
                     }
                 }
-                QT[e] = sum;
+                QT[e0] = sum0;
+                if (two) QT[e1] = sum1;
             }
             __syncthreads();
         }
@@ -480,8 +531,10 @@ psgd_small_round_body(const SmallItem& it, int slice, unsigned tag, int mq_mode,
     const int pairs = pqt_mode == 2 ? n * w : 0;
     float aux[kCells];
 #pragma unroll
-    for (int u = 0; u < kCells; ++u)
-        aux[u] = pairs > 0 ? gcs[tid + u * kSmallThreads < pairs ? tid + u * kSmallThreads : pairs - 1] : 0.f;
+    for (int u = 0; u < kCells; ++u) {
+        aux[u] = 0.f;
+        if (tid + u * kSmallThreads < pairs) aux[u] = gcs[tid + u * kSmallThreads];
+    }
 
     // ---- 6. M = P Q^T, residual kept in LDS (and, dense error feedback, written out)
     {
@@ -560,10 +613,10 @@ template <int RP>
 __global__ void __launch_bounds__(kSmallThreads)
 psgd_small_round_kernel(SmallBatch batch, unsigned tag, int mq_mode, int pqt_mode, float alpha, double one_minus_beta, float eps)
 {
-    int k = 0;
-    while (k + 1 < batch.count && (int)blockIdx.x >= batch.item[k + 1].first) ++k;
-    const SmallItem& it = batch.item[k];
-    const int slice = (int)blockIdx.x - it.first;
+    const unsigned where = batch.where[blockIdx.x];
+    if (where == kSmallIdle) return;
+    const SmallItem& it = batch.item[where & 0xffu];
+    const int slice = (int)(where >> 8);
     if (it.fast) psgd_small_round_body<RP, true>(it, slice, tag, mq_mode, pqt_mode, alpha, one_minus_beta, eps);
     else psgd_small_round_body<RP, false>(it, slice, tag, mq_mode, pqt_mode, alpha, one_minus_beta, eps);
 }
