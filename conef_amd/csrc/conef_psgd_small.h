@@ -44,7 +44,7 @@ constexpr size_t kSmallLdsLimit = 160 * 1024;     // all of a CU's LDS: one work
 // Matrices above kSmallWholeElements go over slices of about kSmallSliceElements ([64,576] over
 // eight workgroups: 15 us against 33 us on one), at most kSmallMaxSlices of them; a launch holds at
 // most kSmallMaxWgs workgroups, far fewer than the machine has CUs, so the slices of a matrix (which
-// are neighbours in the grid) are resident together.
+// the launch's table keeps side by side) are resident together.
 constexpr int64_t kSmallWholeElements = 10240;
 constexpr int64_t kSmallSliceElements = 4608;
 constexpr int kSmallMaxSlices = 16;
